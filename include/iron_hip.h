@@ -1,0 +1,134 @@
+/* libiron_hip.so -- C ABI of the hand-written gfx950 (MI355X) kernels behind the
+ * IRON operator hot path.
+ *
+ * Every entry point: plain pointers and sizes, all data pointers are DEVICE
+ * pointers owned by the caller, bf16 is 16-bit storage (uint16_t), one HIP
+ * stream is passed in (void* = hipStream_t, NULL = the default stream).  No
+ * entry point allocates, frees or synchronizes, so each may be recorded into a
+ * HIP graph.  Return value: 0 = launched, 1 = arguments refused (the text is
+ * in iron_last_error()), any other value = the hipError_t the launch raised.
+ *
+ * "const int* valid"-style arguments are per-call bounds read on the device at
+ * run time (the reference's per-call scratchpad words,
+ * iron/common/image/packaging.py:20); NULL means the whole extent.
+ *
+ * Citations are into the reference tree (amd/IRON).
+ */
+#ifndef IRON_HIP_H
+#define IRON_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Library version (major*10000 + minor*100 + patch). */
+int iron_version(void);
+/* Text of the last refusal on this thread ("" if none). */
+const char* iron_last_error(void);
+
+/* C = A @ B, f32 accumulation, one rounding to bf16.
+ * A (M,K) row-major.  B (K,N) row-major, or (N,K) row-major if b_col_maj.
+ * C (M,N) row-major, or (N,M) if c_col_maj.  K % 8 == 0.
+ * valid: rows of A computed (others of C untouched); valid_k: K actually summed.
+ * Replaces GEMM.build()/kernels.linalg.mm: iron/operators/gemm.py:143,397-410,696-702. */
+int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K,
+                   int b_col_maj, int c_col_maj, const int* valid, const int* valid_k,
+                   void* stream);
+
+/* y[b] = W[b / repeat] @ x[b] for b in [0, batches): W (batches/repeat, M, K), x (batches, K),
+ * y (batches, M); f32 accumulation, one rounding.  K % 8 == 0.
+ * valid: rows of W computed.
+ * Replaces GEMV.build()/linalg.mv: iron/operators/gemv.py:79,267-275,408-417. */
+int iron_gemv_bf16(const uint16_t* W, const uint16_t* x, uint16_t* y, int M, int K, int batches,
+                   int repeat, const int* valid, void* stream);
+/* The same with the launch shape forced (rows a wave takes, waves splitting K); 0 = heuristic. */
+int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16_t* y, int M, int K,
+                         int batches, int repeat, const int* valid, int rows_per_wave,
+                         int k_split, void* stream);
+
+/* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; w NULL = unweighted (one rounding).
+ * x,y (rows, cols); w (cols).  cols % 8 == 0.  valid: rows computed.
+ * Replaces norm.rms_norm_eps + eltwise.mul_sized: iron/operators/rms_norm.py:10,
+ * iron/common/elementwise.py:619-682. */
+int iron_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int rows, int cols,
+                      float eps, const int* valid, void* stream);
+
+/* Rotary embedding of x (rows, cols) by the packed table angles (angle_rows, cols), cos and
+ * sin interleaved; row r uses angle row r / (rows / angle_rows).  two_halves: rotate the two
+ * halves of a row (else interleaved pairs).  cols % 16 == 0.  valid: rows computed.
+ * Replaces datamovement.rope: iron/operators/rope.py:58,161-184. */
+int iron_rope_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows, int cols,
+                   int angle_rows, int two_halves, const int* valid, void* stream);
+
+/* Elementwise over n elements (valid: elements computed), f32 math, one rounding each:
+ *   silu: y = x*sigmoid(x)   mul: y = a*b   add: y = a+b
+ *   silu_mul: y = bf16(bf16(silu(g)) * u)  -- SiLU then ElementwiseMul, rounded between,
+ * as two reference steps are.
+ * Replaces activation.silu / eltwise.mul_sized / eltwise.add_sized:
+ * iron/operators/silu.py:12, elementwise_mul.py:11, elementwise_add.py:11,
+ * iron/common/elementwise.py:255-285. */
+int iron_silu_bf16(const uint16_t* x, uint16_t* y, int64_t n, const int* valid, void* stream);
+int iron_mul_bf16(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, const int* valid,
+                  void* stream);
+int iron_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, const int* valid,
+                  void* stream);
+int iron_silu_mul_bf16(const uint16_t* g, const uint16_t* u, uint16_t* y, int64_t n,
+                       const int* valid, void* stream);
+
+/* Attention, many queries (prefill / prompt chunk).  Q,O: (seq, heads, d) if q_interleaved
+ * else (heads, seq, d); K,V: (kv_len, kv_heads, d) if kv_interleaved else (kv_heads, kv_len, d).
+ * The queries are the last rows of the keys: query i sits at position kv_tokens - q_tokens + i,
+ * q_tokens = *valid (or seq_len), kv_tokens = *kv_valid (or kv_len - seq + q_tokens).
+ * causal masks key > position; window >= 0 also masks key < position - window (and, when not
+ * causal, key > position + window); window < 0 = none.  Rows >= q_tokens of O are zeros.
+ * d in {64, 128}; heads % kv_heads == 0.
+ * Replaces kernels.linalg.mha + partial_softmax + matmul_PV:
+ * iron/operators/mha.py:191,574-667,1073-1116. */
+int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
+                          int heads, int kv_heads, int d, int seq, int seq_len, int kv_len,
+                          float scale, int causal, int window, int q_interleaved,
+                          int kv_interleaved, const int* valid, const int* kv_valid, void* stream);
+
+/* Attention, one query (decode; the reference's "packed" MHA, seq_len == 1).
+ * Q,O: (heads, d).  K,V as above.  kv_tokens = *kv_valid (or kv_len); the query sits at
+ * kv_tokens - 1.  workspace: iron_mha_decode_workspace_bytes(heads, d) bytes of device memory.
+ * Replaces the packed single-query MHA: iron/operators/mha.py:476-477,1073-1116. */
+int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
+                         int heads, int kv_heads, int d, int kv_len, float scale, int window,
+                         int kv_interleaved, const int* kv_valid, void* workspace, void* stream);
+int64_t iron_mha_decode_workspace_bytes(int heads, int d);
+
+/* out[i] = table[ids[i]] for i < *valid (or n_ids); rows of row_bytes bytes (multiple of 4).
+ * ids outside [0, table_rows) are skipped (the row is left untouched).
+ * Replaces Copy's gather (embedding lookup): iron/operators/copy.py:72,546,839-902. */
+int iron_gather_rows(const void* table, const int* ids, void* out, int n_ids, int table_rows,
+                     int64_t row_bytes, const int* valid, void* stream);
+
+/* dst[(*dst_row + i)] = src[(*src_row + i)] for i < *valid (or rows); NULL row index = 0.
+ * Rows are row_bytes bytes (multiple of 4) at src_stride/dst_stride bytes apart; rows that
+ * would land outside [0, src_rows) / [0, dst_rows) are skipped.
+ * Replaces Copy between views with per-call offsets (KV-cache write, RoPE-table row,
+ * last-row pick): iron/operators/copy.py:546,839-902. */
+int iron_copy_rows(const void* src, void* dst, int rows, int64_t row_bytes, int64_t src_stride,
+                   int64_t dst_stride, int src_rows, int dst_rows, const int* src_row,
+                   const int* dst_row, const int* valid, void* stream);
+
+/* Greedy draw: *token = index of the first largest logit among logits[0..n); when record is
+ * not NULL also record[*at] = token (at NULL = 0; skipped if outside [0, record_len)).
+ * Replaces Sample with an all-zero draw row: iron/operators/sample.py:72-79,106,324-333. */
+int iron_argmax_bf16(const uint16_t* logits, int n, int* token, int* record, int record_len,
+                     const int* at, void* stream);
+
+/* Evaluate n per-call word expressions in order, on the device, in one thread:
+ *   words[e.dst] = clamp(((words[e.src] * e.mul + e.add) >> e.shift), e.lo, e.hi)
+ * exprs is n records of 7 int32 {dst, src, mul, add, shift, lo, hi} in device memory.
+ * The device-side carry/Emit of a decode loop (position += 1, kv_valid = position + 1):
+ * iron/common/graph/carried.py:189-276, iron/operators/emit.py. */
+int iron_eval_words(int* words, int n_words, const int* exprs, int n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IRON_HIP_H */

@@ -1,0 +1,104 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define IRON_OK 0
+#define IRON_EINVAL 1
+
+namespace iron {
+
+constexpr int kWave = 64;
+
+// Set by an entry point that refuses its arguments; read back by iron_last_error().
+void set_error(const char* fmt, ...);
+
+#define IRON_REQUIRE(cond, ...)        \
+  do {                                 \
+    if (!(cond)) {                     \
+      ::iron::set_error(__VA_ARGS__);  \
+      return IRON_EINVAL;              \
+    }                                  \
+  } while (0)
+
+#define IRON_LAUNCH_CHECK()                          \
+  do {                                               \
+    hipError_t e__ = hipPeekAtLastError();           \
+    if (e__ != hipSuccess) {                         \
+      ::iron::set_error("%s", hipGetErrorString(e__)); \
+      return (int)e__;                               \
+    }                                                \
+    return IRON_OK;                                  \
+  } while (0)
+
+typedef uint16_t bf16_t;  // storage
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) {
+  return __builtin_bit_cast(float, w & 0xffff0000u);
+}
+
+// float -> bf16, round to nearest even (NaN stays quiet NaN).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+// Round a float to the nearest bf16 and return it as float.
+__device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+  f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x);
+  f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+  f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z);
+  f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+  uint4 v;
+  v.x = pack_bf16(f[0], f[1]); v.y = pack_bf16(f[2], f[3]);
+  v.z = pack_bf16(f[4], f[5]); v.w = pack_bf16(f[6], f[7]);
+  return v;
+}
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// 16-byte streaming load that does not displace reusable lines in the caches.
+__device__ __forceinline__ uint4 load_stream(const uint4* p) {
+  u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_stream(uint4* p, const uint4& v) {
+  u32x4 w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(p));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// A per-call bound read from device memory; a null pointer reads as `whole`.
+__device__ __forceinline__ int bound_or(const int* p, int whole) {
+  if (p == nullptr) return whole;
+  int v = *p;
+  return v < 0 ? 0 : (v > whole ? whole : v);
+}
+
+}  // namespace iron

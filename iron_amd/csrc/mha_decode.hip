@@ -1,0 +1,239 @@
+// Attention for one query token over a KV cache (decode): pure KV streaming,
+// HBM-bandwidth bound.
+//
+// grid = (splits, kv_heads).  A block of 4 waves takes one contiguous slice of the
+// keys of one KV head and serves all G query heads of its group from that single
+// stream.  D/8 lanes cover one key row with 16-byte loads (a wave covers 512/D rows
+// per step); scores are reduced across those lanes, the softmax is kept online in
+// f32 in the exp2 domain per lane group, and lane groups, waves and finally splits
+// are merged by the usual (max, sum, acc) rule.  A second small kernel merges the
+// splits and writes bf16.
+#include "../../include/iron_hip.h"
+#include "common.h"
+
+namespace iron {
+
+constexpr int kMaxSplits = 128;
+
+template <int D, int G>
+__global__ __launch_bounds__(256) void mha_decode_kernel(
+    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
+    float* __restrict__ part, int kv_len, float scale_log2, int window, long row_stride,
+    long head_stride, const int* __restrict__ kv_valid) {
+  constexpr int LPR = D / 8;     // lanes per key row
+  constexpr int RW = 64 / LPR;   // rows a wave covers per step
+  constexpr int U = 4;           // steps in flight
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPR, rg = lane / LPR;
+  const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y;
+
+  const int kv_tokens = bound_or(kv_valid, kv_len);
+  const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
+  const int n = kv_tokens - first;
+  // Slice of this block, in whole wave-steps so that waves split it evenly.
+  int chunk = (n + nsplit - 1) / nsplit;
+  chunk = (chunk + 4 * RW - 1) / (4 * RW) * (4 * RW);
+  const int blo = first + split * chunk;
+  const int wlo = blo + wave * (chunk / 4);
+  const int whi = min(min(wlo + chunk / 4, blo + chunk), kv_tokens);
+
+  float qf[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float t[8];
+    unpack8(*reinterpret_cast<const uint4*>(Q + (size_t)(kvh * G + g) * D + sub * 8), t);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[g][i] = t[i] * scale_log2;
+  }
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+  }
+
+  const bf16_t* Kh = K + (size_t)kvh * head_stride + sub * 8;
+  const bf16_t* Vh = V + (size_t)kvh * head_stride + sub * 8;
+
+  for (int base = wlo; base < whi; base += U * RW) {
+    uint4 kv[U], vv[U];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int r = base + u * RW + rg;
+      live[u] = r < whi;
+      const size_t off = (size_t)(live[u] ? r : (whi - 1)) * row_stride;
+      kv[u] = load_stream(reinterpret_cast<const uint4*>(Kh + off));
+      vv[u] = load_stream(reinterpret_cast<const uint4*>(Vh + off));
+    }
+    float s[U][G];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float kf[8];
+      unpack8(kv[u], kf);
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
+#pragma unroll
+        for (int o = 1; o < LPR; o <<= 1) d += __shfl_xor(d, o, 64);
+        s[u][g] = live[u] ? d : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float mx = m[g];
+#pragma unroll
+      for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[u][g]);
+      // A lane group whose rows are all past the end keeps -inf; exp2(-inf - 0) = 0.
+      const float ref = (mx == -INFINITY) ? 0.f : mx;
+      const float alpha = exp2f(m[g] - ref);
+      float p[U];
+      float ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        p[u] = exp2f(s[u][g] - ref);
+        ps += p[u];
+      }
+      l[g] = l[g] * alpha + ps;
+      m[g] = mx;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float vf[8];
+        unpack8(vv[u], vf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p[u], vf[i], acc[g][i]);
+      }
+    }
+  }
+
+  // Merge the RW lane groups of the wave (lanes that share `sub`).
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int o = LPR; o < 64; o <<= 1) {
+      const float mo = __shfl_xor(m[g], o, 64);
+      const float lo = __shfl_xor(l[g], o, 64);
+      const float mx = fmaxf(m[g], mo);
+      const float ref = (mx == -INFINITY) ? 0.f : mx;
+      const float a = exp2f(m[g] - ref), b = exp2f(mo - ref);
+      l[g] = l[g] * a + lo * b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float ao = __shfl_xor(acc[g][i], o, 64);
+        acc[g][i] = acc[g][i] * a + ao * b;
+      }
+      m[g] = mx;
+    }
+  }
+
+  // Merge the 4 waves through LDS; wave 0 writes the block's partial.
+  __shared__ float sm[4][G];
+  __shared__ float sl[4][G];
+  __shared__ float sacc[4][G][D];
+  if (rg == 0) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      if (sub == 0) {
+        sm[wave][g] = m[g];
+        sl[wave][g] = l[g];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sacc[wave][g][sub * 8 + i] = acc[g][i];
+    }
+  }
+  __syncthreads();
+  // part layout: [head][split][D + 2] = {m, l, acc[D]}.
+  for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+    const int g = idx / D, dd = idx % D;
+    float mx = fmaxf(fmaxf(sm[0][g], sm[1][g]), fmaxf(sm[2][g], sm[3][g]));
+    const float ref = (mx == -INFINITY) ? 0.f : mx;
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float e = exp2f(sm[w][g] - ref);
+      lt += sl[w][g] * e;
+      at += sacc[w][g][dd] * e;
+    }
+    float* out = part + ((size_t)(kvh * G + g) * nsplit + split) * (D + 2);
+    out[2 + dd] = at;
+    if (dd == 0) {
+      out[0] = mx;
+      out[1] = lt;
+    }
+  }
+}
+
+template <int D>
+__global__ void mha_decode_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ O,
+                                        int nsplit) {
+  const int head = blockIdx.x, dd = threadIdx.x;
+  const float* p = part + (size_t)head * nsplit * (D + 2);
+  float mx = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, p[s * (D + 2)]);
+  const float ref = (mx == -INFINITY) ? 0.f : mx;
+  float lt = 0.f, at = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float e = exp2f(p[s * (D + 2)] - ref);
+    lt += p[s * (D + 2) + 1] * e;
+    at += p[s * (D + 2) + 2 + dd] * e;
+  }
+  O[(size_t)head * D + dd] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
+}
+
+template <int D, int G>
+static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, float* part,
+                          int kv_heads, int kv_len, float scale_log2, int window, long row_stride,
+                          long head_stride, const int* kv_valid, int nsplit, hipStream_t s) {
+  hipLaunchKernelGGL((mha_decode_kernel<D, G>), dim3(nsplit, kv_heads), dim3(256), 0, s, Q, K, V,
+                     part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid);
+  hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D), 0, s, part, O,
+                     nsplit);
+}
+
+}  // namespace iron
+
+using namespace iron;
+
+extern "C" int64_t iron_mha_decode_workspace_bytes(int heads, int d) {
+  return (int64_t)heads * kMaxSplits * (d + 2) * sizeof(float);
+}
+
+extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                    uint16_t* O, int heads, int kv_heads, int d, int kv_len,
+                                    float scale, int window, int kv_interleaved,
+                                    const int* kv_valid, void* workspace, void* stream) {
+  IRON_REQUIRE(Q && K && V && O && workspace, "mha_decode: null operand");
+  IRON_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
+               "mha_decode: heads (%d) must be a positive multiple of kv_heads (%d)", heads, kv_heads);
+  IRON_REQUIRE(kv_len > 0, "mha_decode: kv_len (%d) must be positive", kv_len);
+  IRON_REQUIRE(scale >= 0.f && scale < INFINITY, "mha_decode: scale must be finite and not negative");
+  IRON_REQUIRE((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)workspace) & 15) == 0,
+               "mha_decode: operands must be 16-byte aligned");
+  const int G = heads / kv_heads;
+  const long row_stride = kv_interleaved ? (long)kv_heads * d : d;
+  const long head_stride = kv_interleaved ? d : (long)kv_len * d;
+  int nsplit = (kv_len + 63) / 64;
+  nsplit = nsplit < 1 ? 1 : (nsplit > kMaxSplits ? kMaxSplits : nsplit);
+  const float scale_log2 = scale * 1.4426950408889634f;
+  hipStream_t s = (hipStream_t)stream;
+  float* part = (float*)workspace;
+#define IRON_DEC(DD, GG)                                                                        \
+  if (d == DD && G == GG) {                                                                     \
+    launch_decode<DD, GG>(Q, K, V, O, part, kv_heads, kv_len, scale_log2, window, row_stride,   \
+                          head_stride, kv_valid, nsplit, s);                                    \
+    IRON_LAUNCH_CHECK();                                                                        \
+  }
+#define IRON_DEC_D(DD) \
+  IRON_DEC(DD, 1) IRON_DEC(DD, 2) IRON_DEC(DD, 3) IRON_DEC(DD, 4) IRON_DEC(DD, 5) IRON_DEC(DD, 6) IRON_DEC(DD, 8)
+  IRON_DEC_D(64) IRON_DEC_D(128) IRON_DEC_D(256)
+#undef IRON_DEC_D
+#undef IRON_DEC
+  IRON_REQUIRE(false, "mha_decode: no kernel for d=%d with %d query heads per KV head "
+               "(d in {64,128,256}, group in {1,2,3,4,5,6,8})", d, G);
+}

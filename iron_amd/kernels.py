@@ -1,0 +1,232 @@
+"""Thin, typed Python calls onto the C ABI: torch CUDA tensors in, launches out.
+
+Each function checks what the C side cannot see (dtype, device, contiguity,
+element counts), passes raw device pointers and the current HIP stream, and
+raises ``IronHipError`` on refusal.  Nothing here computes.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ._lib import check, current_stream, lib, ptr
+
+BF16 = torch.bfloat16
+
+
+def _dev(t, name, dtype=BF16):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise TypeError(f"{name}: expected a tensor on the GPU, got {t.device}")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: expected a contiguous tensor")
+    return t
+
+
+def _word(t, name):
+    """An optional per-call word: a 1-element int32 device tensor, or None."""
+    if t is None:
+        return None
+    _dev(t, name, torch.int32)
+    if t.numel() < 1:
+        raise ValueError(f"{name}: expected at least one int32 word")
+    return t
+
+
+def _numel(t, n, name):
+    if t.numel() != n:
+        raise ValueError(f"{name}: expected {n} elements, got {t.numel()} {tuple(t.shape)}")
+
+
+def gemm(A, B, C, *, M, N, K, b_col_maj=False, c_col_maj=False, valid=None, valid_k=None):
+    _numel(_dev(A, "A"), M * K, "A")
+    _numel(_dev(B, "B"), K * N, "B")
+    _numel(_dev(C, "C"), M * N, "C")
+    check(
+        lib().iron_gemm_bf16(
+            ptr(A), ptr(B), ptr(C), M, N, K, int(b_col_maj), int(c_col_maj),
+            ptr(_word(valid, "valid")), ptr(_word(valid_k, "valid_k")), current_stream(),
+        ),
+        "iron_gemm_bf16",
+    )
+
+
+def gemv(W, x, y, *, M, K, batches=1, repeat=1, valid=None, rows_per_wave=0, k_split=0):
+    _numel(_dev(W, "A"), (batches // repeat) * M * K, "A")
+    _numel(_dev(x, "B"), batches * K, "B")
+    _numel(_dev(y, "C"), batches * M, "C")
+    check(
+        lib().iron_gemv_bf16_tuned(
+            ptr(W), ptr(x), ptr(y), M, K, batches, repeat, ptr(_word(valid, "valid")),
+            rows_per_wave, k_split, current_stream(),
+        ),
+        "iron_gemv_bf16",
+    )
+
+
+def rmsnorm(x, w, y, *, rows, cols, eps, valid=None):
+    _numel(_dev(x, "x"), rows * cols, "x")
+    _numel(_dev(y, "y"), rows * cols, "y")
+    if w is not None:
+        _numel(_dev(w, "weight"), cols, "weight")
+    check(
+        lib().iron_rmsnorm_bf16(
+            ptr(x), ptr(w), ptr(y), rows, cols, float(eps), ptr(_word(valid, "valid")),
+            current_stream(),
+        ),
+        "iron_rmsnorm_bf16",
+    )
+
+
+def rope(x, angles, y, *, rows, cols, angle_rows, two_halves=True, valid=None):
+    _numel(_dev(x, "x"), rows * cols, "x")
+    _numel(_dev(angles, "angles"), angle_rows * cols, "angles")
+    _numel(_dev(y, "y"), rows * cols, "y")
+    check(
+        lib().iron_rope_bf16(
+            ptr(x), ptr(angles), ptr(y), rows, cols, angle_rows, int(two_halves),
+            ptr(_word(valid, "valid")), current_stream(),
+        ),
+        "iron_rope_bf16",
+    )
+
+
+def _binary(name):
+    def call(a, b, y, *, n=None, valid=None):
+        n = y.numel() if n is None else n
+        _numel(_dev(a, "a"), n, "a")
+        _numel(_dev(b, "b"), n, "b")
+        _numel(_dev(y, "y"), n, "y")
+        check(
+            getattr(lib(), name)(ptr(a), ptr(b), ptr(y), n, ptr(_word(valid, "valid")), current_stream()),
+            name,
+        )
+
+    call.__name__ = name
+    return call
+
+
+mul = _binary("iron_mul_bf16")
+add = _binary("iron_add_bf16")
+silu_mul = _binary("iron_silu_mul_bf16")
+
+
+def silu(x, y, *, n=None, valid=None):
+    n = y.numel() if n is None else n
+    _numel(_dev(x, "x"), n, "x")
+    _numel(_dev(y, "y"), n, "y")
+    check(lib().iron_silu_bf16(ptr(x), ptr(y), n, ptr(_word(valid, "valid")), current_stream()), "iron_silu_bf16")
+
+
+def mha_prefill(
+    Q, K, V, O, *, heads, kv_heads, d, seq, seq_len=None, kv_len, scale=None, causal=True,
+    window=None, q_interleaved=False, kv_interleaved=False, valid=None, kv_valid=None,
+):
+    seq_len = seq if seq_len is None else seq_len
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    _numel(_dev(Q, "Q"), seq * heads * d, "Q")
+    _numel(_dev(O, "O"), seq * heads * d, "O")
+    _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
+    _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
+    check(
+        lib().iron_mha_prefill_bf16(
+            ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, seq, seq_len, kv_len, float(scale),
+            int(causal), -1 if window is None else int(window), int(q_interleaved),
+            int(kv_interleaved), ptr(_word(valid, "valid")), ptr(_word(kv_valid, "kv_valid")),
+            current_stream(),
+        ),
+        "iron_mha_prefill_bf16",
+    )
+
+
+def mha_decode_workspace(heads, d, device="cuda"):
+    n = lib().iron_mha_decode_workspace_bytes(heads, d)
+    return torch.empty(n // 4, dtype=torch.float32, device=device)
+
+
+def mha_decode(
+    Q, K, V, O, *, heads, kv_heads, d, kv_len, scale=None, window=None, kv_interleaved=False,
+    kv_valid=None, workspace,
+):
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    _numel(_dev(Q, "Q"), heads * d, "Q")
+    _numel(_dev(O, "O"), heads * d, "O")
+    _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
+    _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
+    _dev(workspace, "workspace", torch.float32)
+    need = lib().iron_mha_decode_workspace_bytes(heads, d)
+    if workspace.numel() * 4 < need:
+        raise ValueError(f"workspace: {workspace.numel() * 4} bytes, need {need}")
+    check(
+        lib().iron_mha_decode_bf16(
+            ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, kv_len, float(scale),
+            -1 if window is None else int(window), int(kv_interleaved),
+            ptr(_word(kv_valid, "kv_valid")), ptr(workspace), current_stream(),
+        ),
+        "iron_mha_decode_bf16",
+    )
+
+
+def gather_rows(table, ids, out, *, valid=None):
+    _dev(table, "table", None)
+    _dev(ids, "ids", torch.int32)
+    _dev(out, "out", table.dtype)
+    row_bytes = table[0].numel() * table.element_size()
+    n_ids = ids.numel()
+    _numel(out, n_ids * table[0].numel(), "out")
+    check(
+        lib().iron_gather_rows(
+            ptr(table), ptr(ids), ptr(out), n_ids, table.shape[0], row_bytes,
+            ptr(_word(valid, "valid")), current_stream(),
+        ),
+        "iron_gather_rows",
+    )
+
+
+def copy_rows(src, dst, *, rows, row_elems, src_rows, dst_rows, src_stride=None, dst_stride=None,
+              src_row=None, dst_row=None, valid=None):
+    """``dst[dst_row + i] = src[src_row + i]`` for ``i < rows``; strides in elements."""
+    _dev(src, "src", None)
+    _dev(dst, "dst", src.dtype)
+    es = src.element_size()
+    src_stride = row_elems if src_stride is None else src_stride
+    dst_stride = row_elems if dst_stride is None else dst_stride
+    if src.numel() < (src_rows - 1) * src_stride + row_elems:
+        raise ValueError(f"src: {src.numel()} elements do not hold {src_rows} rows")
+    if dst.numel() < (dst_rows - 1) * dst_stride + row_elems:
+        raise ValueError(f"dst: {dst.numel()} elements do not hold {dst_rows} rows")
+    check(
+        lib().iron_copy_rows(
+            ptr(src), ptr(dst), rows, row_elems * es, src_stride * es, dst_stride * es, src_rows,
+            dst_rows, ptr(_word(src_row, "src_row")), ptr(_word(dst_row, "dst_row")),
+            ptr(_word(valid, "valid")), current_stream(),
+        ),
+        "iron_copy_rows",
+    )
+
+
+def argmax(logits, token, *, n=None, record=None, at=None):
+    n = logits.numel() if n is None else n
+    _dev(logits, "logits")
+    _dev(token, "token", torch.int32)
+    if record is not None:
+        _dev(record, "record", torch.int32)
+    check(
+        lib().iron_argmax_bf16(
+            ptr(logits), n, ptr(token), ptr(record), 0 if record is None else record.numel(),
+            ptr(_word(at, "at")), current_stream(),
+        ),
+        "iron_argmax_bf16",
+    )
+
+
+def eval_words(words, exprs, n=None):
+    _dev(words, "words", torch.int32)
+    _dev(exprs, "exprs", torch.int32)
+    n = exprs.numel() // 7 if n is None else n
+    check(lib().iron_eval_words(ptr(words), words.numel(), ptr(exprs), n, current_stream()), "iron_eval_words")

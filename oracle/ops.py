@@ -1,0 +1,262 @@
+"""CPU restatement of the reference operators' ``reference()`` methods.
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke``
+and by ``bench.py``'s cpu_baseline leg as the checker; the product package
+never imports it.
+
+Conventions: a bf16 operand is a float32 numpy array whose values are exactly
+representable in bf16 (``iron_amd.bf16``); every function computes in float32
+as the reference does and rounds once to bf16 where the reference casts
+``astype(bfloat16)``.
+
+Pinned by (see tests/test_oracle.py):
+  gemm        f64 matmul + one rounding; tolerance formula      gemm.py:696-735
+  gemv        f64 matvec + one rounding                          gemv.py:408-421
+  rope        closed form row by row, array_equal                test_rope_reference_convention.py:27-64
+  mha         brute force per query on tiny inputs, chunk-vs-whole,
+              padding rows zero                                  mha.py:1073-1116, test_mha_bounded_rows.py
+  add         bit-exact bf16(f32(a)+f32(b))                      test_elementwise.py:125-132
+  copy/gather exact                                              copy.py:839-902
+  argmax      np.argmax of f32 logits (first of ties)            sample.py:72-79
+  rope_angles closed forms                                       test_rope_angles.py:20-107
+Parity unpinned (arithmetic lives in mlir-aie 1.4.6.dev15, absent here; textbook
+formula used, bounded by the stated bf16 tolerance and the model-level goldens):
+  rms_norm inner summation order / rsqrt, silu (LUT kernel), mul.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from iron_amd.bf16 import round_bf16
+
+
+def _f32(x):
+    return np.asarray(x, dtype=np.float32)
+
+
+# ---------------------------------------------------------------- GEMM / GEMV
+
+
+def gemm(A, B, *, b_col_maj=False, c_col_maj=False, valid_k=None):
+    """``A @ B`` in float32 over the first ``valid_k`` of K, rounded once (gemm.py:696-702)."""
+    a = _f32(A)
+    K = a.shape[1]
+    valid_k = K if valid_k is None else int(valid_k)
+    a = a[:, :valid_k]
+    b = (_f32(B).T if b_col_maj else _f32(B))[:valid_k]
+    C = np.matmul(b.T, a.T) if c_col_maj else np.matmul(a, b)
+    return round_bf16(C)
+
+
+def gemm_bound(A, B, *, b_col_maj=False, c_col_maj=False, units=2.0):
+    """The admitted |error| of GEMM at HIGHEST: ``units`` · 2^-8 · |A|@|B| (gemm.py:704-735)."""
+    a = _f32(A)
+    b = _f32(B).T if b_col_maj else _f32(B)
+    err = units * (np.abs(a) @ np.abs(b)) * 2.0**-8
+    return err.T if c_col_maj else err
+
+
+def gemv(A, B, *, repeat=1):
+    """``C = A @ B``, one product per batch, float32, rounded once (gemv.py:408-417)."""
+    A, B = _f32(A), _f32(B)
+    if repeat > 1:
+        A = np.repeat(A.reshape(-1, *A.shape[-2:]), repeat, axis=0)
+    if A.ndim == 3:
+        b = B.reshape(A.shape[0], A.shape[2], 1)
+        return round_bf16(np.matmul(A, b).reshape(A.shape[0], A.shape[1]))
+    return round_bf16(A @ B.reshape(A.shape[-1]))
+
+
+# ------------------------------------------------------------ rowwise / eltwise
+
+
+def rms_norm(x, weight=None, *, epsilon=1e-5):
+    """Each row over its RMS, rounded to bf16; then times ``weight``, rounded again.
+
+    Structure from elementwise.py:676-682 (the norm's row is rounded before the
+    multiply); the row formula ``x * 1/sqrt(mean(x^2) + eps)`` is the textbook one
+    (flm/layer/reference.py:108-119 hints the same) -- parity unpinned.
+    """
+    x = _f32(x)
+    ms = np.mean(x * x, axis=-1, keepdims=True, dtype=np.float32)
+    inv = (np.float32(1.0) / np.sqrt(ms + np.float32(epsilon))).astype(np.float32)
+    normed = round_bf16(x * inv)
+    if weight is None:
+        return normed
+    return round_bf16(normed * _f32(weight).reshape(-1))
+
+
+def silu(x):
+    """``x * sigmoid(x)`` in float32, rounded once (silu.py:12; LUT kernel -- parity unpinned)."""
+    x = _f32(x)
+    return round_bf16(x / (np.float32(1.0) + np.exp(-x)))
+
+
+def mul(a, b):
+    """``bf16(f32(a) * f32(b))`` (elementwise_mul.py:11)."""
+    return round_bf16(_f32(a) * _f32(b))
+
+
+def add(a, b):
+    """``bf16(f32(a) + f32(b))`` (elementwise_add.py:11; test_elementwise.py:125-132)."""
+    return round_bf16(_f32(a) + _f32(b))
+
+
+def rope(x, angles, *, two_halves=True):
+    """Rotate each row of ``x`` by its angle row; row r uses angle row ``r // (rows/angle_rows)``.
+
+    ``angles`` is the packed bf16 table, cos and sin interleaved (rope.py:167-184).
+    two_halves=False (interleaved pairs) is the textbook pair rotation -- parity unpinned.
+    """
+    x, angles = _f32(x), _f32(angles)
+    rows, cols, lut_rows = x.shape[0], x.shape[-1], angles.shape[0]
+    if rows % lut_rows:
+        raise ValueError(f"RoPE: angles ({lut_rows} rows) must divide x's {rows} rows")
+    xr = x.reshape(lut_rows, -1, cols)
+    cos = angles[:, None, 0::2]
+    sin = angles[:, None, 1::2]
+    y = np.empty_like(xr)
+    if two_halves:
+        h = cols // 2
+        x1, x2 = xr[..., :h], xr[..., h:]
+        y[..., :h] = x1 * cos - x2 * sin
+        y[..., h:] = x2 * cos + x1 * sin
+    else:
+        x1, x2 = xr[..., 0::2], xr[..., 1::2]
+        y[..., 0::2] = x1 * cos - x2 * sin
+        y[..., 1::2] = x2 * cos + x1 * sin
+    return round_bf16(y.reshape(x.shape))
+
+
+# ------------------------------------------------------------------- attention
+
+
+def mha(
+    Q,
+    K,
+    V,
+    *,
+    num_heads,
+    num_KV_heads=None,
+    seq_len=None,
+    kv_len=None,
+    d=64,
+    causal=True,
+    window=None,
+    scale=None,
+    heads_interleaved=False,
+    kv_interleaved=False,
+    valid=None,
+    kv_valid=None,
+):
+    """Attention per head, the queries the keys' last rows (mha.py:1073-1116).
+
+    ``valid`` / ``kv_valid`` are a bounded call's rows and keys; query rows past
+    the bound come out zero and keys past it are dropped.
+    """
+    Q, K, V = _f32(Q), _f32(K), _f32(V)
+    num_KV_heads = num_heads if num_KV_heads is None else num_KV_heads
+    if heads_interleaved:
+        Q = np.swapaxes(Q, 0, 1)
+    if kv_interleaved:
+        K, V = np.swapaxes(K, 0, 1), np.swapaxes(V, 0, 1)
+    seq_pad = Q.shape[1]
+    seq_len = seq_pad if seq_len is None else seq_len
+    kv_len = K.shape[1] if kv_len is None else kv_len
+    scale = float(1 / np.sqrt(d)) if scale is None else scale
+    q_tokens = seq_len if valid is None else int(valid)
+    kv_tokens = (kv_len - seq_pad + q_tokens) if kv_valid is None else int(kv_valid)
+    groups = num_heads // num_KV_heads
+    offset = kv_tokens - q_tokens
+    if (causal or window) and offset < 0:
+        raise ValueError(f"MHA: the {q_tokens} queries are more than the {kv_tokens} keys")
+    start = offset if causal or window else 0
+    s_q = start + q_tokens
+    K, V = K[:, :kv_tokens], V[:, :kv_tokens]
+    rows = max(s_q - start, 0)
+    q = Q[:, :rows]
+    key = np.arange(K.shape[1])
+    scale = np.float32(scale)
+    out = np.zeros(Q.shape, dtype=np.float32)
+    step = max(1, 2**24 // max(K.shape[1], 1))
+    for first in range(0, rows, step):
+        block = slice(first, min(first + step, rows))
+        position = offset + np.arange(block.start, block.stop)[:, None]
+        masked = np.zeros((len(position), K.shape[1]), dtype=bool)
+        if causal or window:
+            masked |= key > position + (0 if causal else (window or 0))
+        if window:
+            masked |= key < position - window
+        mask = np.where(masked, -np.inf, 0).astype(np.float32)
+        for h in range(q.shape[0]):
+            scores = q[h, block] @ K[h // groups].T * scale + mask
+            e = np.exp(scores - scores.max(axis=-1, keepdims=True))
+            out[h, block] = round_bf16((e / e.sum(axis=-1, keepdims=True)) @ V[h // groups])
+    if heads_interleaved:
+        return np.ascontiguousarray(np.swapaxes(out, 0, 1))
+    return out
+
+
+# --------------------------------------------------------------------- glue
+
+
+def gather_rows(table, ids):
+    """Rows of ``table`` named by ``ids`` (copy.py:839-902: exact)."""
+    return np.asarray(table)[np.asarray(ids, dtype=np.int64)]
+
+
+def argmax(logits) -> int:
+    """Greedy draw: the first largest float32 logit (sample.py:72-79, test_lm_host.py:554-557)."""
+    return int(np.argmax(_f32(logits).reshape(-1)))
+
+
+# --------------------------------------------------------------- RoPE tables
+
+
+def rope_angles(head_dim, context_length, rope_theta=500000.0, scaling=None):
+    """The RoPE table ``(context_length, head_dim)`` float32, cos/sin interleaved (lm/config.py:23-42)."""
+    exponents = np.arange(0, head_dim, 2, dtype=np.float32) / np.float32(head_dim)
+    inv_freq = 1.0 / np.power(rope_theta, exponents.astype(np.float64))
+    if scaling is not None:
+        inv_freq = scaling(inv_freq)
+    inv_freq = inv_freq.astype(np.float32)
+    freqs = np.outer(np.arange(context_length, dtype=np.float32), inv_freq)
+    angles = np.empty((context_length, head_dim), dtype=np.float32)
+    angles[:, ::2] = np.cos(freqs.astype(np.float64))
+    angles[:, 1::2] = np.sin(freqs.astype(np.float64))
+    return angles
+
+
+def llama3_scaling(factor, low_freq_factor, high_freq_factor, original_max_position_embeddings):
+    """Llama 3's RoPE frequency scaling (applications/llama/model.py:22-69)."""
+
+    def scale(inv_freq):
+        original = original_max_position_embeddings
+        wavelen = 2 * np.pi / inv_freq
+        smooth = (original / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
+        between = (1 - smooth) * inv_freq / factor + smooth * inv_freq
+        return np.where(
+            wavelen < original / high_freq_factor,
+            inv_freq,
+            np.where(wavelen > original / low_freq_factor, inv_freq / factor, between),
+        )
+
+    return scale
+
+
+# ------------------------------------------------------------- random weights
+
+
+def filled(named, seed=0):
+    """Weights from their shapes alone: ``filled("random", ...)`` (common/graph/fill.py:13-33), bf16."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for n, shape in named.items():
+        x = rng.standard_normal(shape, dtype=np.float32)
+        if len(shape) >= 2:
+            # numpy >= 2: float32 array / np.float64 scalar divides in float64.
+            out[n] = round_bf16((x / np.sqrt(float(np.prod(shape[1:])))).astype(np.float32))
+        else:
+            out[n] = round_bf16(x / 10 + (not n.endswith("bias")))
+    return out

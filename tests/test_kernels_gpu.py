@@ -1,0 +1,388 @@
+"""Parity of every HIP kernel, called through the C ABI, with the CPU oracle.
+
+Same seeded inputs on both sides; bf16 outputs within rtol 1e-2 / atol 1e-2 of the
+oracle's (f32 accumulation, one rounding), exact for the data movers and the draw.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from iron_amd import kernels as K
+from iron_amd.bf16 import from_torch, round_bf16, to_torch
+from oracle import ops
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-2
+
+
+def bf(rng, *shape, scale=1.0):
+    return round_bf16(rng.standard_normal(shape, dtype=np.float32) * np.float32(scale))
+
+
+def dev(x, cuda):
+    return to_torch(x).to(cuda)
+
+
+def out_like(shape, cuda, fill=None):
+    t = torch.empty(shape, dtype=torch.bfloat16, device=cuda)
+    if fill is not None:
+        t.fill_(fill)
+    return t
+
+
+def word(v, cuda):
+    return torch.tensor([v], dtype=torch.int32, device=cuda)
+
+
+def close(got, want, rtol=RTOL, atol=ATOL, frac=0.0):
+    got = from_torch(got).reshape(np.shape(want)) if isinstance(got, torch.Tensor) else got
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bad = ~(err <= atol + rtol * np.abs(want))
+    assert bad.mean() <= frac, (
+        f"{bad.sum()}/{bad.size} outside rtol {rtol} atol {atol}; max err {np.nanmax(err):.5f} "
+        f"at {np.unravel_index(np.nanargmax(err), err.shape)}"
+    )
+
+
+# ------------------------------------------------------------------------ GEMV
+@pytest.mark.parametrize("Kdim,N", [(2048, 2048), (2048, 512), (2048, 8192), (8192, 2048), (2048, 128256)])
+def test_gemv_decode_sweep(cuda, Kdim, N):
+    rng = np.random.default_rng(42)
+    W, x = bf(rng, N, Kdim, scale=0.02), bf(rng, Kdim)
+    y = out_like((N,), cuda)
+    K.gemv(dev(W, cuda), dev(x, cuda), y, M=N, K=Kdim)
+    close(y, ops.gemv(W, x))
+
+
+@pytest.mark.parametrize("rpw,ks", [(1, 1), (1, 2), (1, 4), (2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4), (8, 1)])
+def test_gemv_every_launch_shape_and_ragged_rows(cuda, rpw, ks):
+    rng = np.random.default_rng(1)
+    M, Kdim = 77, 1096  # rows not a multiple of any block, K not a multiple of 512
+    W, x = bf(rng, M, Kdim), bf(rng, Kdim)
+    y = out_like((M,), cuda)
+    K.gemv(dev(W, cuda), dev(x, cuda), y, M=M, K=Kdim, rows_per_wave=rpw, k_split=ks)
+    close(y, ops.gemv(W, x), rtol=1e-2, atol=3e-2)
+
+
+def test_gemv_batches_repeat_and_bound(cuda):
+    rng = np.random.default_rng(2)
+    # Llama decode's scores shape: 32 heads over 8 groups (gemv.py:51).
+    W, x = bf(rng, 8, 256, 64), bf(rng, 32, 64)
+    y = out_like((32, 256), cuda)
+    K.gemv(dev(W, cuda), dev(x, cuda), y, M=256, K=64, batches=32, repeat=4)
+    close(y, ops.gemv(W, x, repeat=4))
+    # A bound on the rows: rows past it are left as they were.
+    W, x = bf(rng, 300, 128), bf(rng, 128)
+    y = out_like((300,), cuda, fill=7.0)
+    K.gemv(dev(W, cuda), dev(x, cuda), y, M=300, K=128, valid=word(123, cuda))
+    got = from_torch(y)
+    close(got[:123], ops.gemv(W, x)[:123])
+    assert np.all(got[123:] == 7.0)
+
+
+# ------------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize("b_col_maj", [False, True])
+@pytest.mark.parametrize("c_col_maj", [False, True])
+def test_gemm_layouts(cuda, b_col_maj, c_col_maj):
+    rng = np.random.default_rng(3)
+    M, Kdim, N = 384, 512, 640
+    A, B = bf(rng, M, Kdim), bf(rng, (N if b_col_maj else Kdim), (Kdim if b_col_maj else N), scale=0.05)
+    C = out_like((N, M) if c_col_maj else (M, N), cuda)
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=M, N=N, K=Kdim, b_col_maj=b_col_maj, c_col_maj=c_col_maj)
+    want = ops.gemm(A, B, b_col_maj=b_col_maj, c_col_maj=c_col_maj)
+    close(C, want)
+    # And by the reference's own bound: 2 units of 2^-8 |A|@|B| (gemm.py:704-735).
+    bound = ops.gemm_bound(A, B, b_col_maj=b_col_maj, c_col_maj=c_col_maj)
+    assert np.all(np.abs(from_torch(C) - want) <= bound)
+
+
+def test_gemm_headline_shape(cuda):
+    rng = np.random.default_rng(4)
+    A, B = bf(rng, 2048, 2048, scale=0.02), bf(rng, 2048, 2048, scale=0.02)
+    C = out_like((2048, 2048), cuda)
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=2048, N=2048, K=2048)
+    close(C, ops.gemm(A, B), rtol=1e-2, atol=1e-3)
+    Bt = np.ascontiguousarray(B.T)
+    K.gemm(dev(A, cuda), dev(Bt, cuda), C, M=2048, N=2048, K=2048, b_col_maj=True)
+    close(C, ops.gemm(A, B), rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("M,Kdim,N", [(100, 136, 72), (32, 1152, 2048), (1, 64, 8), (130, 8, 264), (2048, 2048, 512), (192, 8192, 128)])
+@pytest.mark.parametrize("b_col_maj", [False, True])
+def test_gemm_ragged_shapes(cuda, M, Kdim, N, b_col_maj):
+    rng = np.random.default_rng(5)
+    A, B = bf(rng, M, Kdim), bf(rng, (N if b_col_maj else Kdim), (Kdim if b_col_maj else N), scale=0.1)
+    C = out_like((M, N), cuda)
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=M, N=N, K=Kdim, b_col_maj=b_col_maj)
+    close(C, ops.gemm(A, B, b_col_maj=b_col_maj), rtol=1e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("b_col_maj", [False, True])
+def test_gemm_bounded_rows_and_k_do_not_read_the_poison(cuda, b_col_maj):
+    """NaN past the bounds must not reach the output (test_gemm_bounded_k.py)."""
+    rng = np.random.default_rng(6)
+    M, Kdim, N, rows, kv = 256, 512, 128, 150, 332
+    A, B = bf(rng, M, Kdim), bf(rng, Kdim, N, scale=0.1)
+    want = ops.gemm(A, B, valid_k=kv)
+    A[:, kv:], B[kv:], A[rows:] = np.nan, np.nan, np.nan
+    Bs = np.ascontiguousarray(B.T) if b_col_maj else B
+    C = out_like((M, N), cuda, fill=5.0)
+    K.gemm(dev(A, cuda), dev(Bs, cuda), C, M=M, N=N, K=Kdim, b_col_maj=b_col_maj,
+           valid=word(rows, cuda), valid_k=word(kv, cuda))
+    got = from_torch(C)
+    close(got[:rows], want[:rows], rtol=1e-2, atol=2e-2)
+    assert np.all(got[rows:] == 5.0)
+
+
+# --------------------------------------------------------------------- rowwise
+@pytest.mark.parametrize("rows,cols", [(1, 2048), (2048, 2048), (7, 64), (3, 8192), (2, 16640)])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_rmsnorm(cuda, rows, cols, weighted):
+    rng = np.random.default_rng(7)
+    x = bf(rng, rows, cols)
+    w = round_bf16(rng.uniform(0.9, 1.1, cols)) if weighted else None
+    y = out_like((rows, cols), cuda)
+    K.rmsnorm(dev(x, cuda), None if w is None else dev(w, cuda), y, rows=rows, cols=cols, eps=1e-5)
+    close(y, ops.rms_norm(x, w, epsilon=1e-5))
+
+
+def test_rmsnorm_bound(cuda):
+    rng = np.random.default_rng(8)
+    x = bf(rng, 16, 256)
+    y = out_like((16, 256), cuda, fill=3.0)
+    K.rmsnorm(dev(x, cuda), None, y, rows=16, cols=256, eps=1e-5, valid=word(5, cuda))
+    got = from_torch(y)
+    close(got[:5], ops.rms_norm(x[:5]))
+    assert np.all(got[5:] == 3.0)
+
+
+def angle_table(rng, angle_rows, cols):
+    theta = rng.uniform(-np.pi, np.pi, (angle_rows, cols // 2))
+    table = np.empty((angle_rows, cols), np.float32)
+    table[:, ::2], table[:, 1::2] = np.cos(theta), np.sin(theta)
+    return round_bf16(table)
+
+
+@pytest.mark.parametrize("rows,cols,angle_rows", [(8, 32, 2), (1024, 32, 1), (13, 32, 13), (12, 32, 4),
+                                                  (32, 64, 1), (8, 64, 1), (2048 * 32, 64, 2048),
+                                                  (32, 512, 8), (64, 128, 16)])
+@pytest.mark.parametrize("two_halves", [True, False])
+def test_rope(cuda, rows, cols, angle_rows, two_halves):
+    rng = np.random.default_rng(0)
+    x, ang = bf(rng, rows, cols), angle_table(rng, angle_rows, cols)
+    y = out_like((rows, cols), cuda)
+    K.rope(dev(x, cuda), dev(ang, cuda), y, rows=rows, cols=cols, angle_rows=angle_rows, two_halves=two_halves)
+    want = ops.rope(x, ang, two_halves=two_halves)
+    got = from_torch(y)
+    close(got, want)
+    # Same f32 formula, one rounding: all but fused-multiply-add ties agree bit for bit.
+    assert (got != want).mean() < 0.02
+
+
+def test_rope_bound(cuda):
+    rng = np.random.default_rng(1)
+    x, ang = bf(rng, 64 * 4, 64), angle_table(rng, 64, 64)
+    y = out_like((256, 64), cuda, fill=9.0)
+    K.rope(dev(x, cuda), dev(ang, cuda), y, rows=256, cols=64, angle_rows=64, valid=word(40, cuda))
+    got = from_torch(y)
+    close(got[:40], ops.rope(x, ang)[:40])
+    assert np.all(got[40:] == 9.0)
+
+
+@pytest.mark.parametrize("n", [8192, 2048, 1003, 5, 2048 * 8192])
+def test_elementwise(cuda, n):
+    rng = np.random.default_rng(9)
+    a, b = bf(rng, n, scale=3), bf(rng, n, scale=3)
+    da, db = dev(a, cuda), dev(b, cuda)
+    y = out_like((n,), cuda)
+    K.add(da, db, y)
+    assert np.array_equal(from_torch(y), ops.add(a, b))  # bit-exact (test_elementwise.py:125-132)
+    K.mul(da, db, y)
+    assert np.array_equal(from_torch(y), ops.mul(a, b))
+    K.silu(da, y)
+    close(y, ops.silu(a))
+    K.silu_mul(da, db, y)
+    close(y, ops.mul(ops.silu(a), b), atol=2e-2)
+
+
+def test_elementwise_bound(cuda):
+    rng = np.random.default_rng(10)
+    a, b = bf(rng, 4096), bf(rng, 4096)
+    y = out_like((4096,), cuda, fill=2.0)
+    K.add(dev(a, cuda), dev(b, cuda), y, valid=word(1001, cuda))
+    got = from_torch(y)
+    assert np.array_equal(got[:1001], ops.add(a, b)[:1001]) and np.all(got[1001:] == 2.0)
+
+
+# ------------------------------------------------------------------- attention
+def run_prefill(cuda, Q, Kc, Vc, *, H, G, d, seq, seq_len, kv_len, causal=True, window=None,
+                interleaved=True, valid=None, kv_valid=None, scale=None):
+    O = out_like(Q.shape, cuda, fill=float("nan"))
+    K.mha_prefill(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, seq=seq,
+                  seq_len=seq_len, kv_len=kv_len, scale=scale, causal=causal, window=window,
+                  q_interleaved=interleaved, kv_interleaved=interleaved,
+                  valid=None if valid is None else word(valid, cuda),
+                  kv_valid=None if kv_valid is None else word(kv_valid, cuda))
+    want = ops.mha(Q, Kc, Vc, num_heads=H, num_KV_heads=G, seq_len=seq_len, kv_len=kv_len, d=d,
+                   causal=causal, window=window, scale=scale, heads_interleaved=interleaved,
+                   kv_interleaved=interleaved, valid=valid, kv_valid=kv_valid)
+    return from_torch(O), want
+
+
+@pytest.mark.parametrize("S", [512, 2048])
+def test_mha_prefill_llama_shape(cuda, S):
+    rng = np.random.default_rng(11)
+    H, G, d = 32, 8, 64
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=S, scale=0.125)
+    close(got, want)
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("causal,window", [(True, None), (True, 100), (False, 70), (False, None)])
+def test_mha_prefill_masks_and_layouts(cuda, causal, window, interleaved):
+    rng = np.random.default_rng(12)
+    H, G, d, S, L = 8, 2, 64, 192, 448
+    qs = (S, H, d) if interleaved else (H, S, d)
+    ks = (L, G, d) if interleaved else (G, L, d)
+    Q, Kc, Vc = bf(rng, *qs), bf(rng, *ks), bf(rng, *ks)
+    got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=L, causal=causal,
+                            window=window, interleaved=interleaved)
+    close(got, want)
+
+
+def test_mha_prefill_chunk_over_cache_bounded(cuda):
+    """A prompt chunk: `valid` of 256 rows at the end of `kv_valid` keys of a longer cache; NaN
+    past the bounds must not reach the output and padding rows are exactly zero
+    (test_mha_bounded_rows.py:98-102,197-225)."""
+    rng = np.random.default_rng(13)
+    H, G, d, C, L = 8, 2, 64, 256, 1024
+    rows, kv = 150, 600
+    Q, Kc, Vc = bf(rng, C, H, d), bf(rng, L, G, d), bf(rng, L, G, d)
+    Q[rows:], Kc[kv:], Vc[kv:] = np.nan, np.nan, np.nan
+    got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=C, seq_len=C, kv_len=L, valid=rows, kv_valid=kv)
+    assert np.all(got[rows:] == 0)
+    close(got[:rows], want[:rows])
+
+
+def test_mha_prefill_d128_and_ragged_seq(cuda):
+    rng = np.random.default_rng(14)
+    H, G, d, S = 6, 2, 128, 200
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=S)
+    close(got, want)
+
+
+@pytest.mark.parametrize("L", [1024, 4096, 16384])
+def test_mha_decode_llama_shape(cuda, L):
+    rng = np.random.default_rng(15)
+    H, G, d = 32, 8, 64
+    Q, Kc, Vc = bf(rng, 1, H, d), bf(rng, L, G, d), bf(rng, L, G, d)
+    O = out_like((1, H, d), cuda, fill=float("nan"))
+    ws = K.mha_decode_workspace(H, d, cuda)
+    K.mha_decode(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, kv_len=L,
+                 scale=0.125, kv_interleaved=True, workspace=ws)
+    want = ops.mha(Q, Kc, Vc, num_heads=H, num_KV_heads=G, seq_len=1, kv_len=L, d=d, scale=0.125,
+                   heads_interleaved=True, kv_interleaved=True)
+    close(O, want)
+
+
+@pytest.mark.parametrize("H,G,d", [(32, 8, 64), (8, 8, 64), (24, 8, 128), (40, 8, 64), (4, 1, 256), (16, 8, 64), (12, 2, 64), (3, 1, 64)])
+@pytest.mark.parametrize("kv_valid,window", [(1, None), (77, None), (700, None), (700, 99), (2048, 511)])
+def test_mha_decode_bounds_windows_groups(cuda, H, G, d, kv_valid, window):
+    rng = np.random.default_rng(16)
+    L = 2048
+    for interleaved in (True, False):
+        ks = (L, G, d) if interleaved else (G, L, d)
+        Q, Kc, Vc = bf(rng, 1, H, d), bf(rng, *ks), bf(rng, *ks)
+        if interleaved:
+            Kc[kv_valid:], Vc[kv_valid:] = np.nan, np.nan
+        else:
+            Kc[:, kv_valid:], Vc[:, kv_valid:] = np.nan, np.nan
+        O = out_like((1, H, d), cuda, fill=float("nan"))
+        ws = K.mha_decode_workspace(H, d, cuda)
+        K.mha_decode(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, kv_len=L,
+                     window=window, kv_interleaved=interleaved, kv_valid=word(kv_valid, cuda), workspace=ws)
+        want = ops.mha(Q, Kc, Vc, num_heads=H, num_KV_heads=G, seq_len=1, kv_len=L, d=d, window=window,
+                       heads_interleaved=True, kv_interleaved=interleaved, kv_valid=kv_valid)
+        close(O, want)
+
+
+def test_mha_decode_equals_last_row_of_prefill(cuda):
+    """A size-independent property: the one-query kernel and the last row of the many-query one agree."""
+    rng = np.random.default_rng(17)
+    H, G, d, S = 32, 8, 64, 1536
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    dQ, dK, dV = dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda)
+    O = out_like((S, H, d), cuda)
+    K.mha_prefill(dQ, dK, dV, O, heads=H, kv_heads=G, d=d, seq=S, kv_len=S, q_interleaved=True, kv_interleaved=True)
+    o1 = out_like((1, H, d), cuda)
+    K.mha_decode(dQ[S - 1 :].contiguous(), dK, dV, o1, heads=H, kv_heads=G, d=d, kv_len=S, kv_interleaved=True,
+                 workspace=K.mha_decode_workspace(H, d, cuda))
+    close(from_torch(o1)[0], from_torch(O)[S - 1], rtol=1e-2, atol=1e-2)
+
+
+# ------------------------------------------------------------------------ glue
+def test_gather_rows_exact(cuda):
+    rng = np.random.default_rng(18)
+    table = bf(rng, 1000, 2048)
+    ids = rng.integers(0, 1000, 300).astype(np.int32)
+    out = out_like((300, 2048), cuda, fill=1.0)
+    K.gather_rows(dev(table, cuda), torch.from_numpy(ids).to(cuda), out, valid=word(256, cuda))
+    got = from_torch(out)
+    assert np.array_equal(got[:256], ops.gather_rows(table, ids[:256])) and np.all(got[256:] == 1.0)
+    # int32 rows, a row width that is not a multiple of 16 bytes.
+    t32 = torch.arange(50 * 3, dtype=torch.int32, device=cuda).reshape(50, 3)
+    o32 = torch.zeros((4, 3), dtype=torch.int32, device=cuda)
+    K.gather_rows(t32, torch.tensor([7, 0, 49, 7], dtype=torch.int32, device=cuda), o32)
+    assert torch.equal(o32.cpu(), t32.cpu()[[7, 0, 49, 7]])
+
+
+def test_copy_rows_cache_write_table_row_and_last_row(cuda):
+    rng = np.random.default_rng(19)
+    L, G, d = 128, 8, 64
+    cache = dev(np.zeros((L, G * d), np.float32), cuda)
+    k = bf(rng, 1, G * d)
+    K.copy_rows(dev(k, cuda), cache, rows=1, row_elems=G * d, src_rows=1, dst_rows=L, dst_row=word(37, cuda))
+    got = from_torch(cache)
+    assert np.array_equal(got[37], k[0]) and np.count_nonzero(got) == np.count_nonzero(k)
+    # A chunk of rows at a per-call start, bounded.
+    x = bf(rng, 32, G * d)
+    K.copy_rows(dev(x, cuda), cache, rows=32, row_elems=G * d, src_rows=32, dst_rows=L,
+                dst_row=word(64, cuda), valid=word(20, cuda))
+    got = from_torch(cache)
+    assert np.array_equal(got[64:84], x[:20]) and np.all(got[84:] == 0)
+    # The last valid row picked out (src index), and a row past the end skipped.
+    last = out_like((1, G * d), cuda, fill=4.0)
+    K.copy_rows(dev(x, cuda), last, rows=1, row_elems=G * d, src_rows=32, dst_rows=1, src_row=word(19, cuda))
+    assert np.array_equal(from_torch(last)[0], x[19])
+    K.copy_rows(dev(x, cuda), last, rows=1, row_elems=G * d, src_rows=32, dst_rows=1, src_row=word(32, cuda))
+    assert np.array_equal(from_torch(last)[0], x[19])
+
+
+def test_argmax_first_of_ties_and_record(cuda):
+    rng = np.random.default_rng(11)
+    logits = round_bf16(rng.normal(0, 3, 128256))
+    top = rng.choice(128256, 8, replace=False)
+    logits[top] = logits.max()
+    tok = torch.full((1,), -1, dtype=torch.int32, device=cuda)
+    rec = torch.full((16,), -1, dtype=torch.int32, device=cuda)
+    K.argmax(dev(logits, cuda), tok, record=rec, at=word(5, cuda))
+    assert int(tok.item()) == ops.argmax(logits) == int(top.min())
+    assert rec.cpu().tolist() == [-1] * 5 + [int(top.min())] + [-1] * 10
+    odd = round_bf16(rng.normal(0, 1, 1003))
+    K.argmax(dev(odd, cuda), tok)
+    assert int(tok.item()) == ops.argmax(odd)
+
+
+def test_eval_words_advances_a_decode_step(cuda):
+    words = torch.tensor([11, 40, 0, 0, 0, 0, 0, 0], dtype=torch.int32, device=cuda)
+    # position += 1; kv_valid = position + 1; rope_row = min(position, 5); half = position >> 1
+    exprs = torch.tensor([[1, 1, 1, 1, 0, -(2**31), 2**31 - 1], [2, 1, 1, 1, 0, -(2**31), 2**31 - 1],
+                          [3, 1, 1, 0, 0, 0, 5], [4, 1, 1, 0, 1, -(2**31), 2**31 - 1]], dtype=torch.int32, device=cuda)
+    K.eval_words(words, exprs)
+    assert words.cpu().tolist() == [11, 41, 42, 5, 20, 0, 0, 0]
