@@ -8,3 +8,18 @@ float32 numpy arrays holding bf16-representable values (``iron_amd.bf16``).
 from .bf16 import bfloat16, round_bf16  # noqa: F401
 
 __version__ = "0.1.0"
+
+
+_LAZY = dict.fromkeys(
+    ["Carried", "CompiledGraph", "Graph", "Scratchpad", "carry", "clamp", "param", "state", "weight"],
+    "iron_amd.common.graph",
+) | dict.fromkeys(["Precision"], "iron_amd.common.declare")
+
+
+def __getattr__(name):
+    import importlib
+
+    module = _LAZY.get(name)
+    if module is None:
+        raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+    return getattr(importlib.import_module(module), name)

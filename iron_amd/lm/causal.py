@@ -1,0 +1,216 @@
+"""A decoder-only language model on the GPU, as one graph (iron/lm/causal.py:40-508).
+
+A call with no tensor is a decode step; ``prefill_chunk`` token ``ids`` are a prompt chunk
+from ``start``, of which a call runs the first ``rows``.  Both draw the next token on the
+device and carry it and ``position + 1`` into the next call.  The decode step is captured
+in a HIP graph that carries its own values, so a run of decode steps is a run of replays.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import time
+from collections.abc import Iterator
+from typing import Any
+
+import numpy as np
+
+from ..common import graph as iron
+from ..common.graph import Carried, Scratchpad
+from ..operators.copy import Copy
+from ..operators.sample import ROW_WORDS, Sample
+from .blocks import DecoderLayer, Embedding, Linear, RMSNorm, Rope
+from .config import DecoderConfig
+from .session import Session
+
+
+@dataclasses.dataclass(kw_only=True)
+class Call:
+    """One call's values, built once in ``body`` and read by every memory module
+    (``KVCache``, ``Rope``): a prompt chunk's ``rows`` from ``start``, or the decode step's
+    one at ``position``."""
+
+    prompt: bool
+    start: Any
+    rows: Any
+    position: Any
+    rope_start: Any = None
+    ropes: dict = dataclasses.field(default_factory=dict)
+    ids: Any = None
+    token: Any = None
+    embeddings: Any = None
+
+
+@dataclasses.dataclass
+class Stats:
+    """What a generation measured: seconds to the first token, tokens per second after it."""
+
+    ttft: float = 0.0
+    tokens_per_s: float = 0.0
+    tokens: int = 0
+
+
+class Decoder(iron.Graph):
+    """A decoder's modules as a checkpoint's ``model`` names them."""
+
+    def __init__(self, c: DecoderConfig, layer=DecoderLayer):
+        self.embed_tokens = Embedding(c.vocab_size, c.hidden_size)
+        self.layers = [layer(c, i) for i in range(c.num_hidden_layers)]
+        self.norm = RMSNorm(c.hidden_size, c.eps)
+
+
+class CausalLM(iron.Graph):
+    """A decoder on ``config``'s shape: ``model``, ``lm_head`` and ``rotary_emb``."""
+
+    decoder_class = Decoder
+    layer_class = DecoderLayer
+
+    def __init__(self, config: DecoderConfig, weights):
+        self.config = config
+        self.rotary_emb = None if config.rope_theta is None else Rope(config)
+        # Zero until the host writes draws: a row of zeros is greedy.
+        self.draws = iron.state((config.max_seq_len, ROW_WORDS), np.int32)
+        self.drawn = iron.state((config.max_seq_len,), np.int32)
+        self.prompt_chunk = None
+        self.decode_step = None
+        self.holder = None
+        self.session = Session(self)
+        self.stats = Stats()
+        self.model = self.decoder_class(config, self.layer_class)
+        for layer in self.model.layers:
+            layer.rope = self.rotary_emb
+        self.lm_head = Linear(config.hidden_size, config.vocab_size, False, precision=config.precision)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.model.embed_tokens.weight
+        self.load_state_dict(weights)
+        self.layers = self.model.layers
+
+    @property
+    def recurrent(self) -> list:
+        """States that restart only at some positions (ring caches): none in this build."""
+        return []
+
+    def head(self, x):
+        """The final norm, then the output head (the embedding, if tied)."""
+        return self.lm_head(self.model.norm(x))
+
+    def lookup(self, ids):
+        return self.model.embed_tokens(ids)
+
+    def body(self, ids=None, *, token: Carried[np.int32], position: Carried[np.int32],
+             start: Scratchpad[np.int32] = np.int32(0), rows: Scratchpad[np.int32] = np.int32(1),
+             rope_start: Scratchpad[np.int32] = np.int32(0)):
+        prompt = ids is not None
+        call = Call(prompt=prompt, start=start if prompt else position, rows=rows, position=position,
+                    rope_start=rope_start, ids=ids[:rows] if prompt else token, token=token)
+        if prompt:
+            return self.forward(self.lookup(call.ids), call)
+        return self.forward(self.lookup(token).reshape(1, self.config.hidden_size), call)
+
+    def forward(self, x, call: Call):
+        """The layers, the head and the draw over ``x``, the rows ``call`` runs."""
+        c = self.config
+        call.embeddings = x
+        for rope in (layer.rope for layer in self.layers):
+            if rope is not None and id(rope) not in call.ropes:
+                call.ropes[id(rope)] = rope.rows(call)
+        for layer in self.layers:
+            x = layer(x, call)
+        if call.prompt:
+            x = Copy.step(x[call.rows - 1]).reshape(1, c.hidden_size)  # the last row's logits alone
+        return self.draw(self.head(x), call)
+
+    def draw(self, logits, call: Call):
+        """``logits`` and the token drawn from them on the device, carried with the next position."""
+        c = self.config
+        _, drawn = Sample.step(logits.reshape(c.vocab_size), self.draws, self.drawn,
+                               row=call.position * ROW_WORDS, at=call.position, drawable=c.vocab_size)
+        return logits, iron.carry(token=drawn, position=call.position + 1)
+
+    # -- versions ------------------------------------------------------------
+    def shapes(self) -> list[dict]:
+        """The input shapes of each version: the decode step's (none), then the prompt chunk's ids."""
+        return [{}, dict(ids=((self.config.prefill_chunk,), np.int32))]
+
+    def load_versions(self, *, capture: bool = True, check: bool = False) -> None:
+        """Compile the decode step and the prompt chunk into one arena and load them."""
+        decode_shapes, prompt_shapes = self.shapes()
+        try:
+            decode = self.compile(capture=capture, check=check, **decode_shapes)
+            prompt = self.compile(capture=False, check=check, **prompt_shapes)
+            decode.load()
+            prompt.load()
+        except Exception:
+            self.release()
+            raise
+        self.use(decode, prompt)
+
+    def use(self, decode, prompt) -> None:
+        self.decode_step, self.prompt_chunk = decode, prompt
+        self.holder = None
+
+    def release(self) -> None:
+        self.decode_step = self.prompt_chunk = None
+        super().release()
+
+    def __call__(self, ids=None, **values):
+        """One call of the prompt version or else the decode step."""
+        if iron.graph_recorder.get() is not None:
+            return super().__call__(ids, **values)
+        if self.decode_step is None:
+            raise RuntimeError(f"{type(self).__name__}: load_versions() first")
+        if ids is None:
+            return self.decode_step(**values)
+        return self.prompt_chunk(ids, **values)
+
+    def logits(self, tokens) -> np.ndarray:
+        """The logits after the last of ``tokens``, the whole history (``Session.logits``)."""
+        return self.session.logits(tokens)
+
+    def generate(self, tokens, max_tokens: int) -> list[int]:
+        """Greedy: ``max_tokens`` tokens drawn on the device after ``tokens``; fills ``stats``."""
+        return list(self.stream(tokens, max_tokens))
+
+    def stream(self, tokens, max_tokens: int) -> Iterator[int]:
+        t0 = time.perf_counter()
+        first = None
+        n = 0
+        for token in self.session.draw(tokens, max_tokens):
+            n += 1
+            if first is None:
+                first = time.perf_counter()
+            yield token
+        end = time.perf_counter()
+        self.stats = Stats(ttft=(first or end) - t0,
+                           tokens_per_s=(n - 1) / (end - first) if n > 1 and end > first else 0.0, tokens=n)
+
+
+class _HostOutput:
+    def __init__(self, array):
+        self.array = array
+
+    def numpy(self):
+        return self.array
+
+
+class _HostVersion:
+    """A version stood in by the graph's host reference: same call, numpy underneath."""
+
+    captured = False
+
+    def __init__(self, graph, takes_ids: bool):
+        self.graph, self.takes_ids = graph, takes_ids
+
+    def __call__(self, *tensors, **values):
+        outs, carried = iron.Graph.reference(self.graph, *tensors, **values)
+        return (*(_HostOutput(o) for o in outs), iron.Carry(carried))
+
+
+class OnHost:
+    """Mix-in: the model with its compiled versions replaced by ``Graph.reference``, which runs
+    the graph operator by operator on host arrays with the caches as state -- the fake backend
+    of the device-free model tests (iron/lm/model.py:667-695).  Needs a registered CPU
+    reference for every operator (the test oracle)."""
+
+    def load_versions(self, **_):
+        self.use(_HostVersion(self, False), _HostVersion(self, True))

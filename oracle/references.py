@@ -1,0 +1,78 @@
+"""The operators' ``reference()`` methods, restated on ``oracle.ops`` -- TEST INFRASTRUCTURE.
+
+``install()`` registers one function per operator class into
+``iron_amd.common.declare.REFERENCES``; each takes the constructed operator and its
+inputs as numpy arrays, as the reference's methods do (file:line cited per function).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from . import ops
+
+
+def gemm(op, A, B):
+    """iron/operators/gemm.py:696-702."""
+    return ops.gemm(A, B, b_col_maj=op.b_col_maj, c_col_maj=op.c_col_maj, valid_k=op.valid_k)
+
+
+def gemv(op, A, B):
+    """iron/operators/gemv.py:408-417."""
+    return ops.gemv(A, B, repeat=op.repeat)
+
+
+def rms_norm(op, x, weight=None):
+    """iron/common/elementwise.py:676-682 over norm.rms_norm_eps."""
+    return ops.rms_norm(np.asarray(x).reshape(op.rows, op.tile_size), weight, epsilon=op.epsilon)
+
+
+def silu(op, x):
+    return ops.silu(x)
+
+
+def mul(op, a, b):
+    return ops.mul(a, np.asarray(b).reshape(np.shape(a)))
+
+
+def add(op, a, b):
+    return ops.add(a, np.asarray(b).reshape(np.shape(a)))
+
+
+def rope(op, x, angles):
+    """iron/operators/rope.py:167-184."""
+    return ops.rope(x, angles, two_halves=op.two_halves)
+
+
+def mha(op, Q, K, V):
+    """iron/operators/mha.py:1073-1116; a bounded call's extents read off the operator."""
+    ext = vars(op).get("_extents", {})
+    return ops.mha(Q, K, V, num_heads=op.num_heads, num_KV_heads=op.num_KV_heads, seq_len=op.seq_len,
+                   kv_len=op.kv_len, d=op.d, causal=op.causal, window=op.window, scale=op.scale,
+                   heads_interleaved=op.heads_interleaved, kv_interleaved=op.kv_interleaved,
+                   valid=ext.get("valid"), kv_valid=ext.get("kv_valid"))
+
+
+def copy(op, src):
+    """iron/operators/copy.py:839-902: exact."""
+    return np.array(src).reshape(op.shape)
+
+
+def sample(op, logits, draws, tokens, *, row=0, at=0):
+    """iron/operators/sample.py:324-333; only the greedy draw (an all-zero row) is restated."""
+    words = np.asarray(draws).reshape(-1)[row : row + 4]
+    if np.any(words != 0):
+        raise NotImplementedError("the oracle restates the greedy draw only (an all-zero draw row)")
+    token = ops.argmax(np.asarray(logits).reshape(-1)[: op.drawable])
+    tokens = np.array(tokens, dtype=np.int32).reshape(-1)
+    tokens[at] = token
+    return tokens, np.array([token], dtype=np.int32)
+
+
+def install() -> None:
+    from iron_amd.common.declare import REFERENCES
+
+    REFERENCES.update(
+        GEMM=gemm, GEMV=gemv, RMSNorm=rms_norm, SiLU=silu, ElementwiseMul=mul, ElementwiseAdd=add,
+        RoPE=rope, MHA=mha, Copy=copy, Sample=sample,
+    )
