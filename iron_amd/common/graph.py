@@ -456,6 +456,9 @@ class Limit:
     expr: Affine
     lo: int
     hi: int  # inclusive
+    # A bounded window: the rows a call touches from `expr` on, which must end within `rows`.
+    span: Affine | None = None
+    rows: int = 0
 
 
 class Recorder:
@@ -558,7 +561,11 @@ class Recorder:
         for name, h in {**inputs, **outputs}.items():
             if h.index is not None:
                 width = max(h.elements // h.index_stride, 1)  # rows the view spans
-                self.limits.append(Limit(f"{cls.__name__}.{name}", h.index, 0, h.index_rows - width))
+                if 0 in h.valid:  # only the bounded rows are touched
+                    self.limits.append(Limit(f"{cls.__name__}.{name}", h.index, 0, h.index_rows - 1,
+                                             span=h.valid[0], rows=h.index_rows))
+                else:
+                    self.limits.append(Limit(f"{cls.__name__}.{name}", h.index, 0, h.index_rows - width))
             if 0 in h.valid:
                 self.limits.append(Limit(f"{cls.__name__}.{name}[:n]", h.valid[0], 0, h.shape[0]))
         self.steps.append(Step(op, inputs, outputs, bound))
@@ -774,6 +781,9 @@ class Recording:
             if not lim.lo <= got <= lim.hi:
                 raise IndexError(f"{self.name}: {lim.what} = {got} ({lim.expr.name}) is outside "
                                  f"[{lim.lo}, {lim.hi}]")
+            if lim.span is not None and got + lim.span.evaluate(full) > lim.rows:
+                raise IndexError(f"{self.name}: {lim.what}: {lim.span.evaluate(full)} rows from {got} "
+                                 f"({lim.expr.name}) end outside {lim.rows}")
         return full
 
     def transients(self) -> list[tuple[Buffer, int, int]]:
@@ -1031,7 +1041,10 @@ class CompiledGraph:
                     self._slot(h.ids.valid[0])
         if len(self.slots) + len(self.exprs) > WORD_SLOTS:
             raise ValueError(f"{graph.name}: more than {WORD_SLOTS} per-call words")
-        self.words_offset = pool.place(LiveRange(WORD_SLOTS * 4 + WORD_SLOTS * 7 * 4, -1, len(recording.steps) + 1))
+        # The words and the expression table outlive a call (a replay starts from the last
+        # one's values; the table is written once), so they are residents of this version.
+        self._words_resident = State((WORD_SLOTS * 8,), np.int32)
+        arena.place_resident(self._words_resident)
         arena.reserve_transients(pool.size)
         self._loaded_generation = None
         self._graph = None
@@ -1070,7 +1083,7 @@ class CompiledGraph:
         self.arena.load()
         if self._loaded_generation == self.arena.generation:
             return self
-        base = self.arena.resident_bytes + self.words_offset
+        base = self.arena.resident_offsets[id(self._words_resident)]
         self.words = self.arena.view(base, (WORD_SLOTS,), np.int32)
         self.expr_table = self.arena.view(base + WORD_SLOTS * 4, (WORD_SLOTS * 7,), np.int32)
         self.host_words = torch.zeros(WORD_SLOTS, dtype=torch.int32).pin_memory()
@@ -1282,8 +1295,9 @@ class CompiledGraph:
             values = {k: e.evaluate(full) for k, e in step.values.items()}
             extents = {k: v for k, v in values.items()
                        if next(m for m in op.declaration.per_calls if m.name == k).bounds is not None}
+            others = {k: v for k, v in values.items() if k not in extents}
             at = op._at_extents(**extents) if extents else op
-            verdicts = at.judge(ins, written, tol)
+            verdicts = at.judge(ins, written, tol, at._call_reference(ins, values=others))
             bad = {n: v.detail for n, v in verdicts.items() if not v}
             if bad:
                 raise AssertionError(f"{self.recording.name}: step {op.name}: {bad}")
