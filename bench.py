@@ -115,11 +115,120 @@ def cpu_gemv_baseline(rng, budget_s=12.0):
             "kind": "port", "sample": f"{calls} oracle GEMV calls over K->N {sample}, {total_s:.1f} s wall"}
 
 
+def llama_weights(torch, config, dev, seed=0):
+    """Random-init weights of ``config``'s shape on the GPU: matrices N(0, 0.02), norm gains 1, bf16."""
+    from iron_amd.applications.llama import shapes
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    out = {}
+    for name, shape in shapes(config).items():
+        if len(shape) >= 2:
+            w = torch.randn(shape, generator=g, device=dev, dtype=torch.float32).mul_(0.02)
+            out[name] = w.to(torch.bfloat16)
+            del w
+        else:
+            out[name] = torch.ones(shape, device=dev, dtype=torch.bfloat16)
+    return out
+
+
+def bench_decoder(torch, dev, steps, warmup, with_cpu):
+    """Llama-3.2-1B shape: a 512-token prompt prefill, then ``steps`` greedy decode steps as
+    replays of the captured decode step (each starts from the token and position the last one
+    carried on the device)."""
+    import dataclasses
+
+    from iron_amd.applications.llama import LLAMA_3_2_1B, Llama
+
+    config = dataclasses.replace(LLAMA_3_2_1B, max_seq_len=2048, prefill_chunk=2048)
+    weights = llama_weights(torch, config, dev)
+    model = Llama(config, weights)
+    model.load_versions()
+    prompt = np.random.default_rng(512).integers(0, config.vocab_size, 512)
+    session, decode = model.session, model.decode_step
+
+    def prefill():
+        carry = None
+        for inputs, values in session._chunks(prompt, 0):
+            _, carry = model(*inputs, **values)
+        return carry
+
+    carry = prefill()
+    decode.start(**carry)
+    decode.replay(max(warmup, 1))
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    carry = prefill()
+    torch.cuda.synchronize()
+    ttft = time.perf_counter() - t0
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    decode.start(**carry)
+    decode.replay(steps - 1)
+    stop.record()
+    stop.synchronize()
+    wall = time.perf_counter() - t0
+    ms = start.elapsed_time(stop)
+    tokens = decode.read(model.drawn)[512 : 512 + steps]
+    weight_bytes = 2 * (sum(int(np.prod(s)) for n, s in __import__("iron_amd.applications.llama", fromlist=["shapes"]).shapes(config).items()
+                            if "embed" not in n) + config.vocab_size * config.hidden_size)
+    kv_bytes = sum((512 + 1 + i) * 2 * config.num_key_value_heads * config.head_dim * 2 * config.num_hidden_layers
+                   for i in range(steps)) / steps
+    per_token = weight_bytes + kv_bytes
+    tok_s = steps / (ms / 1e3)
+    out = {"tok_s": round(tok_s, 1), "ms_per_token": round(ms / steps, 4), "ttft_ms": round(ttft * 1e3, 2),
+           "prefill_tokens": 512, "decode_steps": steps, "wall_s": round(wall, 4),
+           "bytes_per_token": int(per_token), "GBps": round(per_token * tok_s / 1e9, 1),
+           "frac_hbm": round(per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
+           "kernels_per_step": len(decode.recording.steps), "first_tokens": [int(t) for t in tokens[:4]]}
+    cpu = None
+    if with_cpu:
+        cpu = cpu_decoder_baseline(torch, config, weights)
+    model.release()
+    return out, cpu
+
+
+def cpu_decoder_baseline(torch, config, weights, budget_s=12.0):
+    """The oracle's graph reference (the reference's CPU path: the graph run step by step through
+    each operator's numpy reference) timed on the host cores for a few decode steps of the same
+    16-layer model at position 512 (the prompt is not prefilled on the CPU: the cost of a decode
+    step does not depend on what the cache holds)."""
+    import oracle
+    from iron_amd.applications.llama import Llama
+    from iron_amd.bf16 import from_torch
+    from iron_amd.lm.causal import OnHost
+
+    oracle.install()
+
+    class HostLlama(OnHost, Llama):
+        pass
+
+    host_weights = {n: from_torch(t) for n, t in weights.items()}
+    model = HostLlama(config, host_weights)
+    model.load_versions()
+    carry = {"token": 1, "position": 512}
+    _, carry = model(**carry)  # records the graph and warms the caches
+    t0 = time.perf_counter()
+    steps = 0
+    while time.perf_counter() - t0 < budget_s and carry["position"] < config.max_seq_len - 1:
+        _, carry = model(**carry)
+        steps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(steps / dt, 3), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{steps} decode steps at positions 513.. of the same 16-layer model through the oracle's "
+                      f"graph reference, {dt:.1f} s wall; weights held as float32, prompt not prefilled on the CPU"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=128, help="timed decode steps (tokens)")
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--kernel-launches", type=int, default=400, help="timed launches per kernel micro-benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -149,9 +258,12 @@ def main():
     torch.cuda.synchronize()
 
     t_wall = time.perf_counter()
-    gemv = [bench_gemv(torch, K, dev, Kd, N, args.steps, rng) for Kd, N in GEMV_SWEEP]
-    gemm = [bench_gemm(torch, K, dev, args.steps, rng, b) for b in (False, True)]
+    n = args.kernel_launches
+    gemv = [bench_gemv(torch, K, dev, Kd, N, n, rng) for Kd, N in GEMV_SWEEP]
+    gemm = [bench_gemm(torch, K, dev, n, rng, b) for b in (False, True)]
     torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    decoder, cpu = bench_decoder(torch, dev, args.steps, args.warmup, not args.no_cpu)
     wall = time.perf_counter() - t_wall
 
     sweep_bytes = sum(g["bytes"] for g in gemv)
@@ -159,28 +271,34 @@ def main():
     head = gemv[-1]
     out = {
         "metric": "bf16 GEMM TFLOP/s, GEMV GB/s (% roofline); Llama-3.2-1B-shape decode tok/s",
-        "value": round(sweep_bytes / sweep_us / 1e3, 1),
-        "unit": "GB/s",
+        "value": decoder["tok_s"],
+        "unit": "tok/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(sweep_us / 1e3, 4),
+        "ms_per_step": decoder["ms_per_token"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "decode GEMV sweep K->N 2048->2048, 2048->512, 2048->8192, 8192->2048, "
-                               "2048->128256 (batch 1, bf16, f32 accumulation); one step = the five GEMVs"},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel (2048->128256 LM head)",
+        "config": {"workload": "Llama-3.2-1B-shape decoder (16 layers, hidden 2048, 32 q / 8 kv heads, head_dim 64, "
+                               "SwiGLU 8192, vocab 128256, tied embeddings), random-init bf16 N(0,0.02), batch 1: "
+                               "512-token prompt prefill, then greedy decode steps replayed as a HIP graph; "
+                               "one step = one decoded token",
+                   "prefill_tokens": 512, "decode_steps": args.steps},
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<4,1> (the 2048->128256 LM head, the largest launch of a "
+                                               "decode step)",
                      "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["frac_hbm"], "traffic": None},
-        "gemv": gemv,
+        "decoder": decoder,
+        "gemv_sweep": {"GBps": round(sweep_bytes / sweep_us / 1e3, 1), "shapes": gemv},
         "gemm": gemm,
         "bench_wall_s": round(wall, 1),
     }
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_gemv_baseline(np.random.default_rng(7))
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+        out["cpu_baseline_gemv"] = cpu_gemv_baseline(np.random.default_rng(7), budget_s=6.0)
     print(json.dumps(out))
     return 0
 

@@ -654,8 +654,14 @@ class Graph:
         bound: dict[int, Param] = {}
         for paths in tied.values():
             p = params[paths[0]]
-            a = np.asarray(tensors[paths[0]])
-            a = round_bf16(a) if p.dtype is bfloat16 else a.astype(p.dtype)
+            a = tensors[paths[0]]
+            if _is_torch(a):  # a bf16 tensor (host or device) is taken as it is
+                want = "torch.bfloat16" if p.dtype is bfloat16 else f"torch.{np.dtype(p.dtype).name}"
+                if str(a.dtype) != want:
+                    raise ValueError(f"{self.name}: cannot load: wrong kind {paths[0]} {a.dtype}, not {want}")
+            else:
+                a = np.asarray(a)
+                a = round_bf16(a) if p.dtype is bfloat16 else a.astype(p.dtype)
             bound_param = Param(p.shape, p.dtype, a)
             for n, x, parent, key in walk(self):
                 if x is p:
@@ -751,6 +757,10 @@ class Graph:
         return recording.reference({n: np.asarray(t) for n, t in given.items() if t is not None}, values)
 
 
+def _is_torch(x) -> bool:
+    return type(x).__module__.startswith("torch")
+
+
 def _host_dtype(t):
     a = np.asarray(t)
     return bfloat16 if a.dtype == np.float32 else a.dtype.type
@@ -815,6 +825,8 @@ class Recording:
                 r = b.source
                 if getattr(r, "host", None) is None:
                     init = r.array if r.array is not None else np.zeros(r.shape, _np_dtype(r.dtype))
+                    if _is_torch(init):
+                        init = from_torch(init)
                     r.host = np.array(init, dtype=_np_dtype(r.dtype)).reshape(-1)
                 host[id(b)] = r.host
             elif b.kind == "input":
@@ -986,6 +998,8 @@ class ScratchArena:
 def _host_tensor(array, dtype):
     import torch
 
+    if isinstance(array, torch.Tensor):
+        return array
     if dtype is bfloat16:
         return torch.from_numpy(to_bits(array).view(np.int16)).view(torch.bfloat16)
     return torch.from_numpy(np.ascontiguousarray(array, dtype=dtype))
