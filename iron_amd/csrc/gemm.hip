@@ -269,6 +269,174 @@ __global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A,
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// Fast path: A (M,K) and B (N,K) both K-contiguous, K a multiple of 64, row-major C.
+//
+// Tiles stream global -> LDS directly (global_load_lds_dwordx4: no VGPR staging, and the
+// L2 -> CU path delivers more per clock to LDS than to registers), four 32 KB stages deep.
+// A wave instruction moves 8 rows x 128 B; the 16-byte chunk a lane fetches is XOR-swizzled
+// by its row ((row >> 1) & 7) so the fragment reads of 16 consecutive rows fall in distinct
+// bank groups although LDS rows are unpadded.  The stage barrier is a bare s_barrier: the
+// fence __syncthreads() carries would wait for every outstanding load (vmcnt(0)) and drain
+// the prefetch; each wave instead waits until only the two youngest stages are in flight.
+// Blocks are ordered so each XCD (block id mod 8) owns 8x4-tile patches and re-reads its
+// A/B panels from its own L2.
+#define IRON_GLOBAL_PTR(p) ((const void __attribute__((address_space(1)))*)(p))
+#define IRON_LDS_PTR(p) ((void __attribute__((address_space(3)))*)(p))
+
+__device__ __forceinline__ void block_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // gfx9 encoding: vmcnt = bits [3:0] and [15:14]; expcnt and lgkmcnt left at "no wait".
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+constexpr int NT_BM = 128, NT_BN = 128, NT_STAGES = 4;
+constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
+
+__global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
+                                                      const bf16_t* __restrict__ B,
+                                                      bf16_t* __restrict__ C, int M, int N, int K,
+                                                      const int* __restrict__ valid, int tiles_m,
+                                                      int tiles_n, int patched) {
+  constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
+  constexpr int LOADS = 2 * INST;
+  extern __shared__ __align__(16) char smem_nt[];
+  const int Mv = bound_or(valid, M);
+
+  int tm, tn;
+  const int bid = blockIdx.x;
+  if (patched) {
+    const int xcd = bid & 7, loc = bid >> 3;
+    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
+    const int patches_n = tiles_n >> 2;
+    tm = (patch / patches_n) * 8 + (within & 7);
+    tn = (patch % patches_n) * 4 + (within >> 3);
+  } else {
+    constexpr int BAND = 8;
+    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
+    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
+    tm = first + in_band % height;
+    tn = in_band / height;
+  }
+  const int m0 = tm * NT_BM, n0 = tn * NT_BN;
+  if (m0 >= Mv) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane >> 3, pch = lane & 7;
+  const bf16_t* a_src[INST];
+  const bf16_t* b_src[INST];
+#pragma unroll
+  for (int i = 0; i < INST; ++i) {
+    const int r = (wave * INST + i) * 8 + lrow;
+    const int lch = pch ^ ((r >> 1) & 7);
+    // Rows past the end re-read the last row; what they produce is never stored.
+    a_src[i] = A + (size_t)min(m0 + r, M - 1) * K + lch * 8;
+    b_src[i] = B + (size_t)min(n0 + r, N - 1) * K + lch * 8;
+  }
+  auto issue = [&](int kt) {
+    char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < INST; ++i)
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_src[i] + k0),
+                                       IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < INST; ++i)
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(b_src[i] + k0),
+                                       IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + i) * 1024), 16, 0, 0);
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int s = 0; s < NT_STAGES - 1; ++s)
+    if (s < nk) issue(s);
+
+  const int fr = lane & 31, kh = lane >> 5;
+  int a_off[2], a_swz[2], b_off[2], b_swz[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int ra = wm * 64 + i * 32 + fr, rb = wn * 64 + i * 32 + fr;
+    a_off[i] = ra * 128; a_swz[i] = (ra >> 1) & 7;
+    b_off[i] = NT_A_BYTES + rb * 128; b_swz[i] = (rb >> 1) & 7;
+  }
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // Stage kt has landed once at most the two younger stages' loads are outstanding.
+    if (kt + NT_STAGES - 2 < nk) wait_vmcnt<(NT_STAGES - 2) * LOADS>(); else wait_vmcnt<0>();
+    block_barrier();  // everyone's loads of stage kt are in; everyone is done reading stage kt-1
+    if (kt + NT_STAGES - 1 < nk) issue(kt + NT_STAGES - 1);  // into the buffer of stage kt-1
+    const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      const int j = ks * 2 + kh;
+      bf16x8 af[2], bfr[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        af[i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
+        bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_off[i] + ((j ^ b_swz[i]) << 4));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[jj], af[i], acc[i][jj], 0, 0, 0);
+    }
+  }
+
+  const int hi = kh * 4;
+  const bool vec = (N & 3) == 0;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = m0 + wm * 64 + i * 32 + fr, nb = n0 + wn * 64 + j * 32;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = nb + 8 * q + hi;
+        if (m >= Mv || n >= N) continue;
+        bf16_t* p = C + (size_t)m * N + n;
+        if (vec && n + 4 <= N) {
+          *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
+                                                    pack_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
+        } else {
+          for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(acc[i][j][4 * q + e]);
+        }
+      }
+    }
+}
+
+static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
+                          const int* valid, hipStream_t s) {
+  const int tiles_m = (M + NT_BM - 1) / NT_BM, tiles_n = (N + NT_BN - 1) / NT_BN;
+  const size_t lds = (size_t)NT_STAGES * NT_STAGE_BYTES;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
+  hipLaunchKernelGGL(gemm_nt_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
+                     valid, tiles_m, tiles_n, patched);
+  IRON_LAUNCH_CHECK();
+}
+
 template <int BM, int BN, int WM, int WN>
 static int launch_gemm(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K, int b_nk,
                        int c_nm, const int* valid, const int* valid_k, hipStream_t s) {
@@ -311,6 +479,8 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   IRON_REQUIRE(b_col_maj || N % 8 == 0,
                "gemm: N (%d) must be a multiple of 8 when B is (K,N) (16-byte loads along N)", N);
   hipStream_t s = (hipStream_t)stream;
+  if (b_col_maj && !c_col_maj && valid_k == nullptr && K % BK == 0 && M >= 64 && N >= 64)
+    return launch_gemm_nt(A, B, C, M, N, K, valid, s);
   // 128x128 tiles fill the 256 CUs once at 2048x2048; narrower problems take 64-wide tiles.
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
   if (tiles128 >= 128 || (M >= 128 && N >= 128))
