@@ -299,6 +299,13 @@ __device__ __forceinline__ void wait_vmcnt() {
 constexpr int NT_BM = 128, NT_BN = 128, NT_STAGES = 4;
 constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
 
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+// B_KN: B is (K,N) row-major.  Its tile lands in LDS as stored, [64 k][128 n] (a wave
+// instruction moves 4 k-rows x 256 B, chunks swizzled by 2*(k & 7)), and the fragments are
+// fetched with the transposing LDS read (ds_read_b64_tr_b16): within 16 lanes, lane i points
+// at 4 consecutive n of row k0 + i/4 and receives k0..k0+3 of column n0 + i%16.
+template <bool B_KN>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
                                                       const bf16_t* __restrict__ B,
                                                       bf16_t* __restrict__ C, int M, int N, int K,
@@ -338,7 +345,13 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     const int lch = pch ^ ((r >> 1) & 7);
     // Rows past the end re-read the last row; what they produce is never stored.
     a_src[i] = A + (size_t)min(m0 + r, M - 1) * K + lch * 8;
-    b_src[i] = B + (size_t)min(n0 + r, N - 1) * K + lch * 8;
+    if constexpr (!B_KN) {
+      b_src[i] = B + (size_t)min(n0 + r, N - 1) * K + lch * 8;
+    } else {
+      const int kr = (wave * INST + i) * 4 + (lane >> 4);       // k row of the tile
+      const int lc = (lane & 15) ^ ((kr & 7) << 1);               // logical 16-byte chunk (8 n)
+      b_src[i] = B + (size_t)kr * N + n0 + lc * 8;
+    }
   }
   auto issue = [&](int kt) {
     char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
@@ -349,7 +362,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                        IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < INST; ++i)
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(b_src[i] + k0),
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(b_src[i] + (B_KN ? (size_t)k0 * N : (size_t)k0)),
                                        IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + i) * 1024), 16, 0, 0);
   };
 
@@ -374,6 +387,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     a_off[i] = ra * 128; a_swz[i] = (ra >> 1) & 7;
     b_off[i] = NT_A_BYTES + rb * 128; b_swz[i] = (rb >> 1) & 7;
   }
+  // (K,N) B: this lane's row within a 16-k step and its 8-byte piece of the row.
+  const int tr_k = (kh << 3) + ((lane & 15) >> 2);
+  int tr_n[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) tr_n[i] = wn * 64 + i * 32 + (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
 
   for (int kt = 0; kt < nk; ++kt) {
     // Stage kt has landed once at most the two younger stages' loads are outstanding.
@@ -388,7 +406,21 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         af[i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
-        bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_off[i] + ((j ^ b_swz[i]) << 4));
+        if constexpr (!B_KN) {
+          bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_off[i] + ((j ^ b_swz[i]) << 4));
+        } else {
+          const int k = ks * 16 + tr_k;  // rows k and k + 4, each with its own swizzle
+          const int c0 = ((tr_n[i] >> 3) ^ ((k & 7) << 1)) << 4;
+          const int c1 = ((tr_n[i] >> 3) ^ (((k + 4) & 7) << 1)) << 4;
+          const int half = (tr_n[i] & 4) << 1;
+          const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + k * 256 + c0 + half));
+          const short4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + (k + 4) * 256 + c1 + half));
+          typedef short short8v __attribute__((ext_vector_type(8)));
+          const short8v both = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+          bfr[i] = __builtin_bit_cast(bf16x8, both);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i)
@@ -420,19 +452,20 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     }
 }
 
+template <bool B_KN>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                           const int* valid, hipStream_t s) {
   const int tiles_m = (M + NT_BM - 1) / NT_BM, tiles_n = (N + NT_BN - 1) / NT_BN;
   const size_t lds = (size_t)NT_STAGES * NT_STAGE_BYTES;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_kernel<B_KN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL(gemm_nt_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
+  hipLaunchKernelGGL(gemm_nt_kernel<B_KN>, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
                      valid, tiles_m, tiles_n, patched);
   IRON_LAUNCH_CHECK();
 }
@@ -479,8 +512,11 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   IRON_REQUIRE(b_col_maj || N % 8 == 0,
                "gemm: N (%d) must be a multiple of 8 when B is (K,N) (16-byte loads along N)", N);
   hipStream_t s = (hipStream_t)stream;
-  if (b_col_maj && !c_col_maj && valid_k == nullptr && K % BK == 0 && M >= 64 && N >= 64)
-    return launch_gemm_nt(A, B, C, M, N, K, valid, s);
+  if (!c_col_maj && valid_k == nullptr && K % BK == 0 && M >= 64 && N >= 64) {
+    if (b_col_maj) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s);
+    // (K,N) B is read in whole 128-column tiles straight into LDS: N must be whole tiles.
+    if (N % NT_BN == 0) return launch_gemm_nt<true>(A, B, C, M, N, K, valid, s);
+  }
   // 128x128 tiles fill the 256 CUs once at 2048x2048; narrower problems take 64-wide tiles.
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
   if (tiles128 >= 128 || (M >= 128 && N >= 128))
