@@ -48,6 +48,26 @@ int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16_t* y, int 
                          int batches, int repeat, const int* valid, int rows_per_wave,
                          int k_split, void* stream);
 
+/* One-row fusions of a decoder layer (no single counterpart in the reference: each replaces a run
+ * of its steps, iron/lm/blocks.py:627-648,697-699,723-733, and rounds where those steps round).
+ *   y = E(W @ N(x)):  N = RMSNorm(x, eps) * norm_w when norm_w is not NULL (else x itself);
+ *   epilogue 0: y = bf16(W N(x));  1: y = bf16(bf16(W N(x)) + residual);
+ *   2: y = bf16(bf16(silu(bf16(W N(x)))) * bf16(W2 N(x)))   (gate, up -> SiLU -> Mul).
+ * W, W2 (M,K); x, norm_w (K); residual, y (M).  K % 8 == 0. */
+int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const uint16_t* x,
+                         const uint16_t* norm_w, float eps, const uint16_t* residual, uint16_t* y,
+                         int M, int K, int epilogue, void* stream);
+
+/* Attention's first half for one token: n = RMSNorm(x) * norm_w; q = Wq n, k = Wk n, v = Wv n
+ * (each rounded to bf16); q and k rotated by the RoPE row `angles` (d bf16, cos/sin interleaved,
+ * two halves); q -> q_out (heads*d), k -> keys[*position], v -> values[*position], caches
+ * (cache_rows, kv_heads, d).  Replaces RMSNorm, 3 GEMV, 2 RoPE and 2 Copy steps
+ * (iron/lm/blocks.py:472-502,627-648). */
+int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* Wq,
+                         const uint16_t* Wk, const uint16_t* Wv, const uint16_t* angles,
+                         uint16_t* q_out, uint16_t* keys, uint16_t* values, int hidden, int heads,
+                         int kv_heads, int d, int cache_rows, const int* position, void* stream);
+
 /* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; w NULL = unweighted (one rounding).
  * x,y (rows, cols); w (cols).  cols % 8 == 0.  valid: rows computed.
  * Replaces norm.rms_norm_eps + eltwise.mul_sized: iron/operators/rms_norm.py:10,

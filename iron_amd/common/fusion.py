@@ -1,0 +1,175 @@
+"""Step fusion for a one-row (decode) version of a graph.
+
+The recorded steps stay what the reference records -- one operator per step, which is
+what ``Graph.reference`` and check mode run.  When a version is loaded for the GPU, runs
+of single-row steps that a decoder layer always records together are launched as one
+fused kernel each (``iron_amd/csrc/fused.hip``), which rounds wherever the separate steps
+round:
+
+  RMSNorm, GEMV q/k/v, RoPE q/k, Copy k/v -> cache      => iron_decode_qkv_bf16
+  RMSNorm, GEMV gate, GEMV up, SiLU, ElementwiseMul      => iron_gemv_fused_bf16 (epilogue 2)
+  GEMV, ElementwiseAdd (the residual)                    => iron_gemv_fused_bf16 (epilogue 1)
+  RMSNorm, GEMV (the head)                               => iron_gemv_fused_bf16 (epilogue 0)
+
+A run is fused only if every intermediate it hides is read by nothing else.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from collections import Counter
+from collections.abc import Callable
+from typing import Any
+
+
+@dataclasses.dataclass
+class Fused:
+    """One launch standing for ``steps`` consecutive recorded steps."""
+
+    kind: str
+    first: int
+    count: int
+    launch: Callable[[], None]
+
+
+class _Anything:
+    """Stands for a tensor while runs are only being matched (before the arena is loaded)."""
+
+    def reshape(self, *a):
+        return self
+
+    def __getitem__(self, key):
+        return self
+
+
+def match(recording) -> list[Fused]:
+    """The runs ``plan`` would fuse, without binding any tensor: for the arena plan, which must
+    keep every buffer a run touches alive across the whole run."""
+    return plan(recording, lambda h: _Anything(), lambda e: None)
+
+
+def _plain(h) -> bool:
+    return h.index is None and h.ids is None and not h.valid
+
+
+def _name(step) -> str:
+    return type(step.op).__name__
+
+
+def _same(a, b) -> bool:
+    """Two handles that are the same elements of the same buffer."""
+    return a.buffer is b.buffer and a.offset == b.offset and a.elements == b.elements and _plain(a) and _plain(b)
+
+
+def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) -> list[Fused]:
+    """The fused launches of ``recording``'s steps, by the first step each covers.
+
+    ``tensor(handle)`` is the device tensor behind a handle, ``word(expr)`` the device word
+    of a per-call expression.
+    """
+    from .. import kernels
+
+    steps = recording.steps
+    reads: Counter = Counter()
+    for s in steps:
+        for h in s.inputs.values():
+            reads[id(h.buffer)] += 1
+            if h.ids is not None:
+                reads[id(h.ids.buffer)] += 1
+    for h in recording.outputs:
+        reads[id(h.buffer)] += 1
+    for v in (recording.carry or {}).values():
+        if hasattr(v, "buffer"):
+            reads[id(v.buffer)] += 1
+
+    def once(h, n=1) -> bool:
+        return h.buffer.kind == "transient" and reads[id(h.buffer)] == n
+
+    def norm_row(s) -> bool:
+        return (_name(s) == "RMSNorm" and s.op.rows == 1 and s.op.weighted and not s.values
+                and all(_plain(h) for h in (*s.inputs.values(), *s.outputs.values())))
+
+    def gemv_row(s, x=None) -> bool:
+        ok = (_name(s) == "GEMV" and s.op.num_batches is None and not s.values
+              and all(_plain(h) for h in (*s.inputs.values(), *s.outputs.values())))
+        return ok and (x is None or _same(s.inputs["B"], x))
+
+    fused: list[Fused] = []
+    i = 0
+    while i < len(steps):
+        s = steps[i]
+        got = None
+        if norm_row(s):
+            n = s.outputs["y"]
+            rest = steps[i + 1 :]
+            # attention's first half
+            if (len(rest) >= 7 and all(gemv_row(g, n) for g in rest[:3]) and once(n, 3)
+                    and _name(rest[3]) == "RoPE" and _name(rest[4]) == "RoPE"
+                    and _name(rest[5]) == "Copy" and _name(rest[6]) == "Copy"):
+                gq, gk, gv, rq, rk, ck, cv = rest[:7]
+                q, k, v = (g.outputs["C"] for g in (gq, gk, gv))
+                d = rq.op.cols
+                kd, vd = ck.outputs["dst"], cv.outputs["dst"]
+                ok = (
+                    _same(rq.inputs["x"], q) and _same(rk.inputs["x"], k) and once(q) and once(k) and once(v)
+                    and rq.op.two_halves and rk.op.two_halves and rq.op.angle_rows == 1 and rk.op.angle_rows == 1
+                    and rk.op.cols == d and d in (64, 128) and not rq.values and not rk.values
+                    and rq.inputs["angles"].buffer is rk.inputs["angles"].buffer and _plain(rq.inputs["angles"])
+                    and _same(ck.inputs["src"], rk.outputs["y"]) and once(rk.outputs["y"])
+                    and _same(cv.inputs["src"], v)
+                    and kd.index is not None and vd.index is not None and kd.index == vd.index
+                    and kd.ids is None and vd.ids is None and not kd.valid and not vd.valid
+                    and kd.offset == 0 and vd.offset == 0
+                    and kd.index_stride == k.elements and vd.index_stride == v.elements
+                    and k.elements == v.elements and k.elements % d == 0 and q.elements % d == 0
+                )
+                if ok:
+                    args = dict(
+                        x=tensor(s.inputs["x"]).reshape(-1), norm_w=tensor(s.inputs["weight"]).reshape(-1),
+                        Wq=tensor(gq.inputs["A"]), Wk=tensor(gk.inputs["A"]), Wv=tensor(gv.inputs["A"]),
+                        angles=tensor(rq.inputs["angles"]).reshape(-1), q_out=tensor(rq.outputs["y"]).reshape(-1),
+                        keys=tensor(kd)[: kd.index_rows * kd.index_stride],
+                        values=tensor(vd)[: vd.index_rows * vd.index_stride],
+                    )
+                    kw = dict(eps=float(s.op.epsilon), hidden=s.op.tile_size, heads=q.elements // d,
+                              kv_heads=k.elements // d, d=d, cache_rows=kd.index_rows, position=word(kd.index))
+                    got = Fused("decode_qkv", i, 8, lambda a=args, kw=kw: kernels.decode_qkv(**a, **kw))
+            # the gated MLP's first half
+            if (got is None and len(rest) >= 4 and gemv_row(rest[0], n) and gemv_row(rest[1], n) and once(n, 2)
+                    and _name(rest[2]) == "SiLU" and _name(rest[3]) == "ElementwiseMul"):
+                gg, gu, si, mu = rest[:4]
+                g, u = gg.outputs["C"], gu.outputs["C"]
+                ok = (_same(si.inputs["x"], g) and once(g) and once(u) and once(si.outputs["y"])
+                      and not si.values and not mu.values
+                      and _same(mu.inputs["a"], si.outputs["y"]) and _same(mu.inputs["b"], u)
+                      and gg.op.M == gu.op.M and gg.op.K == gu.op.K and _plain(mu.outputs["y"]))
+                if ok:
+                    args = dict(W=tensor(gg.inputs["A"]), W2=tensor(gu.inputs["A"]),
+                                x=tensor(s.inputs["x"]).reshape(-1), norm_w=tensor(s.inputs["weight"]).reshape(-1),
+                                y=tensor(mu.outputs["y"]).reshape(-1))
+                    kw = dict(M=gg.op.M, K=gg.op.K, eps=float(s.op.epsilon), epilogue=2)
+                    got = Fused("norm_gate_up_silu_mul", i, 5, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+            # the head: norm, then one projection
+            if got is None and rest and gemv_row(rest[0], n) and once(n, 1):
+                g0 = rest[0]
+                args = dict(W=tensor(g0.inputs["A"]), x=tensor(s.inputs["x"]).reshape(-1),
+                            norm_w=tensor(s.inputs["weight"]).reshape(-1), y=tensor(g0.outputs["C"]).reshape(-1))
+                kw = dict(M=g0.op.M, K=g0.op.K, eps=float(s.op.epsilon), epilogue=0)
+                got = Fused("norm_gemv", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+        elif gemv_row(s) and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseAdd":
+            ad = steps[i + 1]
+            c = s.outputs["C"]
+            a, b = ad.inputs["a"], ad.inputs["b"]
+            other = a if _same(b, c) else (b if _same(a, c) else None)
+            if other is not None and once(c) and _plain(other) and not ad.values and _plain(ad.outputs["y"]) \
+                    and other.elements == c.elements:
+                args = dict(W=tensor(s.inputs["A"]), x=tensor(s.inputs["B"]).reshape(-1),
+                            residual=tensor(other).reshape(-1), y=tensor(ad.outputs["y"]).reshape(-1))
+                kw = dict(M=s.op.M, K=s.op.K, epilogue=1)
+                got = Fused("gemv_add", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+        if got is not None:
+            fused.append(got)
+            i += got.count
+        else:
+            i += 1
+    return fused

@@ -710,7 +710,7 @@ class Graph:
                          recorder.residents, recorder.limits)
 
     def compile(self, *, arena: "ScratchArena | None" = None, capture: bool | None = None, check: bool = False,
-                full_elf: bool | None = None, **shapes) -> "CompiledGraph":
+                full_elf: bool | None = None, fuse: bool = True, **shapes) -> "CompiledGraph":
         """Record a version and plan it into this graph's arena.
 
         ``capture``: replay the version as one HIP graph (default: when it takes no
@@ -721,7 +721,7 @@ class Graph:
             capture = full_elf
         recording = self.record(**shapes)
         arena = arena if arena is not None else self.arena
-        version = CompiledGraph(self, recording, arena, capture=capture, check=check)
+        version = CompiledGraph(self, recording, arena, capture=capture, check=check, fuse=fuse)
         self._versions.append(version)
         return version
 
@@ -796,15 +796,25 @@ class Recording:
                                  f"({lim.expr.name}) end outside {lim.rows}")
         return full
 
-    def transients(self) -> list[tuple[Buffer, int, int]]:
-        """Each transient buffer with the first and last step that touches it."""
+    def transients(self, runs=()) -> list[tuple[Buffer, int, int]]:
+        """Each transient buffer with the first and last step that touches it.
+
+        ``runs``: ``(first, last)`` step ranges launched as one kernel each; a buffer touched
+        inside a run is live across the whole run (its last step's output is written while its
+        first step's input is still being read).
+        """
+        run_of = {}
+        for first, last in runs:
+            for i in range(first, last + 1):
+                run_of[i] = (first, last)
         spans: dict[int, list] = {}
         for i, step in enumerate(self.steps):
+            lo, hi = run_of.get(i, (i, i))
             for h in (*step.inputs.values(), *step.outputs.values()):
                 for b in [h.buffer] + ([h.ids.buffer] if h.ids is not None else []):
                     if b.kind == "transient":
-                        span = spans.setdefault(id(b), [b, i, i])
-                        span[2] = i
+                        span = spans.setdefault(id(b), [b, lo, hi])
+                        span[1], span[2] = min(span[1], lo), max(span[2], hi)
         for h in self.outputs:  # an output lives to the end
             if id(h.buffer) in spans:
                 spans[id(h.buffer)][2] = len(self.steps)
@@ -1024,9 +1034,13 @@ class DeviceOutput:
 class CompiledGraph:
     """One version of a graph, placed in its arena; call it with tensors and per-call values."""
 
-    def __init__(self, graph: Graph, recording: Recording, arena: ScratchArena, *, capture=None, check=False):
+    def __init__(self, graph: Graph, recording: Recording, arena: ScratchArena, *, capture=None, check=False,
+                 fuse=True):
         self.graph, self.recording, self.arena = graph, recording, arena
         self.check = check
+        # Launch the runs of one-row steps a decoder layer records together as fused kernels.
+        self.fuse = fuse and not check
+        self._fused: dict[int, Any] = {}
         self.capture = (not recording.inputs) if capture is None else bool(capture)
         if check:
             self.capture = False
@@ -1038,7 +1052,12 @@ class CompiledGraph:
         # Inputs are transients that live from the start.
         for h in recording.inputs:
             self.transient_offsets[id(h.buffer)] = pool.place(LiveRange(h.buffer.nbytes, -1, len(recording.steps)))
-        for b, first, last in recording.transients():
+        runs = []
+        if self.fuse:
+            from . import fusion
+
+            runs = [(f.first, f.first + f.count - 1) for f in fusion.match(recording)]
+        for b, first, last in recording.transients(runs):
             self.transient_offsets[id(b)] = pool.place(LiveRange(b.nbytes, first, last))
         # The per-call words: one slot per declared value, then one per derived expression.
         self.slots: dict[str, int] = {v.name: i for i, v in enumerate(recording.values)}
@@ -1126,6 +1145,11 @@ class CompiledGraph:
             table = torch.tensor(rows, dtype=torch.int32).reshape(-1)
             self.expr_table[: table.numel()].copy_(table)
         self._launches = [self._bind(step) for step in self.recording.steps]
+        self._fused = {}
+        if self.fuse:
+            from . import fusion
+
+            self._fused = {f.first: f for f in fusion.plan(self.recording, self._tensor, self.word)}
         self.input_tensors = [self._tensor(h) for h in self.recording.inputs]
         self.output_tensors = [self._tensor(h) for h in self.recording.outputs]
         self._loaded_generation = self.arena.generation
@@ -1151,8 +1175,21 @@ class CompiledGraph:
         return built.launch, tensors, words
 
     def _run_steps(self) -> None:
-        for launch, tensors, words in self._launches:
+        i, n = 0, len(self._launches)
+        while i < n:
+            fused = self._fused.get(i)
+            if fused is not None:
+                fused.launch()
+                i += fused.count
+                continue
+            launch, tensors, words = self._launches[i]
             launch(tensors, words)
+            i += 1
+
+    @property
+    def launches_per_call(self) -> int:
+        """Kernel-launching units a call runs (recorded steps less those fused away)."""
+        return len(self._launches) - sum(f.count - 1 for f in self._fused.values())
 
     def _derive(self) -> None:
         from .. import kernels

@@ -169,21 +169,39 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
   }
 }
 
+// One block per head merges the splits: thread s < nsplit turns split s's (m, l) into a weight
+// in LDS, then thread dd sums column dd over the splits with independent (unrolled) loads.
 template <int D>
 __global__ void mha_decode_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ O,
                                         int nsplit) {
-  const int head = blockIdx.x, dd = threadIdx.x;
+  __shared__ float wgt[kMaxSplits];
+  __shared__ float red[2][4];
+  const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const float* p = part + (size_t)head * nsplit * (D + 2);
-  float mx = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, p[s * (D + 2)]);
-  const float ref = (mx == -INFINITY) ? 0.f : mx;
-  float lt = 0.f, at = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float e = exp2f(p[s * (D + 2)] - ref);
-    lt += p[s * (D + 2) + 1] * e;
-    at += p[s * (D + 2) + 2 + dd] * e;
+  float m = -INFINITY, l = 0.f;
+  if (t < nsplit) {
+    m = p[t * (D + 2)];
+    l = p[t * (D + 2) + 1];
   }
-  O[(size_t)head * D + dd] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
+  float mx = wave_max(m);
+  if (lane == 0) red[0][wave] = mx;
+  __syncthreads();
+  mx = -INFINITY;
+  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) mx = fmaxf(mx, red[0][w]);
+  const float ref = (mx == -INFINITY) ? 0.f : mx;
+  const float e = exp2f(m - ref);  // 0 for the lanes past nsplit (m = -inf)
+  if (t < nsplit) wgt[t] = e;
+  float ls = wave_sum(l * e);
+  if (lane == 0) red[1][wave] = ls;
+  __syncthreads();
+  float lt = 0.f;
+  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) lt += red[1][w];
+  if (t < D) {
+    float at = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < nsplit; ++s) at = fmaf(p[s * (D + 2) + 2 + t], wgt[s], at);
+    O[(size_t)head * D + t] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
+  }
 }
 
 template <int D, int G>
@@ -192,8 +210,8 @@ static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf1
                           long head_stride, const int* kv_valid, int nsplit, hipStream_t s) {
   hipLaunchKernelGGL((mha_decode_kernel<D, G>), dim3(nsplit, kv_heads), dim3(256), 0, s, Q, K, V,
                      part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid);
-  hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D), 0, s, part, O,
-                     nsplit);
+  hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D > kMaxSplits ? D : kMaxSplits), 0, s,
+                     part, O, nsplit);
 }
 
 }  // namespace iron

@@ -69,6 +69,44 @@ def gemv(W, x, y, *, M, K, batches=1, repeat=1, valid=None, rows_per_wave=0, k_s
     )
 
 
+def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, epilogue=0):
+    """One-row fusion: ``[RMSNorm ->] GEMV [-> + residual | gate/up -> SiLU -> Mul]``."""
+    _numel(_dev(W, "W"), M * K, "W")
+    _numel(_dev(x, "x"), K, "x")
+    _numel(_dev(y, "y"), M, "y")
+    if W2 is not None:
+        _numel(_dev(W2, "W2"), M * K, "W2")
+    if norm_w is not None:
+        _numel(_dev(norm_w, "norm_w"), K, "norm_w")
+    if residual is not None:
+        _numel(_dev(residual, "residual"), M, "residual")
+    check(
+        lib().iron_gemv_fused_bf16(ptr(W), ptr(W2), ptr(x), ptr(norm_w), float(eps), ptr(residual), ptr(y),
+                                   M, K, int(epilogue), current_stream()),
+        "iron_gemv_fused_bf16",
+    )
+
+
+def decode_qkv(x, norm_w, Wq, Wk, Wv, angles, q_out, keys, values, *, eps, hidden, heads, kv_heads, d,
+               cache_rows, position):
+    """Attention's first half for one token: norm, q/k/v projections, RoPE, cache writes."""
+    _numel(_dev(x, "x"), hidden, "x")
+    _numel(_dev(norm_w, "norm_w"), hidden, "norm_w")
+    _numel(_dev(Wq, "Wq"), heads * d * hidden, "Wq")
+    _numel(_dev(Wk, "Wk"), kv_heads * d * hidden, "Wk")
+    _numel(_dev(Wv, "Wv"), kv_heads * d * hidden, "Wv")
+    _numel(_dev(angles, "angles"), d, "angles")
+    _numel(_dev(q_out, "q_out"), heads * d, "q_out")
+    _numel(_dev(keys, "keys"), cache_rows * kv_heads * d, "keys")
+    _numel(_dev(values, "values"), cache_rows * kv_heads * d, "values")
+    check(
+        lib().iron_decode_qkv_bf16(ptr(x), ptr(norm_w), float(eps), ptr(Wq), ptr(Wk), ptr(Wv), ptr(angles),
+                                   ptr(q_out), ptr(keys), ptr(values), hidden, heads, kv_heads, d, cache_rows,
+                                   ptr(_word(position, "position")), current_stream()),
+        "iron_decode_qkv_bf16",
+    )
+
+
 def rmsnorm(x, w, y, *, rows, cols, eps, valid=None):
     _numel(_dev(x, "x"), rows * cols, "x")
     _numel(_dev(y, "y"), rows * cols, "y")

@@ -132,12 +132,15 @@ class CausalLM(iron.Graph):
         """The input shapes of each version: the decode step's (none), then the prompt chunk's ids."""
         return [{}, dict(ids=((self.config.prefill_chunk,), np.int32))]
 
-    def load_versions(self, *, capture: bool = True, check: bool = False) -> None:
-        """Compile the decode step and the prompt chunk into one arena and load them."""
+    def load_versions(self, *, capture: bool = True, check: bool = False, fuse: bool = True) -> None:
+        """Compile the decode step and the prompt chunk into one arena and load them.
+
+        ``fuse``: launch the decode step's runs of one-row steps as fused kernels.
+        """
         decode_shapes, prompt_shapes = self.shapes()
         try:
-            decode = self.compile(capture=capture, check=check, **decode_shapes)
-            prompt = self.compile(capture=False, check=check, **prompt_shapes)
+            decode = self.compile(capture=capture, check=check, fuse=fuse, **decode_shapes)
+            prompt = self.compile(capture=False, check=check, fuse=fuse, **prompt_shapes)
             decode.load()
             prompt.load()
         except Exception:

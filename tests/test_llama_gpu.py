@@ -134,3 +134,80 @@ def test_two_layers_at_llama_1b_width_match_the_host_reference(cuda):
     tokens = np.append(tokens, want.argmax())
     assert_close(gpu.logits(tokens), cpu.logits(tokens), "decode")
     gpu.release()
+
+
+def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
+    """The fused launches compute what the recorded steps compute: same greedy tokens, logits
+    within bf16 rounding, and far fewer launches per decode step."""
+    fused, plain = Llama(SCALED, weights()), Llama(SCALED, weights())
+    fused.load_versions(fuse=True)
+    plain.load_versions(fuse=False)
+    steps = len(fused.decode_step.recording.steps)
+    assert plain.decode_step.launches_per_call == steps
+    # per layer 18 steps become 5 launches (qkv, attention, o+add, gate/up, down+add); the head 2 -> 1.
+    assert fused.decode_step.launches_per_call == 2 + 5 * SCALED.num_hidden_layers + 2
+    prompt = np.random.default_rng(7).integers(0, SCALED.vocab_size, 8)
+    a, b = fused.logits(prompt), plain.logits(prompt)
+    tokens = prompt
+    for step in range(6):
+        tokens = np.append(tokens, golden.logits(tokens).argmax())
+        a, b = fused.logits(tokens), plain.logits(tokens)
+        assert np.abs(a - b).max() <= 0.02 * np.abs(b).max(), step
+        assert_close(a, golden.logits(tokens), f"fused step {step}")
+    prompt = np.random.default_rng(8).integers(0, SCALED.vocab_size, 40)
+    assert fused.generate(prompt, 24) == plain.generate(prompt, 24)
+    fused.release()
+    plain.release()
+
+
+def test_fused_kernels_against_the_oracle_at_llama_1b_width(cuda):
+    """Each fused kernel through the C ABI against the oracle's steps composed on the host."""
+    import torch
+
+    from iron_amd import kernels as K
+    from iron_amd.bf16 import from_torch, round_bf16, to_torch
+    from oracle import ops
+
+    rng = np.random.default_rng(21)
+    E, F, H, G, D, L, pos = 2048, 8192, 32, 8, 64, 64, 37
+
+    def bf(*shape, scale=1.0):
+        return round_bf16(rng.standard_normal(shape, dtype=np.float32) * np.float32(scale))
+
+    def dev(a):
+        return to_torch(a).to(cuda)
+
+    def close(got, want, atol=2e-2):
+        got = (from_torch(got) if isinstance(got, torch.Tensor) else got).reshape(want.shape)
+        assert np.all(np.abs(got - want) <= atol + 1e-2 * np.abs(want)), np.abs(got - want).max()
+
+    x, g = bf(E), round_bf16(rng.uniform(0.9, 1.1, E))
+    n = ops.rms_norm(x[None], g, epsilon=1e-5)[0]
+    # attention's first half
+    Wq, Wk, Wv = bf(H * D, E, scale=0.02), bf(G * D, E, scale=0.02), bf(G * D, E, scale=0.02)
+    table = round_bf16(ops.rope_angles(D, L))
+    keys, values = dev(np.zeros((L, G, D), np.float32)), dev(np.zeros((L, G, D), np.float32))
+    q_out = torch.empty(H * D, dtype=torch.bfloat16, device=cuda)
+    K.decode_qkv(dev(x), dev(g), dev(Wq), dev(Wk), dev(Wv), dev(table[pos]), q_out, keys, values, eps=1e-5,
+                 hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
+                 position=torch.tensor([pos], dtype=torch.int32, device=cuda))
+    close(q_out, ops.rope(ops.gemv(Wq, n).reshape(H, D), table[pos : pos + 1]).reshape(-1))
+    kc, vc = from_torch(keys), from_torch(values)
+    close(kc[pos], ops.rope(ops.gemv(Wk, n).reshape(G, D), table[pos : pos + 1]))
+    close(vc[pos], ops.gemv(Wv, n).reshape(G, D))
+    assert not kc[:pos].any() and not kc[pos + 1 :].any() and not vc[:pos].any() and not vc[pos + 1 :].any()
+    # the gated MLP's first half, and a projection with its residual
+    Wg, Wu, Wd = bf(F, E, scale=0.02), bf(F, E, scale=0.02), bf(E, F, scale=0.02)
+    m = torch.empty(F, dtype=torch.bfloat16, device=cuda)
+    K.gemv_fused(dev(Wg), dev(x), m, M=F, K=E, W2=dev(Wu), norm_w=dev(g), eps=1e-5, epilogue=2)
+    want_m = ops.mul(ops.silu(ops.gemv(Wg, n)), ops.gemv(Wu, n))
+    close(m, want_m)
+    y = torch.empty(E, dtype=torch.bfloat16, device=cuda)
+    K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, residual=dev(x), epilogue=1)
+    close(y, ops.add(x, ops.gemv(Wd, want_m)))
+    # the head: norm then projection
+    for rows in (4096, 10000, 128256):  # one, two and four rows a wave
+        Wh = bf(rows, E, scale=0.02)
+        lg = torch.empty(rows, dtype=torch.bfloat16, device=cuda)
+        K.gemv_fused(dev(Wh), dev(x), lg, M=rows, K=E, norm_w=dev(g), eps=1e-5, epilogue=0)
+        close(lg, ops.gemv(Wh, n))
