@@ -13,101 +13,135 @@ namespace iron {
 
 __device__ __forceinline__ float silu_ref(float v) { return v / (1.0f + __expf(-v)); }
 
-// 1 / sqrt(mean(x^2) + eps) of a K-vector, computed by every wave for itself (x is L2-resident).
-__device__ __forceinline__ float wave_inv_rms(const bf16_t* __restrict__ x, int K, float eps, int lane) {
-  const uint4* xv = reinterpret_cast<const uint4*>(x);
-  float ss = 0.f;
-  for (int c = lane; c < (K >> 3); c += 64) {
-    float f[8];
-    unpack8(xv[c], f);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
-  }
-  ss = wave_sum(ss);
-  return 1.0f / sqrtf(ss / (float)K + eps);
+// All fused kernels share one shape: a block of 4 waves owns a few rows and its 256 threads
+// split K in 16-byte chunks (thread t takes chunks t, t+256, ...), so the weight loads of a row
+// are one contiguous stream per block, every lane has all its loads in flight before it needs
+// any of them, and the activation chunk a thread normalises is the one it multiplies by.
+
+// Block-wide sum through LDS (one barrier); every thread gets the total.
+__device__ __forceinline__ float block_sum(float v, float* scratch4) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) scratch4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return scratch4[0] + scratch4[1] + scratch4[2] + scratch4[3];
 }
 
-// The 8 activations of chunk c as the GEMV sees them: x itself, or RMSNorm(x) * w rounded as
-// the RMSNorm step rounds (the normed row to bf16, then the product to bf16).
-template <bool NORM>
-__device__ __forceinline__ void load_x(const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw,
-                                       float inv, int c, float (&xf)[8]) {
-  unpack8(reinterpret_cast<const uint4*>(x)[c], xf);
-  if (NORM) {
-    float g[8];
-    unpack8(reinterpret_cast<const uint4*>(nw)[c], g);
+// This thread's CH chunks of the activation as the GEMV sees them: x itself, or
+// RMSNorm(x) * w rounded as the RMSNorm step rounds (the normed row to bf16, then the
+// product to bf16).  In two halves so the caller can put its weight loads between them:
+// memory returns in order, so the small activation loads go out first and are not held up
+// behind the long weight stream.
+template <int CH, bool NORM>
+struct Activation {
+  uint4 xv[CH], gv[CH];
+  __device__ __forceinline__ void issue(const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw, int K) {
+    const int chunks = K >> 3;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) xf[j] = round_bf16(round_bf16(xf[j] * inv) * g[j]);
+    for (int i = 0; i < CH; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      xv[i] = c < chunks ? reinterpret_cast<const uint4*>(x)[c] : make_uint4(0, 0, 0, 0);
+      if (NORM) gv[i] = c < chunks ? reinterpret_cast<const uint4*>(nw)[c] : make_uint4(0, 0, 0, 0);
+    }
   }
+  // With NORM the block sums the squares together (one barrier).
+  __device__ __forceinline__ void finish(float eps, int K, float* scratch4, float (&xf)[CH][8]) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      unpack8(xv[i], xf[i]);
+      if (NORM) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = fmaf(xf[i][j], xf[i][j], ss);
+      }
+    }
+    if (NORM) {
+      const float inv = 1.0f / sqrtf(block_sum(ss, scratch4) / (float)K + eps);
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        float g[8];
+        unpack8(gv[i], g);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xf[i][j] = round_bf16(round_bf16(xf[i][j] * inv) * g[j]);
+      }
+    }
+  }
+};
+
+template <int CH>
+__device__ __forceinline__ void load_row(const bf16_t* __restrict__ row, int K, uint4 (&w)[CH]) {
+  const int chunks = K >> 3;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    w[i] = c < chunks ? load_stream(reinterpret_cast<const uint4*>(row) + c) : make_uint4(0, 0, 0, 0);
+  }
+}
+
+template <int CH>
+__device__ __forceinline__ float dot_row(const uint4 (&w)[CH], const float (&xf)[CH][8]) {
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    float wf[8];
+    unpack8(w[i], wf);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc = fmaf(wf[j], xf[i][j], acc);
+  }
+  return acc;
 }
 
 enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2 };
 
-// One wave per RPW rows, full K (so the rows' sums need no cross-wave merge).
-template <int RPW, bool NORM, int EPI>
+// y = E(W @ N(x)) for RPW rows a block; K <= CH * 2048.
+template <int RPW, int CH, bool NORM, int EPI>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restrict__ W,
                                                          const bf16_t* __restrict__ W2,
                                                          const bf16_t* __restrict__ x,
                                                          const bf16_t* __restrict__ nw, float eps,
                                                          const bf16_t* __restrict__ res,
                                                          bf16_t* __restrict__ y, int M, int K) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int row0 = (blockIdx.x * 4 + wave) * RPW;
-  if (row0 >= M) return;
-  const float inv = NORM ? wave_inv_rms(x, K, eps, lane) : 1.f;
   constexpr int MATS = EPI == EPI_SILU_MUL ? 2 : 1;
-  float acc[MATS][RPW];
-  const uint4* wrow[MATS][RPW];
+  __shared__ float scratch4[4];
+  __shared__ float part[4][MATS][RPW];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row0 = blockIdx.x * RPW;
+  Activation<CH, NORM> act;
+  act.issue(x, nw, K);
+  uint4 w[MATS][RPW][CH];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
     const int row = min(row0 + r, M - 1);
-    acc[0][r] = 0.f;
-    wrow[0][r] = reinterpret_cast<const uint4*>(W + (size_t)row * K);
-    if (MATS == 2) {
-      acc[MATS - 1][r] = 0.f;
-      wrow[MATS - 1][r] = reinterpret_cast<const uint4*>(W2 + (size_t)row * K);
-    }
+    load_row<CH>(W + (size_t)row * K, K, w[0][r]);
+    if (MATS == 2) load_row<CH>(W2 + (size_t)row * K, K, w[MATS - 1][r]);
   }
-  const int chunks = K >> 3;
-#pragma unroll 4
-  for (int c = lane; c < chunks; c += 64) {
-    uint4 wv[MATS][RPW];
-#pragma unroll
-    for (int m = 0; m < MATS; ++m)
-#pragma unroll
-      for (int r = 0; r < RPW; ++r) wv[m][r] = load_stream(wrow[m][r] + c);
-    float xf[8];
-    load_x<NORM>(x, nw, inv, c, xf);
-#pragma unroll
-    for (int m = 0; m < MATS; ++m)
-#pragma unroll
-      for (int r = 0; r < RPW; ++r) {
-        float wf[8];
-        unpack8(wv[m][r], wf);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[m][r] = fmaf(wf[i], xf[i], acc[m][r]);
-      }
-  }
+  float xf[CH][8];
+  act.finish(eps, K, scratch4, xf);
 #pragma unroll
   for (int m = 0; m < MATS; ++m)
 #pragma unroll
-    for (int r = 0; r < RPW; ++r) acc[m][r] = wave_sum(acc[m][r]);
-  if (lane == 0) {
-#pragma unroll
     for (int r = 0; r < RPW; ++r) {
-      const int row = row0 + r;
-      if (row >= M) break;
-      float v = round_bf16(acc[0][r]);  // the GEMV step's own rounding
+      const float a = wave_sum(dot_row<CH>(w[m][r], xf));
+      if (lane == 0) part[wave][m][r] = a;
+    }
+  __syncthreads();
+  if (threadIdx.x < RPW) {
+    const int r = threadIdx.x, row = row0 + r;
+    if (row < M) {
+      float v = round_bf16(part[0][0][r] + part[1][0][r] + part[2][0][r] + part[3][0][r]);  // the GEMV's own rounding
       if (EPI == EPI_ADD) v = v + bf16_to_f32(res[row]);
-      if (EPI == EPI_SILU_MUL) v = round_bf16(silu_ref(v)) * round_bf16(acc[MATS - 1][r]);
+      if (EPI == EPI_SILU_MUL) {
+        const float u = round_bf16(part[0][MATS - 1][r] + part[1][MATS - 1][r] + part[2][MATS - 1][r] +
+                                   part[3][MATS - 1][r]);
+        v = round_bf16(silu_ref(v)) * u;
+      }
       y[row] = f32_to_bf16(v);
     }
   }
 }
 
-// Attention's first half for one token.  A wave takes a PAIR of projection rows: for q and k
+// Attention's first half for one token.  A block takes a PAIR of projection rows: for q and k
 // the rows (h, j) and (h, j + D/2) that RoPE rotates together, for v two adjacent rows.
-template <int D>
+template <int D, int CH>
 __global__ __launch_bounds__(256) void decode_qkv_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw, float eps,
     const bf16_t* __restrict__ Wq, const bf16_t* __restrict__ Wk, const bf16_t* __restrict__ Wv,
@@ -115,12 +149,11 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
     bf16_t* __restrict__ values, int K, int heads, int kv_heads, int cache_rows,
     const int* __restrict__ position) {
   constexpr int HALF = D / 2;
+  __shared__ float scratch4[4];
+  __shared__ float part[4][2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int pair = blockIdx.x * 4 + wave;
+  const int pair = blockIdx.x;
   const int q_pairs = heads * HALF, k_pairs = kv_heads * HALF;
-  if (pair >= q_pairs + 2 * k_pairs) return;
-  const int pos = *position;
-  const float inv = wave_inv_rms(x, K, eps, lane);
 
   const bf16_t* Wm;
   int r0, r1, j = 0, kind;  // kind 0 q, 1 k, 2 v
@@ -128,23 +161,19 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   else if (pair < q_pairs + k_pairs) { kind = 1; Wm = Wk; const int p = pair - q_pairs; const int h = p / HALF; j = p % HALF; r0 = h * D + j; r1 = r0 + HALF; }
   else { kind = 2; Wm = Wv; const int p = pair - q_pairs - k_pairs; r0 = 2 * p; r1 = r0 + 1; }
 
-  const uint4* w0 = reinterpret_cast<const uint4*>(Wm + (size_t)r0 * K);
-  const uint4* w1 = reinterpret_cast<const uint4*>(Wm + (size_t)r1 * K);
-  float a0 = 0.f, a1 = 0.f;
-#pragma unroll 4
-  for (int c = lane; c < (K >> 3); c += 64) {
-    const uint4 v0 = load_stream(w0 + c), v1 = load_stream(w1 + c);
-    float xf[8], f0[8], f1[8];
-    load_x<true>(x, nw, inv, c, xf);
-    unpack8(v0, f0);
-    unpack8(v1, f1);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { a0 = fmaf(f0[i], xf[i], a0); a1 = fmaf(f1[i], xf[i], a1); }
-  }
-  a0 = wave_sum(a0);
-  a1 = wave_sum(a1);
-  if (lane != 0) return;
-  float y0 = round_bf16(a0), y1 = round_bf16(a1);  // the projections' own rounding
+  Activation<CH, true> act;
+  act.issue(x, nw, K);
+  uint4 w0[CH], w1[CH];
+  load_row<CH>(Wm + (size_t)r0 * K, K, w0);
+  load_row<CH>(Wm + (size_t)r1 * K, K, w1);
+  float xf[CH][8];
+  act.finish(eps, K, scratch4, xf);
+  const float a0 = wave_sum(dot_row<CH>(w0, xf)), a1 = wave_sum(dot_row<CH>(w1, xf));
+  if (lane == 0) { part[wave][0] = a0; part[wave][1] = a1; }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  float y0 = round_bf16(part[0][0] + part[1][0] + part[2][0] + part[3][0]);  // the projections' own rounding
+  float y1 = round_bf16(part[0][1] + part[1][1] + part[2][1] + part[3][1]);
   if (kind != 2) {
     const float c = bf16_to_f32(angles[2 * j]), s = bf16_to_f32(angles[2 * j + 1]);
     const float t0 = y0 * c - y1 * s, t1 = y1 * c + y0 * s;
@@ -153,10 +182,13 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   if (kind == 0) {
     q_out[r0] = f32_to_bf16(y0);
     q_out[r1] = f32_to_bf16(y1);
-  } else if (pos >= 0 && pos < cache_rows) {
-    bf16_t* dst = (kind == 1 ? keys : values) + (size_t)pos * kv_heads * D;
-    dst[r0] = f32_to_bf16(y0);
-    dst[r1] = f32_to_bf16(y1);
+  } else {
+    const int pos = *position;
+    if (pos >= 0 && pos < cache_rows) {
+      bf16_t* dst = (kind == 1 ? keys : values) + (size_t)pos * kv_heads * D;
+      dst[r0] = f32_to_bf16(y0);
+      dst[r1] = f32_to_bf16(y1);
+    }
   }
 }
 
@@ -176,20 +208,23 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
                "gemv_fused: operands must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   const bool norm = norm_w != nullptr;
-  // Rows a wave takes: enough waves to fill the chip, several loads in flight a lane.
-  const int rpw = (epilogue == EPI_SILU_MUL) ? 1 : (M >= 65536 ? 4 : (M >= 8192 ? 2 : 1));
-  const int blocks = (M + 4 * rpw - 1) / (4 * rpw);
-#define IRON_FUSED(R, NRM, E)                                                                      \
-  if (rpw == R && norm == NRM && epilogue == E) {                                                  \
-    hipLaunchKernelGGL((gemv_fused_kernel<R, NRM, E>), dim3(blocks), dim3(256), 0, s, W, W2, x,    \
+  IRON_REQUIRE(K <= 8 * 2048, "gemv_fused: K (%d) exceeds %d", K, 8 * 2048);
+  const int ch = K <= 2048 ? 1 : (K <= 4096 ? 2 : (K <= 8192 ? 4 : 8));
+  // Rows a block takes: two where the matrix is tall and a row is short, else one.
+  const int rpw = (epilogue == EPI_SILU_MUL) ? (ch == 1 ? 2 : 1) : (ch == 1 && M > 2048 ? (M >= 65536 ? 4 : 2) : 1);
+  const int blocks = (M + rpw - 1) / rpw;
+#define IRON_FUSED(R, C, NRM, E)                                                                   \
+  if (rpw == R && ch == C && norm == NRM && epilogue == E) {                                       \
+    hipLaunchKernelGGL((gemv_fused_kernel<R, C, NRM, E>), dim3(blocks), dim3(256), 0, s, W, W2, x, \
                        norm_w, eps, residual, y, M, K);                                            \
     IRON_LAUNCH_CHECK();                                                                           \
   }
-  IRON_FUSED(1, false, 0) IRON_FUSED(2, false, 0) IRON_FUSED(4, false, 0)
-  IRON_FUSED(1, true, 0) IRON_FUSED(2, true, 0) IRON_FUSED(4, true, 0)
-  IRON_FUSED(1, false, 1) IRON_FUSED(2, false, 1) IRON_FUSED(4, false, 1)
-  IRON_FUSED(1, true, 1) IRON_FUSED(2, true, 1) IRON_FUSED(4, true, 1)
-  IRON_FUSED(1, false, 2) IRON_FUSED(1, true, 2)
+#define IRON_FUSED_NE(R, C)                                                                        \
+  IRON_FUSED(R, C, false, 0) IRON_FUSED(R, C, true, 0) IRON_FUSED(R, C, false, 1) IRON_FUSED(R, C, true, 1)
+  IRON_FUSED_NE(1, 1) IRON_FUSED_NE(2, 1) IRON_FUSED_NE(4, 1) IRON_FUSED_NE(1, 2) IRON_FUSED_NE(1, 4) IRON_FUSED_NE(1, 8)
+  IRON_FUSED(2, 1, false, 2) IRON_FUSED(2, 1, true, 2) IRON_FUSED(1, 2, false, 2) IRON_FUSED(1, 2, true, 2)
+  IRON_FUSED(1, 4, false, 2) IRON_FUSED(1, 4, true, 2) IRON_FUSED(1, 8, false, 2) IRON_FUSED(1, 8, true, 2)
+#undef IRON_FUSED_NE
 #undef IRON_FUSED
   IRON_REQUIRE(false, "gemv_fused: no kernel for this combination");
 }
@@ -206,14 +241,15 @@ extern "C" int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, f
   IRON_REQUIRE(heads > 0 && kv_heads > 0 && cache_rows > 0, "decode_qkv: heads, kv_heads, cache_rows must be positive");
   IRON_REQUIRE((((uintptr_t)x | (uintptr_t)norm_w | (uintptr_t)Wq | (uintptr_t)Wk | (uintptr_t)Wv) & 15) == 0,
                "decode_qkv: operands must be 16-byte aligned");
+  IRON_REQUIRE(hidden <= 8192, "decode_qkv: hidden (%d) exceeds 8192", hidden);
   const int pairs = heads * (d / 2) + 2 * kv_heads * (d / 2);
-  const int blocks = (pairs + 3) / 4;
+  const int ch = hidden <= 2048 ? 1 : (hidden <= 4096 ? 2 : 4);
   hipStream_t s = (hipStream_t)stream;
-  if (d == 64)
-    hipLaunchKernelGGL((decode_qkv_kernel<64>), dim3(blocks), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv,
+#define IRON_QKV(DD, C)                                                                             \
+  if (d == DD && ch == C)                                                                           \
+    hipLaunchKernelGGL((decode_qkv_kernel<DD, C>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
                        angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position);
-  else
-    hipLaunchKernelGGL((decode_qkv_kernel<128>), dim3(blocks), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv,
-                       angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position);
+  IRON_QKV(64, 1) IRON_QKV(64, 2) IRON_QKV(64, 4) IRON_QKV(128, 1) IRON_QKV(128, 2) IRON_QKV(128, 4)
+#undef IRON_QKV
   IRON_LAUNCH_CHECK();
 }

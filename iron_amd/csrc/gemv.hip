@@ -121,15 +121,14 @@ extern "C" int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16
   hipStream_t s = (hipStream_t)stream;
   int rpw = rows_per_wave, ks = k_split;
   if (rpw == 0 || ks == 0) {
-    // Heuristic: keep >= ~8 waves per CU in flight where the matrix allows it, and
-    // give every lane several independent 16-byte loads.
-    const long waves_1row = (long)M * batches;  // one wave per row
-    const int steps = (K / 8 + 63) / 64;         // loads a lane issues per row at KSPLIT 1
-    if (waves_1row >= 64L * 1024) { rpw = 4; ks = 1; }
-    else if (waves_1row >= 8L * 1024) { rpw = 2; ks = 1; }
-    else if (waves_1row >= 2048) { rpw = 1; ks = steps >= 8 ? 2 : 1; }
-    else if (waves_1row >= 1024) { rpw = 1; ks = steps >= 4 ? 2 : 1; }
-    else { rpw = 1; ks = steps >= 4 ? 4 : (steps >= 2 ? 2 : 1); }
+    // Measured on MI355X under graph replay over weights larger than the last-level cache: the
+    // four waves of a block splitting K (one contiguous row stream per block) win at every
+    // size once a row is at least 2 KB; tall matrices of short rows take 2-4 rows a wave.
+    const long rows = (long)M * batches;
+    const int chunks = K / 8;
+    ks = chunks >= 128 ? 4 : (chunks >= 64 ? 2 : 1);
+    if (chunks >= 1024) rpw = 1;
+    else rpw = rows >= 65536 ? 4 : (rows >= 8192 ? 2 : 1);
   }
   const bf16_t* Wp = W; const bf16_t* xp = x; bf16_t* yp = y;
 #define IRON_GEMV_CASE(R, S)                                                   \
