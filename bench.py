@@ -86,6 +86,68 @@ def bench_gemm(torch, K, dev, steps, rng, b_col_maj):
             "TFLOPs": round(flops / us / 1e6, 1), "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
+def bench_attention(torch, K, dev, n, rng):
+    """GQA causal attention, 32 q / 8 kv heads, d 64, scale 1/8: prefill at S = 512, 2048, 8192 (MFMA bound)
+    and one query over caches of 1024, 4096, 16384 keys (HBM bound)."""
+    H, G, D = 32, 8, 64
+    out = {"prefill": [], "decode": []}
+
+    def rand(*shape):
+        return torch.randn(shape, device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+    for S in (512, 2048, 8192):
+        Q, Kc, Vc = rand(S, H, D), rand(S, G, D), rand(S, G, D)
+        O = torch.empty_like(Q)
+        launches = [lambda: K.mha_prefill(Q, Kc, Vc, O, heads=H, kv_heads=G, d=D, seq=S, kv_len=S, scale=0.125,
+                                          q_interleaved=True, kv_interleaved=True)] * 10
+        us = graph_time_us(torch, launches, max(1, n // (10 * max(1, S // 512))))
+        flops = 4.0 * H * D * S * (S + 1) / 2
+        out["prefill"].append({"S": S, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                               "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)})
+    for L in (1024, 4096, 16384):
+        copies = max(2, min(64, int(np.ceil(400e6 / (L * G * D * 4)))))
+        Q = rand(1, H, D)
+        Ks, Vs = [rand(L, G, D) for _ in range(copies)], [rand(L, G, D) for _ in range(copies)]
+        O = torch.empty_like(Q)
+        ws = K.mha_decode_workspace(H, D, dev)
+        launches = [(lambda a=a, b=b: K.mha_decode(Q, a, b, O, heads=H, kv_heads=G, d=D, kv_len=L, scale=0.125,
+                                                   kv_interleaved=True, workspace=ws)) for a, b in zip(Ks, Vs)]
+        us = graph_time_us(torch, launches, max(1, n // len(launches)))
+        algo = 2 * L * G * D * 2 + 2 * H * D * 2
+        out["decode"].append({"L": L, "us": round(us, 2), "GBps": round(algo / us / 1e3, 1),
+                              "frac_hbm": round(algo / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": algo})
+    return out
+
+
+def bench_pre_attention(torch, K, dev, n):
+    """The pre-attention block at sequence 2048, hidden 2048: RMSNorm, the Q/K/V projections (32 q / 8 kv heads,
+    d 64) and RoPE on q and k, as the prompt chunk runs them (five operator steps)."""
+    S, E, H, G, D = 2048, 2048, 32, 8, 64
+
+    def rand(*shape, scale=1.0):
+        return (torch.randn(shape, device=dev, dtype=torch.float32) * scale).to(torch.bfloat16)
+
+    x, gain = rand(S, E), (torch.rand(E, device=dev) * 0.2 + 0.9).to(torch.bfloat16)
+    Wq, Wk, Wv = rand(H * D, E, scale=0.02), rand(G * D, E, scale=0.02), rand(G * D, E, scale=0.02)
+    theta = torch.rand(S, D // 2, device=dev) * 6.28
+    ang = torch.stack([torch.cos(theta), torch.sin(theta)], dim=-1).reshape(S, D).to(torch.bfloat16)
+    n_, q, k, v = torch.empty_like(x), rand(S, H * D), rand(S, G * D), rand(S, G * D)
+    qr, kr = torch.empty_like(q), torch.empty_like(k)
+
+    def block():
+        K.rmsnorm(x, gain, n_, rows=S, cols=E, eps=1e-5)
+        K.gemm(n_, Wq, q, M=S, N=H * D, K=E, b_col_maj=True)
+        K.gemm(n_, Wk, k, M=S, N=G * D, K=E, b_col_maj=True)
+        K.gemm(n_, Wv, v, M=S, N=G * D, K=E, b_col_maj=True)
+        K.rope(q, ang, qr, rows=S * H, cols=D, angle_rows=S)
+        K.rope(k, ang, kr, rows=S * G, cols=D, angle_rows=S)
+
+    us = graph_time_us(torch, [block] * 4, max(1, n // 8))
+    flops = 2.0 * S * E * (H + 2 * G) * D
+    return {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1), "kernels": 6,
+            "bytes_unfused": 71_600_000, "bytes_fused_min": 33_600_000}
+
+
 def cpu_gemv_baseline(rng, budget_s=12.0):
     """The oracle's GEMV (the reference's CPU path: the weight up-cast to f32 on every call,
     gemv.py:413) timed on the host cores on a bounded sample of the sweep."""
@@ -184,7 +246,8 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu):
            "prefill_tokens": 512, "decode_steps": steps, "wall_s": round(wall, 4),
            "bytes_per_token": int(per_token), "GBps": round(per_token * tok_s / 1e9, 1),
            "frac_hbm": round(per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
-           "kernels_per_step": len(decode.recording.steps), "first_tokens": [int(t) for t in tokens[:4]]}
+           "steps_recorded": len(decode.recording.steps),
+           "launches_per_step": decode.launches_per_call, "first_tokens": [int(t) for t in tokens[:4]]}
     cpu = None
     if with_cpu:
         cpu = cpu_decoder_baseline(torch, config, weights)
@@ -261,6 +324,8 @@ def main():
     n = args.kernel_launches
     gemv = [bench_gemv(torch, K, dev, Kd, N, n, rng) for Kd, N in GEMV_SWEEP]
     gemm = [bench_gemm(torch, K, dev, n, rng, b) for b in (False, True)]
+    attention = bench_attention(torch, K, dev, n, rng)
+    pre_attention = bench_pre_attention(torch, K, dev, n)
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     decoder, cpu = bench_decoder(torch, dev, args.steps, args.warmup, not args.no_cpu)
@@ -287,13 +352,15 @@ def main():
                                "512-token prompt prefill, then greedy decode steps replayed as a HIP graph; "
                                "one step = one decoded token",
                    "prefill_tokens": 512, "decode_steps": args.steps},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<4,1> (the 2048->128256 LM head, the largest launch of a "
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<4,4> (the 2048->128256 LM head, the largest launch of a "
                                                "decode step)",
                      "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["frac_hbm"], "traffic": None},
         "decoder": decoder,
         "gemv_sweep": {"GBps": round(sweep_bytes / sweep_us / 1e3, 1), "shapes": gemv},
         "gemm": gemm,
+        "attention": attention,
+        "pre_attention_block": pre_attention,
         "bench_wall_s": round(wall, 1),
     }
     if cpu is not None:
