@@ -46,16 +46,15 @@ __device__ __forceinline__ float bf16_hi(uint32_t w) {
   return __builtin_bit_cast(float, w & 0xffff0000u);
 }
 
-// float -> bf16, round to nearest even (NaN stays quiet NaN).
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
-}
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// Two floats -> packed bf16, round to nearest even, in hardware (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return (bf16_t)(pack_bf16(f, 0.f) & 0xffffu); }
 // Round a float to the nearest bf16 and return it as float.
 __device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
@@ -83,14 +82,39 @@ __device__ __forceinline__ void store_stream(uint4* p, const uint4& v) {
   __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(p));
 }
 
+// Wave-wide reductions on the DPP data path (no LDS traffic): within quads, half rows and
+// rows, then across rows with the row broadcasts; lane 63 ends with the total.
+#define IRON_DPP(old, v, ctrl, rows) \
+  __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), ctrl, rows, 0xF, false))
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  v += IRON_DPP(0.f, v, 0xB1, 0xF);   // quad_perm [1,0,3,2]
+  v += IRON_DPP(0.f, v, 0x4E, 0xF);   // quad_perm [2,3,0,1]
+  v += IRON_DPP(0.f, v, 0x141, 0xF);  // row_half_mirror
+  v += IRON_DPP(0.f, v, 0x140, 0xF);  // row_mirror: every lane of a row holds the row's sum
+  v += IRON_DPP(0.f, v, 0x142, 0xA);  // row_bcast15 into rows 1 and 3
+  v += IRON_DPP(0.f, v, 0x143, 0xC);  // row_bcast31 into rows 2 and 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  v = fmaxf(v, IRON_DPP(v, v, 0xB1, 0xF));
+  v = fmaxf(v, IRON_DPP(v, v, 0x4E, 0xF));
+  v = fmaxf(v, IRON_DPP(v, v, 0x141, 0xF));
+  v = fmaxf(v, IRON_DPP(v, v, 0x140, 0xF));
+  v = fmaxf(v, IRON_DPP(v, v, 0x142, 0xA));
+  v = fmaxf(v, IRON_DPP(v, v, 0x143, 0xC));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+// Sum over each aligned group of 8 lanes (every lane of the group gets it).
+__device__ __forceinline__ float group8_sum(float v) {
+  v += IRON_DPP(0.f, v, 0xB1, 0xF);
+  v += IRON_DPP(0.f, v, 0x4E, 0xF);
+  v += IRON_DPP(0.f, v, 0x141, 0xF);
+  return v;
+}
+// ... and of 16 lanes (a DPP row).
+__device__ __forceinline__ float group16_sum(float v) {
+  v = group8_sum(v);
+  v += IRON_DPP(0.f, v, 0x140, 0xF);
   return v;
 }
 

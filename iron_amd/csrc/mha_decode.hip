@@ -78,8 +78,9 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
         float d = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
-#pragma unroll
-        for (int o = 1; o < LPR; o <<= 1) d += __shfl_xor(d, o, 64);
+        if (LPR == 8) d = group8_sum(d);
+        else if (LPR == 16) d = group16_sum(d);
+        else { d = group16_sum(d); d += __shfl_xor(d, 16, 64); }
         s[u][g] = live[u] ? d : -INFINITY;
       }
     }
