@@ -237,8 +237,11 @@ extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const 
   const int G = heads / kv_heads;
   const long row_stride = kv_interleaved ? (long)kv_heads * d : d;
   const long head_stride = kv_interleaved ? d : (long)kv_len * d;
-  int nsplit = (kv_len + 63) / 64;
-  nsplit = nsplit < 1 ? 1 : (nsplit > kMaxSplits ? kMaxSplits : nsplit);
+  // Measured: a split per 128 keys, at least 8 (short caches are launch-bound) and at most 64
+  // (beyond that the merge of the splits costs more than the extra parallelism gains).
+  int nsplit = (kv_len + 127) / 128;
+  nsplit = nsplit < 8 ? 8 : (nsplit > 64 ? 64 : nsplit);
+  if (nsplit * 8 > kv_len) nsplit = kv_len >= 8 ? kv_len / 8 : 1;
   const float scale_log2 = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
   float* part = (float*)workspace;

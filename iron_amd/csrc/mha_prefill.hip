@@ -28,8 +28,11 @@ __global__ __launch_bounds__(256) void mha_prefill_kernel(
   constexpr int LDV = BKV + 8;   // V^T tile row
   constexpr int KS = D / 16;     // k16 steps of S^T
   constexpr int DT = D / 32;     // 32-row tiles of O^T
-  __shared__ __align__(16) bf16_t Ks[BKV * LDK];
-  __shared__ __align__(16) bf16_t Vt[D * LDV];
+  constexpr int CPR = D / 8;     // 16-byte chunks a key row has
+  constexpr int NL = BKV * CPR / 256;   // 16-byte loads a thread makes of K (and of V) per tile
+  constexpr int K_TILE = BKV * LDK, V_TILE = D * LDV;
+  __shared__ __align__(16) bf16_t Ks[2 * K_TILE];
+  __shared__ __align__(16) bf16_t Vt[2 * V_TILE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, g = lane >> 5;
@@ -46,12 +49,14 @@ __global__ __launch_bounds__(256) void mha_prefill_kernel(
   const int my_q = q0 + wave * 32 + col;            // this lane's query row
   const bool q_live = my_q < q_tokens;
   const int qpos = offset + my_q;
+  const int wq_lo = offset + q0 + wave * 32;        // positions of the wave's first and last live query
+  const int wq_hi = offset + min(q0 + wave * 32 + 31, q_tokens - 1);
 
   bf16_t* Oh = O + (size_t)head * q_head_stride;
   // Rows of this block past the bound: zeros.  A block wholly past it does only that.
   if (q0 >= q_tokens || offset < 0) {
-    for (int i = tid; i < BQ * (D / 8); i += 256) {
-      const int r = q0 + i / (D / 8), c = (i % (D / 8)) * 8;
+    for (int i = tid; i < BQ * CPR; i += 256) {
+      const int r = q0 + i / CPR, c = (i % CPR) * 8;
       if (r < seq) *reinterpret_cast<uint4*>(Oh + (size_t)r * q_row_stride + c) = make_uint4(0, 0, 0, 0);
     }
     return;
@@ -74,7 +79,7 @@ __global__ __launch_bounds__(256) void mha_prefill_kernel(
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int e = 0; e < 16; ++e) oacc[t][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;   // the running max is of the raw (unscaled) scores
 
   // Keys this block's live queries can see.
   const int q_last = min(q0 + BQ, q_tokens) - 1;
@@ -87,110 +92,138 @@ __global__ __launch_bounds__(256) void mha_prefill_kernel(
   const bf16_t* Kh = K + (size_t)kvh * kv_head_stride;
   const bf16_t* Vh = V + (size_t)kvh * kv_head_stride;
 
-  for (int kv0 = kv_lo; kv0 < kv_hi; kv0 += BKV) {
-    __syncthreads();
-    // K tile: rows kv0..kv0+63, as stored.
+  // Tile staging: K as stored; V two keys a load pair, transposed on the way into LDS.
+  uint4 kreg[NL], vreg[NL];
+  auto fetch = [&](int kv0) {
 #pragma unroll
-    for (int i = 0; i < BKV * (D / 8) / 256; ++i) {
+    for (int i = 0; i < NL; ++i) {
       const int p = tid + i * 256;
-      const int r = p / (D / 8), c = (p % (D / 8)) * 8;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (kv0 + r < kv_tokens)
-        v = *reinterpret_cast<const uint4*>(Kh + (size_t)(kv0 + r) * kv_row_stride + c);
-      *reinterpret_cast<uint4*>(Ks + r * LDK + c) = v;
+      const int r = p / CPR, c = (p % CPR) * 8;
+      kreg[i] = (kv0 + r < kv_tokens) ? *reinterpret_cast<const uint4*>(Kh + (size_t)(kv0 + r) * kv_row_stride + c)
+                                      : make_uint4(0, 0, 0, 0);
     }
-    // V tile, transposed: a thread takes 4 key rows x 8 columns and writes 8 runs of 4 keys.
-    for (int p = tid; p < (BKV / 4) * (D / 8); p += 256) {
-      const int strip = p % (D / 8), kg = p / (D / 8);
-      uint32_t w[4][4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        const int kr = kv0 + kg * 4 + r;
-        if (kr < kv_tokens)
-          v = *reinterpret_cast<const uint4*>(Vh + (size_t)kr * kv_row_stride + strip * 8);
-        w[r][0] = v.x; w[r][1] = v.y; w[r][2] = v.z; w[r][3] = v.w;
-      }
+    for (int i = 0; i < NL; ++i) {
+      // load i is key 2*pair + (i & 1) of strip `tid % CPR`, pair = tid / CPR + (i / 2) * (256 / CPR)
+      const int strip = tid % CPR, key = 2 * (tid / CPR + (i >> 1) * (256 / CPR)) + (i & 1);
+      vreg[i] = (kv0 + key < kv_tokens) ? *reinterpret_cast<const uint4*>(Vh + (size_t)(kv0 + key) * kv_row_stride + strip * 8)
+                                        : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stage = [&](int buf) {
+    bf16_t* kd = Ks + buf * K_TILE;
+    bf16_t* vd = Vt + buf * V_TILE;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int p = tid + i * 256;
+      *reinterpret_cast<uint4*>(kd + (p / CPR) * LDK + (p % CPR) * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NL; i += 2) {
+      const int strip = tid % CPR, key = 2 * (tid / CPR + (i >> 1) * (256 / CPR));
+      const uint32_t a[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+      const uint32_t b[4] = {vreg[i + 1].x, vreg[i + 1].y, vreg[i + 1].z, vreg[i + 1].w};
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-        uint2 out;
-        out.x = __builtin_amdgcn_perm(w[1][c >> 1], w[0][c >> 1], sel);
-        out.y = __builtin_amdgcn_perm(w[3][c >> 1], w[2][c >> 1], sel);
-        *reinterpret_cast<uint2*>(Vt + (strip * 8 + c) * LDV + kg * 4) = out;
+        *reinterpret_cast<uint32_t*>(vd + (strip * 8 + c) * LDV + key) = __builtin_amdgcn_perm(b[c >> 1], a[c >> 1], sel);
       }
     }
-    __syncthreads();
+  };
 
-    // S^T = K Q^T for the two 32-key halves of the tile.
-    f32x16 sacc[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const bf16x8 kf =
-            *reinterpret_cast<const bf16x8*>(Ks + (t * 32 + col) * LDK + 16 * s + 8 * g);
-        sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[t], 0, 0, 0);
-      }
-    }
+  if (kv_lo < kv_hi) {
+    fetch(kv_lo);
+    stage(0);
+  }
+  __syncthreads();
 
-    // Mask, scale, online softmax.  Element e of half t is key
-    // kv0 + 32 t + 8 (e/4) + 4 g + e%4, query `col`.
-    float rmax = -INFINITY;
+  int buf = 0;
+  for (int kv0 = kv_lo; kv0 < kv_hi; kv0 += BKV, buf ^= 1) {
+    const bool more = kv0 + BKV < kv_hi;
+    if (more) fetch(kv0 + BKV);   // in flight during this tile's MFMAs
+
+    // Tiles wholly above the wave's last query (causal) hold nothing for it.
+    const bool skip = causal && kv0 > wq_hi;
+    if (!skip) {
+      const bf16_t* kt = Ks + buf * K_TILE;
+      const bf16_t* vt = Vt + buf * V_TILE;
+      // S^T = K Q^T for the two 32-key halves of the tile.
+      f32x16 sacc[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int kpos = kv0 + 32 * t + 8 * (e >> 2) + 4 * g + (e & 3);
-        bool dead = kpos >= kv_tokens || !q_live;
-        if (causal) dead |= kpos > qpos;
-        else if (window >= 0) dead |= kpos > qpos + window;
-        if (window >= 0) dead |= kpos < qpos - window;
-        const float v = dead ? -INFINITY : sacc[t][e] * scale_log2;
-        sacc[t][e] = v;
-        rmax = fmaxf(rmax, v);
-      }
-    rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
-    const float m_new = fmaxf(m_run, rmax);
-    const float ref = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = exp2f(m_run - ref);
-    m_run = m_new;
-    float rsum = 0.f;
-    bf16x8 pf[2][2];
+        for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        float p[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          p[j] = exp2f(sacc[t][8 * h + j] - ref);
-          rsum += p[j];
+        for (int s = 0; s < KS; ++s) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kt + (t * 32 + col) * LDK + 16 * s + 8 * g);
+          sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[t], 0, 0, 0);
         }
-        pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
       }
-    l_run = l_run * alpha + rsum;
+      // Only tiles that touch a bound or the mask's edge pay for masking.  Element e of half t
+      // is key kv0 + 32 t + 8 (e/4) + 4 g + e%4, query `col`.
+      bool edge = kv0 + BKV > kv_tokens;
+      if (causal) edge |= kv0 + BKV - 1 > wq_lo;
+      else if (window >= 0) edge |= kv0 + BKV - 1 > wq_lo + window;
+      if (window >= 0) edge |= kv0 < wq_hi - window;
+      if (edge) {
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
-
-    // O^T += V^T P^T.  k slots of lane group g at (t, h): keys 32 t + 16 h + 4 g + 0..3
-    // and the same + 8.
+          for (int e = 0; e < 16; ++e) {
+            const int kpos = kv0 + 32 * t + 8 * (e >> 2) + 4 * g + (e & 3);
+            bool dead = kpos >= kv_tokens;
+            if (causal) dead |= kpos > qpos;
+            else if (window >= 0) dead |= kpos > qpos + window;
+            if (window >= 0) dead |= kpos < qpos - window;
+            if (dead) sacc[t][e] = -INFINITY;
+          }
+      }
+      float rmax = sacc[0][0];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
+      rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
+      const float m_new = fmaxf(m_run, rmax);
+      const float mc = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
+      const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc));  // exp2(-inf) = 0 at the start
+      m_run = m_new;
+      float rsum = 0.f;
+      bf16x8 pf[2][2];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const bf16_t* vp = Vt + (dt * 32 + col) * LDV + 32 * t + 16 * h + 4 * g;
-          const uint2 lo = *reinterpret_cast<const uint2*>(vp);
-          const uint2 hi = *reinterpret_cast<const uint2*>(vp + 8);
-          const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[t][h], oacc[dt], 0, 0, 0);
+          float p[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            p[j] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * h + j], scale_log2, -mc));
+            rsum += p[j];
+          }
+          pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
         }
+      l_run = l_run * alpha + rsum;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
+
+      // O^T += V^T P^T.  k slots of lane group g at (t, h): keys 32 t + 16 h + 4 g + 0..3 and the same + 8.
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const bf16_t* vp = vt + (dt * 32 + col) * LDV + 32 * t + 16 * h + 4 * g;
+            const uint2 lo = *reinterpret_cast<const uint2*>(vp);
+            const uint2 hi = *reinterpret_cast<const uint2*>(vp + 8);
+            const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[t][h], oacc[dt], 0, 0, 0);
+          }
+    }
+    if (more) stage(buf ^ 1);   // the other buffer: everyone finished reading it a tile ago
+    __syncthreads();
   }
 
   // Normalize and store: lane holds query `col`, columns 32 dt + 8 q + 4 g + 0..3.
