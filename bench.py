@@ -286,6 +286,38 @@ def cpu_decoder_baseline(torch, config, weights, budget_s=12.0):
                       f"graph reference, {dt:.1f} s wall; weights held as float32, prompt not prefilled on the CPU"}
 
 
+PROBE_COPY_BYTES = 512 << 20
+# HBM bytes one launch of the head GEMV moves, from hardware counters (FETCH_SIZE and WRITE_SIZE of
+# `--counter-probe`, each scaled by what the same counter reads for the probe's 512 MiB copy):
+# 513122 KiB fetched + 1002 KiB written.  The algorithmic figure is 525.6 MB.
+HEAD_GEMV_TRAFFIC_BYTES = (513122 + 1002) * 1024
+
+
+def counter_probe(torch, K, dev, rng):
+    """The dominant kernel (the 2048 -> 128256 head GEMV over two distinct weights, 4 launches) and a
+    plain copy that reads and writes PROBE_COPY_BYTES (2 launches): what a hardware-counter run needs
+    to turn FETCH_SIZE / WRITE_SIZE readings of the GEMV into bytes."""
+    from iron_amd.bf16 import round_bf16, to_torch
+
+    Kdim, N = GEMV_SWEEP[-1]
+    base = to_torch(round_bf16(rng.standard_normal((N, Kdim), dtype=np.float32) * np.float32(0.02))).to(dev)
+    pool = [base, base.clone()]
+    x = to_torch(round_bf16(rng.standard_normal(Kdim, dtype=np.float32))).to(dev)
+    y = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    rows, row_bytes = PROBE_COPY_BYTES // 4096, 4096
+    src = torch.zeros(PROBE_COPY_BYTES // 4, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for i in range(4):
+        K.gemv(pool[i % 2], x, y, M=N, K=Kdim)
+    for _ in range(2):
+        K.copy_rows(src, dst, rows=rows, row_elems=row_bytes // 4, src_rows=rows, dst_rows=rows)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "counter", "gemv": {"K": Kdim, "N": N, "launches": 4,
+                                                     "algorithmic_bytes": 2 * (N * Kdim + Kdim + N)},
+                      "copy": {"launches": 2, "bytes_read": PROBE_COPY_BYTES, "bytes_written": PROBE_COPY_BYTES}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -293,6 +325,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--kernel-launches", type=int, default=400, help="timed launches per kernel micro-benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="launch only the LM-head GEMV and a plain copy of known size (for a rocprofv3 --pmc run) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is a one-GPU hot path; --gpus must be 1 "
@@ -319,6 +353,10 @@ def main():
         yy = torch.empty(512, dtype=torch.bfloat16, device=dev)
         K.gemv(w, xx, yy, M=512, K=2048)
     torch.cuda.synchronize()
+
+    if args.counter_probe:
+        counter_probe(torch, K, dev, rng)
+        return 0
 
     t_wall = time.perf_counter()
     n = args.kernel_launches
@@ -355,7 +393,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gemv_kernel<4,4> (the 2048->128256 LM head, the largest launch of a "
                                                "decode step)",
                      "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["frac_hbm"], "traffic": None},
+                     "frac": head["frac_hbm"], "traffic": HEAD_GEMV_TRAFFIC_BYTES},
         "decoder": decoder,
         "gemv_sweep": {"GBps": round(sweep_bytes / sweep_us / 1e3, 1), "shapes": gemv},
         "gemm": gemm,
