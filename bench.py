@@ -72,12 +72,12 @@ def bench_gemv(torch, K, dev, Kdim, N, steps, rng):
             "frac_hbm": round(algo / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": algo, "copies": copies}
 
 
-def bench_gemm(torch, K, dev, steps, rng, b_col_maj):
+def bench_gemm(torch, K, dev, steps, rng, b_col_maj, M=2048, N=2048, Kd=2048):
     from iron_amd.bf16 import round_bf16, to_torch
 
-    M = N = Kd = 2048
     A = to_torch(round_bf16(rng.standard_normal((M, Kd), dtype=np.float32) * np.float32(0.02))).to(dev)
-    B = to_torch(round_bf16(rng.standard_normal((Kd, N), dtype=np.float32) * np.float32(0.02))).to(dev)
+    B = to_torch(round_bf16(rng.standard_normal((N, Kd) if b_col_maj else (Kd, N), dtype=np.float32)
+                            * np.float32(0.02))).to(dev)
     C = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
     launches = [lambda: K.gemm(A, B, C, M=M, N=N, K=Kd, b_col_maj=b_col_maj)] * 20
     us = graph_time_us(torch, launches, max(1, steps // 20))
@@ -362,6 +362,9 @@ def main():
     n = args.kernel_launches
     gemv = [bench_gemv(torch, K, dev, Kd, N, n, rng) for Kd, N in GEMV_SWEEP]
     gemm = [bench_gemm(torch, K, dev, n, rng, b) for b in (False, True)]
+    # The prefill projections of the decoder (2048 tokens; weights (N,K)) and two larger squares.
+    gemm += [bench_gemm(torch, K, dev, max(20, n // 4), rng, True, M=m, N=nn, Kd=k)
+             for m, nn, k in ((2048, 8192, 2048), (2048, 2048, 8192), (4096, 4096, 4096), (8192, 8192, 8192))]
     attention = bench_attention(torch, K, dev, n, rng)
     pre_attention = bench_pre_attention(torch, K, dev, n)
     torch.cuda.synchronize()

@@ -353,8 +353,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
       b_src[i] = B + (size_t)kr * N + n0 + lc * 8;
     }
   }
-  auto issue = [&](int kt) {
-    char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
+  auto issue = [&](int kt, int buf) {
+    char* st = smem_nt + buf * NT_STAGE_BYTES;
     const int k0 = kt * BK;
 #pragma unroll
     for (int i = 0; i < INST; ++i)
@@ -375,9 +375,10 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int nk = K / BK;
+  // Always three stages in flight before the loop (short K repeats its last stage), so the
+  // loop's wait counts hold from the first iteration.
 #pragma unroll
-  for (int s = 0; s < NT_STAGES - 1; ++s)
-    if (s < nk) issue(s);
+  for (int s = 0; s < NT_STAGES - 1; ++s) issue(min(s, nk - 1), s);
 
   const int fr = lane & 31, kh = lane >> 5;
   int a_off[2], a_swz[2], b_off[2], b_swz[2];
@@ -393,43 +394,75 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < 2; ++i) tr_n[i] = wn * 64 + i * 32 + (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
 
+  // One load of the 2*INST a wave issues per stage (A's first, then B's).
+  auto issue_one = [&](char* st, int kt, int idx) {
+    const int k0 = kt * BK;
+    if (idx < INST)
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_src[idx] + k0),
+                                       IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds(
+          IRON_GLOBAL_PTR(b_src[idx - INST] + (B_KN ? (size_t)k0 * N : (size_t)k0)),
+          IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
+  };
+  auto read_frag_pair = [&](const char* st, int ks, int i, bf16x8& a, bf16x8& b) {
+    const int j = ks * 2 + kh;
+    a = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
+    if constexpr (!B_KN) {
+      b = *reinterpret_cast<const bf16x8*>(st + b_off[i] + ((j ^ b_swz[i]) << 4));
+    } else {
+      const int k = ks * 16 + tr_k;  // rows k and k + 4, each with its own swizzle
+      const int c0 = ((tr_n[i] >> 3) ^ ((k & 7) << 1)) << 4;
+      const int c1 = ((tr_n[i] >> 3) ^ (((k + 4) & 7) << 1)) << 4;
+      const int half = (tr_n[i] & 4) << 1;
+      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + k * 256 + c0 + half));
+      const short4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + (k + 4) * 256 + c1 + half));
+      typedef short short8v __attribute__((ext_vector_type(8)));
+      const short8v both = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+      b = __builtin_bit_cast(bf16x8, both);
+    }
+  };
+  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[2], bf16x8 (&bfr)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) read_frag_pair(st, ks, i, af[i], bfr[i]);
+  };
+  // A wave is alone on its SIMD, so nothing overlaps unless its own instruction stream interleaves:
+  // each k-step's four MFMAs are issued with the next step's fragment reads and a quarter of the
+  // stage being prefetched between them.
   for (int kt = 0; kt < nk; ++kt) {
     // Stage kt has landed once at most the two younger stages' loads are outstanding.
-    if (kt + NT_STAGES - 2 < nk) wait_vmcnt<(NT_STAGES - 2) * LOADS>(); else wait_vmcnt<0>();
+    wait_vmcnt<(NT_STAGES - 2) * LOADS>();
     block_barrier();  // everyone's loads of stage kt are in; everyone is done reading stage kt-1
-    if (kt + NT_STAGES - 1 < nk) issue(kt + NT_STAGES - 1);  // into the buffer of stage kt-1
+    // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
+    // (into buffers nobody reads any more) rather than branch: every iteration issues the same
+    // loads, which keeps the wait count above exact and the scheduling region whole.
+    const int kn = min(kt + NT_STAGES - 1, nk - 1);
+    char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
     const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
+    bf16x8 af[2][2], bfr[2][2];
+    read_frags(st, 0, af[0], bfr[0]);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      const int j = ks * 2 + kh;
-      bf16x8 af[2], bfr[2];
+      const int cur = ks & 1, nxt = cur ^ 1;
+      // Source order is issue order (nothing crosses a sched_barrier): while an MFMA runs, half of
+      // the next k-step's fragment reads or one prefetch load goes out.
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        af[i] = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
-        if constexpr (!B_KN) {
-          bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_off[i] + ((j ^ b_swz[i]) << 4));
-        } else {
-          const int k = ks * 16 + tr_k;  // rows k and k + 4, each with its own swizzle
-          const int c0 = ((tr_n[i] >> 3) ^ ((k & 7) << 1)) << 4;
-          const int c1 = ((tr_n[i] >> 3) ^ (((k + 4) & 7) << 1)) << 4;
-          const int half = (tr_n[i] & 4) << 1;
-          const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + k * 256 + c0 + half));
-          const short4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + (k + 4) * 256 + c1 + half));
-          typedef short short8v __attribute__((ext_vector_type(8)));
-          const short8v both = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
-          bfr[i] = __builtin_bit_cast(bf16x8, both);
-        }
+        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][i], acc[i][0], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks + 1 < BK / 16) read_frag_pair(st, ks + 1, i, af[nxt][i], bfr[nxt][i]);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][1], af[cur][i], acc[i][1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue_one(nst, kn, ks * 2 + i);
+        __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int jj = 0; jj < 2; ++jj)
-          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[jj], af[i], acc[i][jj], 0, 0, 0);
     }
   }
 
+  wait_vmcnt<0>();  // the idle fetches of the last iterations land before the block's LDS is released
   const int hi = kh * 4;
   const bool vec = (N & 3) == 0;
 #pragma unroll
@@ -497,6 +530,188 @@ static int launch_gemm(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N
   IRON_LAUNCH_CHECK();
 }
 
+
+// Large problems, B (N,K): 256x256x64 tiles, two 64 KB stages fed straight into LDS, 4 waves each
+// owning 128x128 of the tile (16 MFMA tiles, 256 accumulator registers).  Against the 128x128
+// kernel a wave reads half as many LDS bytes and a CU pulls half as many global bytes per flop --
+// the 64 B/clk a CU can move from L2 into LDS is what bounds the smaller tile.  A wave is alone on
+// its SIMD, so its own instruction stream interleaves the next k-step's fragment reads and a
+// quarter of the next stage's loads with the 16 MFMAs of a k-step.
+constexpr int BIG_BM = 256, BIG_BN = 256;
+#ifndef IRON_BIG_WAVES
+#define IRON_BIG_WAVES 4
+#endif
+constexpr int BIG_WAVES = IRON_BIG_WAVES;
+#define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
+constexpr int BIG_A_BYTES = BIG_BM * BK * 2, BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
+
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
+                                                         const bf16_t* __restrict__ B,
+                                                         bf16_t* __restrict__ C, int M, int N, int K,
+                                                         const int* __restrict__ valid, int tiles_m,
+                                                         int tiles_n, int patched) {
+  constexpr int INST = BIG_BM / 8 / WAVES;   // 1 KB loads of A (and of B) a wave issues per stage
+  constexpr int TN = 8 / WAVES * 2;          // 32-column MFMA tiles a wave owns along n (4 or 2)
+  constexpr int KSTEPS = BK / 16;
+  extern __shared__ __align__(16) char smem_big[];
+  const int Mv = bound_or(valid, M);
+
+  int tm, tn;
+  const int bid = blockIdx.x;
+  if (patched) {
+    const int xcd = bid & 7, loc = bid >> 3;
+    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
+    const int patches_n = tiles_n >> 2;
+    tm = (patch / patches_n) * 8 + (within & 7);
+    tn = (patch % patches_n) * 4 + (within >> 3);
+  } else {
+    constexpr int BAND = 8;
+    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
+    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
+    tm = first + in_band % height;
+    tn = in_band / height;
+  }
+  const int m0 = tm * BIG_BM, n0 = tn * BIG_BN;
+  if (m0 >= Mv) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / (WAVES / 2), wn = wave % (WAVES / 2);
+  // Loader: instruction i of a wave moves rows (wave*INST + i)*8 .. +7; lane -> (row, physical
+  // chunk); the logical chunk it fetches is the physical one swizzled by the row.
+  const int lrow = lane >> 3, pch = lane & 7;
+  unsigned ld_off[2];   // byte offset of this lane's 16 bytes within an even / odd instruction's rows
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    const int r = par * 8 + lrow;
+    ld_off[par] = (unsigned)(((size_t)lrow * K + (pch ^ ((r >> 1) & 7)) * 8) * 2);
+  }
+  const char* a_base = reinterpret_cast<const char*>(A + (size_t)(m0 + wave * INST * 8) * K);
+  const char* b_base = reinterpret_cast<const char*>(B + (size_t)(n0 + wave * INST * 8) * K);
+  const size_t inst_stride = (size_t)8 * K * 2;   // 8 rows
+  auto issue_one = [&](char* st, int kt, int idx) {
+    const size_t k_off = (size_t)kt * BK * 2;
+    if (idx < INST)
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_base + idx * inst_stride + k_off + ld_off[idx & 1]),
+                                       IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds(
+          IRON_GLOBAL_PTR(b_base + (idx - INST) * inst_stride + k_off + ld_off[idx & 1]),
+          IRON_LDS_PTR(st + BIG_A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
+  };
+
+  f32x16 acc[4][TN];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int idx = 0; idx < 2 * INST; ++idx) issue_one(smem_big, 0, idx);
+
+  const int fr = lane & 31, kh = lane >> 5;
+  const int swz = (fr >> 1) & 7;   // tile rows are multiples of 32 apart: one swizzle for all
+  const int a_row = (wm * 128 + fr) * 128, b_row = BIG_A_BYTES + (wn * TN * 32 + fr) * 128;
+  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[4], bf16x8 (&bfr)[TN]) {
+    const int c = ((ks * 2 + kh) ^ swz) << 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * 128 + c);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * 128 + c);
+  };
+
+  for (int kt = 0; kt < nk; ++kt) {
+    wait_vmcnt<0>();   // this wave's share of stage kt has landed
+    block_barrier();   // so has everyone's; and everyone is done reading stage kt-1
+    // The next stage goes into the buffer stage kt-1 used.  The last iteration fetches its own
+    // stage again (into the idle buffer) rather than branch: a branch would end the scheduling
+    // region and undo the interleaving below.
+    const int kn = min(kt + 1, nk - 1);
+    char* nst = smem_big + ((kt + 1) & 1) * BIG_STAGE_BYTES;
+    const char* st = smem_big + (kt & 1) * BIG_STAGE_BYTES;
+    bf16x8 af[2][4], bfr[2][TN];
+    read_frags(st, 0, af[0], bfr[0]);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      const int c = (((ks + 1) * 2 + kh) ^ swz) << 4;
+      // Source order is issue order (nothing crosses a sched_barrier): after each MFMA one of the
+      // next k-step's fragment reads or one load of the next stage goes out while it runs.
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (j == 0 && ks + 1 < KSTEPS)
+            af[nxt][i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * 128 + c);
+          if (j == 1 && ks + 1 < KSTEPS && i < TN)
+            bfr[nxt][i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * 128 + c);
+          // The whole next stage is requested during the first two k-steps, so that its latency
+          // (about a microsecond when the lines come from beyond L2) hides under the other two.
+          if (ks < 2 && (j & 1)) issue_one(nst, kn, ks * INST + i * (TN / 2) + (j >> 1));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  }
+
+  wait_vmcnt<0>();   // the last iteration's idle fetch must land before LDS is reused
+  block_barrier();   // every wave is done reading the stages
+
+  // Output through LDS: a wave lays its 128 x (32 TN) tile out row-major (rows padded by 16 bytes,
+  // which spreads both the 8-byte writes below and the 16-byte reads over all banks) and stores
+  // whole 16-byte pieces, so a row of the tile leaves as one contiguous segment.
+  // acc[i][j][e]: row fr of A tile i, column 8*(e/4) + 4*kh + e%4 of B tile j.
+  constexpr int ROWB = BIG_OUT_ROW_BYTES(TN);
+  char* ot = smem_big + wave * (128 * ROWB);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<uint2*>(ot + (i * 32 + fr) * ROWB + (j * 32 + 8 * q + 4 * kh) * 2) =
+            make_uint2(pack_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
+                       pack_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
+  // The tile is private to the wave, whose LDS operations execute in order: no block barrier,
+  // only a fence to keep the compiler from moving the reads above other lanes' writes.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  constexpr int LPRW = TN * 4;        // lanes (16 bytes each) per tile row
+  constexpr int RPI = 64 / LPRW;      // rows per instruction
+  const int lr = lane / LPRW, lc = lane % LPRW;
+  bf16_t* cbase = C + (size_t)(m0 + wm * 128) * N + n0 + wn * TN * 32 + lc * 8;
+#pragma unroll 4
+  for (int r0 = 0; r0 < 128; r0 += RPI) {
+    const int r = r0 + lr;
+    const uint4 v = *reinterpret_cast<const uint4*>(ot + r * ROWB + lc * 16);
+    if (m0 + wm * 128 + r < Mv) *reinterpret_cast<uint4*>(cbase + (size_t)r * N) = v;
+  }
+}
+
+static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
+                             const int* valid, hipStream_t s) {
+  const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
+  constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
+  const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt256_kernel<BIG_WAVES>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
+  hipLaunchKernelGGL(gemm_nt256_kernel<BIG_WAVES>, dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
+                     tiles_m, tiles_n, patched);
+  IRON_LAUNCH_CHECK();
+}
+
 }  // namespace iron
 
 using namespace iron;
@@ -513,6 +728,10 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
                "gemm: N (%d) must be a multiple of 8 when B is (K,N) (16-byte loads along N)", N);
   hipStream_t s = (hipStream_t)stream;
   if (!c_col_maj && valid_k == nullptr && K % BK == 0 && M >= 64 && N >= 64) {
+    // Enough whole 256x256 tiles to fill the chip: the large-tile kernel (offsets are 32-bit).
+    if (b_col_maj && M % BIG_BM == 0 && N % BIG_BN == 0 && (long)(M / BIG_BM) * (N / BIG_BN) >= 192 &&
+        K <= (1 << 24))
+      return launch_gemm_nt256(A, B, C, M, N, K, valid, s);
     if (b_col_maj) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s);
     // (K,N) B is read in whole 128-column tiles straight into LDS: N must be whole tiles.
     if (N % NT_BN == 0) return launch_gemm_nt<true>(A, B, C, M, N, K, valid, s);

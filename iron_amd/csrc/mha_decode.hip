@@ -14,38 +14,29 @@
 namespace iron {
 
 constexpr int kMaxSplits = 128;
+constexpr int kSingleMaxKeys = 2048;  // caches up to this many rows take the one-launch kernel
 
-template <int D, int G>
-__global__ __launch_bounds__(256) void mha_decode_kernel(
-    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
-    float* __restrict__ part, int kv_len, float scale_log2, int window, long row_stride,
-    long head_stride, const int* __restrict__ kv_valid) {
+// One wave's pass over key rows base + u*RW + rg for base = lo, lo + stride, ... while < hi, for
+// the G query heads q0.. of one KV head, then the merge of the wave's lane groups: on return every
+// lane holds the wave's (m, l) per head and acc = its 8 columns sub*8.. of the weighted V sum.
+template <int D, int G, int U>
+__device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const bf16_t* __restrict__ Kh,
+                                            const bf16_t* __restrict__ Vh, int q0, int lo, int hi,
+                                            int stride, long row_stride, float scale_log2,
+                                            float (&m)[G], float (&l)[G], float (&acc)[G][8]) {
   constexpr int LPR = D / 8;     // lanes per key row
   constexpr int RW = 64 / LPR;   // rows a wave covers per step
-  constexpr int U = 4;           // steps in flight
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;   // U = steps in flight
   const int sub = lane % LPR, rg = lane / LPR;
-  const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y;
-
-  const int kv_tokens = bound_or(kv_valid, kv_len);
-  const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
-  const int n = kv_tokens - first;
-  // Slice of this block, in whole wave-steps so that waves split it evenly.
-  int chunk = (n + nsplit - 1) / nsplit;
-  chunk = (chunk + 4 * RW - 1) / (4 * RW) * (4 * RW);
-  const int blo = first + split * chunk;
-  const int wlo = blo + wave * (chunk / 4);
-  const int whi = min(min(wlo + chunk / 4, blo + chunk), kv_tokens);
 
   float qf[G][8];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     float t[8];
-    unpack8(*reinterpret_cast<const uint4*>(Q + (size_t)(kvh * G + g) * D + sub * 8), t);
+    unpack8(*reinterpret_cast<const uint4*>(Q + (size_t)(q0 + g) * D + sub * 8), t);
 #pragma unroll
     for (int i = 0; i < 8; ++i) qf[g][i] = t[i] * scale_log2;
   }
-  float m[G], l[G], acc[G][8];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     m[g] = -INFINITY;
@@ -53,18 +44,17 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
   }
+  Kh += sub * 8;
+  Vh += sub * 8;
 
-  const bf16_t* Kh = K + (size_t)kvh * head_stride + sub * 8;
-  const bf16_t* Vh = V + (size_t)kvh * head_stride + sub * 8;
-
-  for (int base = wlo; base < whi; base += U * RW) {
+  for (int base = lo; base < hi; base += stride) {
     uint4 kv[U], vv[U];
     bool live[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int r = base + u * RW + rg;
-      live[u] = r < whi;
-      const size_t off = (size_t)(live[u] ? r : (whi - 1)) * row_stride;
+      live[u] = r < hi;
+      const size_t off = (size_t)(live[u] ? r : (hi - 1)) * row_stride;
       kv[u] = load_stream(reinterpret_cast<const uint4*>(Kh + off));
       vv[u] = load_stream(reinterpret_cast<const uint4*>(Vh + off));
     }
@@ -119,11 +109,11 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
 #pragma unroll
     for (int o = LPR; o < 64; o <<= 1) {
       const float mo = __shfl_xor(m[g], o, 64);
-      const float lo = __shfl_xor(l[g], o, 64);
+      const float lo2 = __shfl_xor(l[g], o, 64);
       const float mx = fmaxf(m[g], mo);
       const float ref = (mx == -INFINITY) ? 0.f : mx;
       const float a = exp2f(m[g] - ref), b = exp2f(mo - ref);
-      l[g] = l[g] * a + lo * b;
+      l[g] = l[g] * a + lo2 * b;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const float ao = __shfl_xor(acc[g][i], o, 64);
@@ -132,6 +122,31 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
       m[g] = mx;
     }
   }
+}
+
+template <int D, int G>
+__global__ __launch_bounds__(256) void mha_decode_kernel(
+    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
+    float* __restrict__ part, int kv_len, float scale_log2, int window, long row_stride,
+    long head_stride, const int* __restrict__ kv_valid) {
+  constexpr int LPR = D / 8, RW = 64 / LPR;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPR, rg = lane / LPR;
+  const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y;
+
+  const int kv_tokens = bound_or(kv_valid, kv_len);
+  const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
+  const int n = kv_tokens - first;
+  // Slice of this block, in whole wave-steps so that waves split it evenly.
+  int chunk = (n + nsplit - 1) / nsplit;
+  chunk = (chunk + 4 * RW - 1) / (4 * RW) * (4 * RW);
+  const int blo = first + split * chunk;
+  const int wlo = blo + wave * (chunk / 4);
+  const int whi = min(min(wlo + chunk / 4, blo + chunk), kv_tokens);
+
+  float m[G], l[G], acc[G][8];
+  decode_scan<D, G, 4>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, kvh * G, wlo, whi,
+                    4 * RW, row_stride, scale_log2, m, l, acc);
 
   // Merge the 4 waves through LDS; wave 0 writes the block's partial.
   __shared__ float sm[4][G];
@@ -205,6 +220,56 @@ __global__ void mha_decode_merge_kernel(const float* __restrict__ part, bf16_t* 
   }
 }
 
+// Short caches: one block of 16 waves per query head scans the whole cache (wave w takes every
+// 16th run of 8 steps), merges its waves through LDS and writes the output row itself -- one
+// launch, no partials.  Blocks b and b + kv_heads serve the same KV head; with kv_heads a multiple
+// of 8 they sit on one XCD and share its L2.
+template <int D>
+__global__ __launch_bounds__(1024) void mha_decode_single_kernel(
+    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
+    bf16_t* __restrict__ O, int kv_len, int kv_heads, int group, float scale_log2, int window,
+    long row_stride, long head_stride, const int* __restrict__ kv_valid) {
+  constexpr int LPR = D / 8, RW = 64 / LPR, WAVES = 16, U = 8;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPR, rg = lane / LPR;
+  const int kvh = blockIdx.x % kv_heads, head = kvh * group + blockIdx.x / kv_heads;
+
+  const int kv_tokens = bound_or(kv_valid, kv_len);
+  const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
+
+  float m[1], l[1], acc[1][8];
+  decode_scan<D, 1, U>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, head,
+                    first + wave * U * RW, kv_tokens, WAVES * U * RW, row_stride, scale_log2, m, l, acc);
+
+  __shared__ float sm[WAVES];
+  __shared__ float sl[WAVES];
+  __shared__ float sacc[WAVES][D];
+  if (rg == 0) {
+    if (sub == 0) {
+      sm[wave] = m[0];
+      sl[wave] = l[0];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sacc[wave][sub * 8 + i] = acc[0][i];
+  }
+  __syncthreads();
+  if (threadIdx.x < D) {
+    const int dd = threadIdx.x;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, sm[w]);
+    const float ref = (mx == -INFINITY) ? 0.f : mx;
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float e = exp2f(sm[w] - ref);
+      lt += sl[w] * e;
+      at += sacc[w][dd] * e;
+    }
+    O[(size_t)head * D + dd] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
+  }
+}
+
 template <int D, int G>
 static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, float* part,
                           int kv_heads, int kv_len, float scale_log2, int window, long row_stride,
@@ -245,6 +310,20 @@ extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const 
   const float scale_log2 = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
   float* part = (float*)workspace;
+  // Caches this short are launch-bound: one launch that needs no merge of splits.
+  if (kv_len <= kSingleMaxKeys && (d == 64 || d == 128 || d == 256)) {
+    const dim3 grid(heads), block(1024);
+    if (d == 64)
+      hipLaunchKernelGGL(mha_decode_single_kernel<64>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
+                         scale_log2, window, row_stride, head_stride, kv_valid);
+    else if (d == 128)
+      hipLaunchKernelGGL(mha_decode_single_kernel<128>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
+                         scale_log2, window, row_stride, head_stride, kv_valid);
+    else
+      hipLaunchKernelGGL(mha_decode_single_kernel<256>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
+                         scale_log2, window, row_stride, head_stride, kv_valid);
+    IRON_LAUNCH_CHECK();
+  }
 #define IRON_DEC(DD, GG)                                                                        \
   if (d == DD && G == GG) {                                                                     \
     launch_decode<DD, GG>(Q, K, V, O, part, kv_heads, kv_len, scale_log2, window, row_stride,   \

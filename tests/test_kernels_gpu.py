@@ -121,6 +121,25 @@ def test_gemm_ragged_shapes(cuda, M, Kdim, N, b_col_maj):
     close(C, ops.gemm(A, B, b_col_maj=b_col_maj), rtol=1e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("M,Kdim,N,rows", [(2048, 512, 8192, None), (2048, 64, 6144, None), (4096, 192, 4096, 1000),
+                                           (128, 64, 128, None), (256, 128, 192, None)])
+def test_gemm_weight_layout_fast_paths(cuda, M, Kdim, N, rows):
+    """B (N,K): the 256x256-tile kernel (>= 192 whole tiles) and the 128x128 one, down to a single
+    k stage, with a row bound that cuts through a tile."""
+    rng = np.random.default_rng(55)
+    A, B = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.1)
+    want = ops.gemm(A, B, b_col_maj=True)
+    if rows is not None:
+        A[rows:] = np.nan
+    C = out_like((M, N), cuda, fill=5.0)
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=M, N=N, K=Kdim, b_col_maj=True,
+           valid=None if rows is None else word(rows, cuda))
+    got = from_torch(C)
+    lim = M if rows is None else rows
+    close(got[:lim], want[:lim], rtol=1e-2, atol=2e-2)
+    assert np.all(got[lim:] == 5.0)
+
+
 @pytest.mark.parametrize("b_col_maj", [False, True])
 def test_gemm_bounded_rows_and_k_do_not_read_the_poison(cuda, b_col_maj):
     """NaN past the bounds must not reach the output (test_gemm_bounded_k.py)."""
@@ -293,9 +312,9 @@ def test_mha_decode_llama_shape(cuda, L):
 
 @pytest.mark.parametrize("H,G,d", [(32, 8, 64), (8, 8, 64), (24, 8, 128), (40, 8, 64), (4, 1, 256), (16, 8, 64), (12, 2, 64), (3, 1, 64)])
 @pytest.mark.parametrize("kv_valid,window", [(1, None), (77, None), (700, None), (700, 99), (2048, 511)])
-def test_mha_decode_bounds_windows_groups(cuda, H, G, d, kv_valid, window):
+@pytest.mark.parametrize("L", [2048, 4096])  # the one-launch kernel, and the split one with its merge
+def test_mha_decode_bounds_windows_groups(cuda, H, G, d, kv_valid, window, L):
     rng = np.random.default_rng(16)
-    L = 2048
     for interleaved in (True, False):
         ks = (L, G, d) if interleaved else (G, L, d)
         Q, Kc, Vc = bf(rng, 1, H, d), bf(rng, *ks), bf(rng, *ks)
