@@ -301,6 +301,29 @@ constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK
 
 typedef short short4v __attribute__((ext_vector_type(4)));
 
+// The transposing LDS read, as inline assembly: through the builtin the compiler cannot tell the
+// read from the direct-to-LDS loads in flight and waits for all of them (vmcnt(0)) before each
+// one, which drains the prefetch.  The compiler does not count these reads, so their consumer
+// must pass the results through lds_tr_wait() first.
+__device__ __forceinline__ short4v lds_read_tr16(unsigned lds_addr) {
+  short4v v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(lds_addr));
+  return v;
+}
+struct TrFrag {   // the two halves of a fragment, as the reads deliver them
+  short4v lo, hi;
+};
+// Waits for every LDS read issued so far; the halves pass through it so that nothing derived from
+// them (not even a register copy) can be scheduled before the wait.
+__device__ __forceinline__ void lds_tr_wait(TrFrag& a, TrFrag& b) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi));
+}
+__device__ __forceinline__ bf16x8 tr_join(const TrFrag& f) {
+  typedef short short8v __attribute__((ext_vector_type(8)));
+  const short8v both = __builtin_shufflevector(f.lo, f.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, both);
+}
+
 // B_KN: B is (K,N) row-major.  Its tile lands in LDS as stored, [64 k][128 n] (a wave
 // instruction moves 4 k-rows x 256 B, chunks swizzled by 2*(k & 7)), and the fragments are
 // fetched with the transposing LDS read (ds_read_b64_tr_b16): within 16 lanes, lane i points
@@ -405,7 +428,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
           IRON_GLOBAL_PTR(b_src[idx - INST] + (B_KN ? (size_t)k0 * N : (size_t)k0)),
           IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
   };
-  auto read_frag_pair = [&](const char* st, int ks, int i, bf16x8& a, bf16x8& b) {
+  auto read_frag_pair = [&](const char* st, int ks, int i, bf16x8& a, bf16x8& b, TrFrag& t) {
     const int j = ks * 2 + kh;
     a = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
     if constexpr (!B_KN) {
@@ -415,18 +438,14 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
       const int c0 = ((tr_n[i] >> 3) ^ ((k & 7) << 1)) << 4;
       const int c1 = ((tr_n[i] >> 3) ^ (((k + 4) & 7) << 1)) << 4;
       const int half = (tr_n[i] & 4) << 1;
-      const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + k * 256 + c0 + half));
-      const short4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (short4v __attribute__((address_space(3)))*)(st + NT_A_BYTES + (k + 4) * 256 + c1 + half));
-      typedef short short8v __attribute__((ext_vector_type(8)));
-      const short8v both = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
-      b = __builtin_bit_cast(bf16x8, both);
+      const unsigned base = (unsigned)(size_t)IRON_LDS_PTR(st + NT_A_BYTES + half);
+      t.lo = lds_read_tr16(base + k * 256 + c0);
+      t.hi = lds_read_tr16(base + (k + 4) * 256 + c1);
     }
   };
-  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[2], bf16x8 (&bfr)[2]) {
+  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[2], bf16x8 (&bfr)[2], TrFrag (&tf)[2]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) read_frag_pair(st, ks, i, af[i], bfr[i]);
+    for (int i = 0; i < 2; ++i) read_frag_pair(st, ks, i, af[i], bfr[i], tf[i]);
   };
   // A wave is alone on its SIMD, so nothing overlaps unless its own instruction stream interleaves:
   // each k-step's four MFMAs are issued with the next step's fragment reads and a quarter of the
@@ -442,17 +461,23 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
     const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
     bf16x8 af[2][2], bfr[2][2];
-    read_frags(st, 0, af[0], bfr[0]);
+    TrFrag tf[2][2];
+    read_frags(st, 0, af[0], bfr[0], tf[0]);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
+      if constexpr (B_KN) {
+        lds_tr_wait(tf[cur][0], tf[cur][1]);
+        bfr[cur][0] = tr_join(tf[cur][0]);
+        bfr[cur][1] = tr_join(tf[cur][1]);
+      }
       // Source order is issue order (nothing crosses a sched_barrier): while an MFMA runs, half of
       // the next k-step's fragment reads or one prefetch load goes out.
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][i], acc[i][0], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (ks + 1 < BK / 16) read_frag_pair(st, ks + 1, i, af[nxt][i], bfr[nxt][i]);
+        if (ks + 1 < BK / 16) read_frag_pair(st, ks + 1, i, af[nxt][i], bfr[nxt][i], tf[nxt][i]);
         __builtin_amdgcn_sched_barrier(0);
         acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][1], af[cur][i], acc[i][1], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
