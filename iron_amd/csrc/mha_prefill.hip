@@ -18,8 +18,11 @@ namespace iron {
 constexpr int BQ = 128;   // query rows per block
 constexpr int BKV = 64;   // key rows per tile
 
+// At least two waves a SIMD caps the register budget at 256, which makes the compiler keep MFMA
+// accumulators in ordinary VGPRs: the softmax reads S and rescales O in place instead of copying
+// every value out of (and back into) accumulation registers.
 template <int D>
-__global__ __launch_bounds__(256) void mha_prefill_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -203,10 +206,13 @@ __global__ __launch_bounds__(256) void mha_prefill_kernel(
           pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
         }
       l_run = l_run * alpha + rsum;
+      // After the first tiles a new maximum is rare: rescale O only when some query's moved.
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
-      for (int t = 0; t < DT; ++t)
+        for (int t = 0; t < DT; ++t)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
+          for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
+      }
 
       // O^T += V^T P^T.  k slots of lane group g at (t, h): keys 32 t + 16 h + 4 g + 0..3 and the same + 8.
 #pragma unroll
