@@ -125,4 +125,46 @@ __device__ __forceinline__ int bound_or(const int* p, int whole) {
   return v < 0 ? 0 : (v > whole ? whole : v);
 }
 
+// ---- direct-to-LDS pipelines
+#define IRON_GLOBAL_PTR(p) ((const void __attribute__((address_space(1)))*)(p))
+#define IRON_LDS_PTR(p) ((void __attribute__((address_space(3)))*)(p))
+
+__device__ __forceinline__ void block_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // gfx9 encoding: vmcnt = bits [3:0] and [15:14]; expcnt and lgkmcnt left at "no wait".
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+// The transposing LDS read, as inline assembly: through the builtin the compiler cannot tell the
+// read from the direct-to-LDS loads in flight and waits for all of them (vmcnt(0)) before each
+// one, which drains the prefetch.  The compiler does not count these reads, so their consumer
+// must pass the results through lds_tr_wait() first.
+__device__ __forceinline__ short4v lds_read_tr16(unsigned lds_addr) {
+  short4v v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(lds_addr));
+  return v;
+}
+struct TrFrag {   // the two halves of a fragment, as the reads deliver them
+  short4v lo, hi;
+};
+// Waits for every LDS read issued so far; the halves pass through it so that nothing derived from
+// them (not even a register copy) can be scheduled before the wait.
+__device__ __forceinline__ void lds_tr_wait(TrFrag& a, TrFrag& b) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.lo), "+v"(a.hi), "+v"(b.lo), "+v"(b.hi));
+}
+__device__ __forceinline__ bf16x8 tr_join(const TrFrag& f) {
+  typedef short short8v __attribute__((ext_vector_type(8)));
+  const short8v both = __builtin_shufflevector(f.lo, f.hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, both);
+}
+
+
 }  // namespace iron

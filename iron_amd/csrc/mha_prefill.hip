@@ -7,9 +7,9 @@
 // rows.  The wave computes the TRANSPOSED score tile S^T = K Q^T (M = keys,
 // N = queries): a lane then owns one query column, so the row max / row sum of
 // the online softmax are in-lane reductions plus one exchange with lane^32, and
-// the probabilities are already laid out as the B operand of O^T = V^T P^T.  V is
-// transposed on its way into LDS so its fragments are k-contiguous.  All softmax
-// state is f32 in the exp2 domain.
+// the probabilities are already laid out as the B operand of O^T = V^T P^T.  V^T
+// fragments come from the transposing LDS read.  All softmax state is f32 in the
+// exp2 domain.
 #include "../../include/iron_hip.h"
 #include "common.h"
 
@@ -18,6 +18,12 @@ namespace iron {
 constexpr int BQ = 128;   // query rows per block
 constexpr int BKV = 64;   // key rows per tile
 
+// K and V tiles go straight from global memory into LDS (global_load_lds, no register staging), as
+// stored: [64 keys][D], STAGES tiles deep.  16-byte chunks of a row are XOR-swizzled so unpadded
+// rows read without bank conflicts: K by (key >> 1) & 7 for its 16-byte fragment reads, V by
+// 2 * (key & 3) for the transposing reads (ds_read_b64_tr_b16) that deliver V^T fragments.  A bare
+// s_barrier and counted s_waitcnt vmcnt keep the younger tiles' loads in flight across the barrier.
+//
 // At least two waves a SIMD caps the register budget at 256, which makes the compiler keep MFMA
 // accumulators in ordinary VGPRs: the softmax reads S and rescales O in place instead of copying
 // every value out of (and back into) accumulation registers.
@@ -27,15 +33,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     bf16_t* __restrict__ O, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
     long kv_head_stride, const int* __restrict__ valid, const int* __restrict__ kv_valid) {
-  constexpr int LDK = D + 8;     // K tile row (elements)
-  constexpr int LDV = BKV + 8;   // V^T tile row
-  constexpr int KS = D / 16;     // k16 steps of S^T
-  constexpr int DT = D / 32;     // 32-row tiles of O^T
-  constexpr int CPR = D / 8;     // 16-byte chunks a key row has
-  constexpr int NL = BKV * CPR / 256;   // 16-byte loads a thread makes of K (and of V) per tile
-  constexpr int K_TILE = BKV * LDK, V_TILE = D * LDV;
-  __shared__ __align__(16) bf16_t Ks[2 * K_TILE];
-  __shared__ __align__(16) bf16_t Vt[2 * V_TILE];
+  constexpr int ROWB = D * 2;            // bytes of a tile row
+  constexpr int KS = D / 16;             // k16 steps of S^T
+  constexpr int DT = D / 32;             // 32-row tiles of O^T
+  constexpr int CPR = D / 8;             // 16-byte chunks a row has
+  constexpr int STAGES = D == 64 ? 3 : 2;
+  constexpr int TILE = BKV * ROWB;       // bytes of a K (or V) tile
+  constexpr int STAGE = 2 * TILE;
+  constexpr int INST = TILE / 1024 / 4;  // 1 KB loads of K (and of V) a wave issues per tile
+  constexpr int RPI = 1024 / ROWB;       // rows one load covers
+  __shared__ __align__(1024) char smem[STAGES * STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, g = lane >> 5;
@@ -91,145 +98,155 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
   else if (window >= 0) kv_hi = min(kv_hi, offset + q_last + window + 1);
   int kv_lo = 0;
   if (window >= 0) kv_lo = max(0, offset + q0 - window) / BKV * BKV;
+  const int ntiles = (kv_hi - kv_lo + BKV - 1) / BKV;
 
-  const bf16_t* Kh = K + (size_t)kvh * kv_head_stride;
-  const bf16_t* Vh = V + (size_t)kvh * kv_head_stride;
+  if (ntiles > 0) {
+    const bf16_t* Kh = K + (size_t)kvh * kv_head_stride;
+    const bf16_t* Vh = V + (size_t)kvh * kv_head_stride;
 
-  // Tile staging: K as stored; V two keys a load pair, transposed on the way into LDS.
-  uint4 kreg[NL], vreg[NL];
-  auto fetch = [&](int kv0) {
+    // Loader: load i of a wave covers tile rows (wave*INST + i)*RPI .. ; lane -> (row, physical
+    // chunk), and fetches the logical chunk that the row's swizzle maps there.  Rows past the
+    // last key re-read it: finite values that the mask below turns into zero weights.
+    const int l_row = lane / CPR, l_pch = lane % CPR;
+    int k_row[INST], k_col[INST], v_col[INST];
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int p = tid + i * 256;
-      const int r = p / CPR, c = (p % CPR) * 8;
-      kreg[i] = (kv0 + r < kv_tokens) ? *reinterpret_cast<const uint4*>(Kh + (size_t)(kv0 + r) * kv_row_stride + c)
-                                      : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < INST; ++i) {
+      const int r = (wave * INST + i) * RPI + l_row;
+      k_row[i] = r;
+      k_col[i] = (l_pch ^ ((r >> 1) & 7)) * 8;
+      v_col[i] = (l_pch ^ ((r & 3) << 1)) * 8;
     }
+    auto issue = [&](int tile, int buf) {
+      char* st = smem + buf * STAGE;
+      const int kv0 = kv_lo + tile * BKV;
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      // load i is key 2*pair + (i & 1) of strip `tid % CPR`, pair = tid / CPR + (i / 2) * (256 / CPR)
-      const int strip = tid % CPR, key = 2 * (tid / CPR + (i >> 1) * (256 / CPR)) + (i & 1);
-      vreg[i] = (kv0 + key < kv_tokens) ? *reinterpret_cast<const uint4*>(Vh + (size_t)(kv0 + key) * kv_row_stride + strip * 8)
-                                        : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto stage = [&](int buf) {
-    bf16_t* kd = Ks + buf * K_TILE;
-    bf16_t* vd = Vt + buf * V_TILE;
-#pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int p = tid + i * 256;
-      *reinterpret_cast<uint4*>(kd + (p / CPR) * LDK + (p % CPR) * 8) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < NL; i += 2) {
-      const int strip = tid % CPR, key = 2 * (tid / CPR + (i >> 1) * (256 / CPR));
-      const uint32_t a[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
-      const uint32_t b[4] = {vreg[i + 1].x, vreg[i + 1].y, vreg[i + 1].z, vreg[i + 1].w};
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-        *reinterpret_cast<uint32_t*>(vd + (strip * 8 + c) * LDV + key) = __builtin_amdgcn_perm(b[c >> 1], a[c >> 1], sel);
+      for (int i = 0; i < INST; ++i) {
+        const size_t row = (size_t)min(kv0 + k_row[i], kv_tokens - 1) * kv_row_stride;
+        __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(Kh + row + k_col[i]),
+                                         IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(Vh + row + v_col[i]),
+                                         IRON_LDS_PTR(st + TILE + (wave * INST + i) * 1024), 16, 0, 0);
       }
+    };
+    // Always STAGES-1 tiles in flight before the loop and one more each iteration (past the end
+    // the last tile again, into a buffer nobody reads), so the wait counts below are exact.
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue(min(s, ntiles - 1), s);
+
+    // Fragment addressing.  K (A operand of S^T): lane reads key t*32 + col, chunk 2s + g.
+    const int k_frag = col * ROWB, k_swz = (col >> 1) & 7;
+    // V^T (A operand of O^T): for (t, h) a lane group g needs keys 32t + 16h + 4g + 0..3 (low
+    // half of its k slots) and the same + 8 (high half) of column d = 32 dt + col.  In the
+    // transposing read a lane points at 4 consecutive d of the key row 4g + (lane & 15) / 4 ...
+    const int v_key = 4 * g + ((lane & 15) >> 2);
+    const int v_swz = ((lane >> 2) & 3) << 1;           // 2 * (key & 3), the same for every (t, h)
+    int v_frag[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int chunk = dt * 4 + (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);
+      v_frag[dt] = v_key * ROWB + ((chunk ^ v_swz) << 4) + ((lane & 1) << 3);
     }
-  };
+    const unsigned lds_base = (unsigned)(size_t)IRON_LDS_PTR(smem);
 
-  if (kv_lo < kv_hi) {
-    fetch(kv_lo);
-    stage(0);
-  }
-  __syncthreads();
+    for (int tile = 0; tile < ntiles; ++tile) {
+      const int kv0 = kv_lo + tile * BKV;
+      wait_vmcnt<(STAGES - 2) * 2 * INST>();   // this wave's share of the tile has landed
+      block_barrier();                          // everyone's has; everyone is done with tile - 1
+      issue(min(tile + STAGES - 1, ntiles - 1), (tile + STAGES - 1) % STAGES);
+      const int buf = tile % STAGES;
 
-  int buf = 0;
-  for (int kv0 = kv_lo; kv0 < kv_hi; kv0 += BKV, buf ^= 1) {
-    const bool more = kv0 + BKV < kv_hi;
-    if (more) fetch(kv0 + BKV);   // in flight during this tile's MFMAs
-
-    // Tiles wholly above the wave's last query (causal) hold nothing for it.
-    const bool skip = causal && kv0 > wq_hi;
-    if (!skip) {
-      const bf16_t* kt = Ks + buf * K_TILE;
-      const bf16_t* vt = Vt + buf * V_TILE;
-      // S^T = K Q^T for the two 32-key halves of the tile.
-      f32x16 sacc[2];
+      // Tiles wholly above the wave's last query (causal) hold nothing for it.
+      const bool skip = causal && kv0 > wq_hi;
+      if (!skip) {
+        const char* kt = smem + buf * STAGE;
+        const unsigned vt = lds_base + buf * STAGE + TILE;
+        // S^T = K Q^T for the two 32-key halves of the tile.
+        f32x16 sacc[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
+          for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kt + (t * 32 + col) * LDK + 16 * s + 8 * g);
-          sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[t], 0, 0, 0);
+          for (int s = 0; s < KS; ++s) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kt + t * 32 * ROWB + k_frag + (((2 * s + g) ^ k_swz) << 4));
+            sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[t], 0, 0, 0);
+          }
         }
-      }
-      // Only tiles that touch a bound or the mask's edge pay for masking.  Element e of half t
-      // is key kv0 + 32 t + 8 (e/4) + 4 g + e%4, query `col`.
-      bool edge = kv0 + BKV > kv_tokens;
-      if (causal) edge |= kv0 + BKV - 1 > wq_lo;
-      else if (window >= 0) edge |= kv0 + BKV - 1 > wq_lo + window;
-      if (window >= 0) edge |= kv0 < wq_hi - window;
-      if (edge) {
+        // Only tiles that touch a bound or the mask's edge pay for masking.  Element e of half t
+        // is key kv0 + 32 t + 8 (e/4) + 4 g + e%4, query `col`.
+        bool edge = kv0 + BKV > kv_tokens;
+        if (causal) edge |= kv0 + BKV - 1 > wq_lo;
+        else if (window >= 0) edge |= kv0 + BKV - 1 > wq_lo + window;
+        if (window >= 0) edge |= kv0 < wq_hi - window;
+        if (edge) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const int kpos = kv0 + 32 * t + 8 * (e >> 2) + 4 * g + (e & 3);
+              bool dead = kpos >= kv_tokens;
+              if (causal) dead |= kpos > qpos;
+              else if (window >= 0) dead |= kpos > qpos + window;
+              if (window >= 0) dead |= kpos < qpos - window;
+              sacc[t][e] = dead ? -INFINITY : sacc[t][e];
+            }
+        }
+        float rmax = sacc[0][0];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int kpos = kv0 + 32 * t + 8 * (e >> 2) + 4 * g + (e & 3);
-            bool dead = kpos >= kv_tokens;
-            if (causal) dead |= kpos > qpos;
-            else if (window >= 0) dead |= kpos > qpos + window;
-            if (window >= 0) dead |= kpos < qpos - window;
-            if (dead) sacc[t][e] = -INFINITY;
-          }
-      }
-      float rmax = sacc[0][0];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
-      const float m_new = fmaxf(m_run, rmax);
-      const float mc = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
-      const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc));  // exp2(-inf) = 0 at the start
-      m_run = m_new;
-      float rsum = 0.f;
-      bf16x8 pf[2][2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          float p[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            p[j] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * h + j], scale_log2, -mc));
-            rsum += p[j];
-          }
-          pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
-        }
-      l_run = l_run * alpha + rsum;
-      // After the first tiles a new maximum is rare: rescale O only when some query's moved.
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
-      }
-
-      // O^T += V^T P^T.  k slots of lane group g at (t, h): keys 32 t + 16 h + 4 g + 0..3 and the same + 8.
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+          for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
+        const float m_new = fmaxf(m_run, rmax);
+        const float mc = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
+        const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc));  // exp2(-inf) = 0 at the start
+        m_run = m_new;
+        float rsum = 0.f;
+        bf16x8 pf[2][2];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
-            const bf16_t* vp = vt + (dt * 32 + col) * LDV + 32 * t + 16 * h + 4 * g;
-            const uint2 lo = *reinterpret_cast<const uint2*>(vp);
-            const uint2 hi = *reinterpret_cast<const uint2*>(vp + 8);
-            const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[t][h], oacc[dt], 0, 0, 0);
+            float p[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              p[j] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * h + j], scale_log2, -mc));
+              rsum += p[j];
+            }
+            pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
           }
+        l_run = l_run * alpha + rsum;
+        // After the first tiles a new maximum is rare: rescale O only when some query's moved.
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+          for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
+        }
+
+        // O^T += V^T P^T, two (t, h) steps at a time so one wait covers a batch of reads.
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          TrFrag vf[DT][2];
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const unsigned a = vt + (32 * t + 16 * h) * ROWB + v_frag[dt];
+              vf[dt][h].lo = lds_read_tr16(a);
+              vf[dt][h].hi = lds_read_tr16(a + 8 * ROWB);
+            }
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            lds_tr_wait(vf[dt][0], vf[dt][1]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+              oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_join(vf[dt][h]), pf[t][h], oacc[dt], 0, 0, 0);
+          }
+        }
+      }
     }
-    if (more) stage(buf ^ 1);   // the other buffer: everyone finished reading it a tile ago
-    __syncthreads();
+    wait_vmcnt<0>();   // the idle fetches of the last iterations land before the block's LDS is released
   }
 
   // Normalize and store: lane holds query `col`, columns 32 dt + 8 q + 4 g + 0..3.
