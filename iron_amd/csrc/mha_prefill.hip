@@ -108,20 +108,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     // chunk), and fetches the logical chunk that the row's swizzle maps there.  Rows past the
     // last key re-read it: finite values that the mask below turns into zero weights.
     const int l_row = lane / CPR, l_pch = lane % CPR;
-    int k_row[INST], k_col[INST], v_col[INST];
+    // Per load: where tile 0's row starts (K and V share it), the same for the last tile with rows
+    // past the last key clamped to it, and the swizzled column of K and of V.
+    long row0[INST], row_last[INST];
+    int k_col[INST], v_col[INST];
 #pragma unroll
     for (int i = 0; i < INST; ++i) {
       const int r = (wave * INST + i) * RPI + l_row;
-      k_row[i] = r;
+      row0[i] = (long)(kv_lo + r) * kv_row_stride;
+      row_last[i] = (long)min(kv_lo + (ntiles - 1) * BKV + r, kv_tokens - 1) * kv_row_stride;
       k_col[i] = (l_pch ^ ((r >> 1) & 7)) * 8;
       v_col[i] = (l_pch ^ ((r & 3) << 1)) * 8;
     }
+    const long tile_stride = (long)BKV * kv_row_stride;
     auto issue = [&](int tile, int buf) {
       char* st = smem + buf * STAGE;
-      const int kv0 = kv_lo + tile * BKV;
+      const bool last = tile == ntiles - 1;   // only the last tile can hold rows past the last key
 #pragma unroll
       for (int i = 0; i < INST; ++i) {
-        const size_t row = (size_t)min(kv0 + k_row[i], kv_tokens - 1) * kv_row_stride;
+        const long row = last ? row_last[i] : row0[i] + tile * tile_stride;
         __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(Kh + row + k_col[i]),
                                          IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(Vh + row + v_col[i]),
@@ -152,12 +157,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
       const int kv0 = kv_lo + tile * BKV;
       wait_vmcnt<(STAGES - 2) * 2 * INST>();   // this wave's share of the tile has landed
       block_barrier();                          // everyone's has; everyone is done with tile - 1
-      issue(min(tile + STAGES - 1, ntiles - 1), (tile + STAGES - 1) % STAGES);
       const int buf = tile % STAGES;
-
-      // Tiles wholly above the wave's last query (causal) hold nothing for it.
-      const bool skip = causal && kv0 > wq_hi;
-      if (!skip) {
+      {
         const char* kt = smem + buf * STAGE;
         const unsigned vt = lds_base + buf * STAGE + TILE;
         // S^T = K Q^T for the two 32-key halves of the tile.
@@ -172,6 +173,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[t], 0, 0, 0);
           }
         }
+        // The prefetch goes out while the score MFMAs run (its buffer, tile - 1's, is free since
+        // the barrier above).
+        issue(min(tile + STAGES - 1, ntiles - 1), (tile + STAGES - 1) % STAGES);
         // Only tiles that touch a bound or the mask's edge pay for masking.  Element e of half t
         // is key kv0 + 32 t + 8 (e/4) + 4 g + e%4, query `col`.
         bool edge = kv0 + BKV > kv_tokens;
