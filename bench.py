@@ -86,6 +86,28 @@ def bench_gemm(torch, K, dev, steps, rng, b_col_maj, M=2048, N=2048, Kd=2048):
             "TFLOPs": round(flops / us / 1e6, 1), "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
+def bench_mfma_ceiling(torch, K, dev, rng):
+    """What the MFMA units sustain from registers alone: with constant operands, and with operands
+    drawn like the GEMM's (N(0,1)*0.02) -- under the power cap the clock depends on the data."""
+    from iron_amd.bf16 import round_bf16, to_torch
+
+    sink = torch.empty(K.PROBE_BLOCKS * 256, dtype=torch.float32, device=dev)
+    drawn = to_torch(round_bf16(rng.standard_normal(1 << 21, dtype=np.float32) * np.float32(0.02))).to(dev)
+    out = {}
+    for name, ops in (("constant", None), ("random", drawn)):
+        iters = 4000
+        flops = K.probe_mfma(ops, sink, iters)
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(3):
+            K.probe_mfma(ops, sink, iters)
+        stop.record()
+        stop.synchronize()
+        out[name] = round(3 * flops / (start.elapsed_time(stop) * 1e-3) / 1e12, 1)
+    return out
+
+
 def bench_attention(torch, K, dev, n, rng):
     """GQA causal attention, 32 q / 8 kv heads, d 64, scale 1/8: prefill at S = 512, 2048, 8192 (MFMA bound)
     and one query over caches of 1024, 4096, 16384 keys (HBM bound)."""
@@ -366,6 +388,9 @@ def main():
     gemm += [bench_gemm(torch, K, dev, max(20, n // 4), rng, True, M=m, N=nn, Kd=k)
              for m, nn, k in ((2048, 8192, 2048), (2048, 2048, 8192), (4096, 4096, 4096), (8192, 8192, 8192))]
     attention = bench_attention(torch, K, dev, n, rng)
+    mfma_ceiling = bench_mfma_ceiling(torch, K, dev, rng)
+    for g in gemm:
+        g["frac_sustained"] = round(g["TFLOPs"] / mfma_ceiling["random"], 4)
     pre_attention = bench_pre_attention(torch, K, dev, n)
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
@@ -400,6 +425,7 @@ def main():
         "decoder": decoder,
         "gemv_sweep": {"GBps": round(sweep_bytes / sweep_us / 1e3, 1), "shapes": gemv},
         "gemm": gemm,
+        "mfma_sustained_TFLOPs": mfma_ceiling,
         "attention": attention,
         "pre_attention_block": pre_attention,
         "bench_wall_s": round(wall, 1),

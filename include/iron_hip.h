@@ -148,6 +148,15 @@ int iron_argmax_bf16(const uint16_t* logits, int n, int* token, int* record, int
  * iron/common/graph/carried.py:189-276, iron/operators/emit.py. */
 int iron_eval_words(int* words, int n_words, const int* exprs, int n, void* stream);
 
+/* Measurement aid (no counterpart in the reference; bench.py's MFMA ceiling): IRON_PROBE_BLOCKS
+ * blocks of 4 waves run `iters` rounds of 16 independent 32x32x16 bf16 MFMAs from registers.
+ * operands: operand_count bf16 values the fragments are drawn from, or NULL for constants.
+ * sink: IRON_PROBE_BLOCKS*256 floats.  iron_probe_mfma_flops(iters) = flops of one launch. */
+#define IRON_PROBE_BLOCKS 512
+int iron_probe_mfma_bf16(const uint16_t* operands, int64_t operand_count, float* sink, int iters,
+                         void* stream);
+int64_t iron_probe_mfma_flops(int iters);
+
 #ifdef __cplusplus
 }
 #endif

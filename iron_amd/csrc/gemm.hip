@@ -528,18 +528,28 @@ constexpr int BIG_BM = 256, BIG_BN = 256;
 #define IRON_BIG_WAVES 4
 #endif
 constexpr int BIG_WAVES = IRON_BIG_WAVES;
+#ifndef IRON_BIG_KB
+#define IRON_BIG_KB 64
+#endif
+constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stages of half-line rows) measured 13 % slower
 #define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
 constexpr int BIG_A_BYTES = BIG_BM * BK * 2, BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
 
-template <int WAVES>
+template <int WAVES, int KB>
 __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
                                                          const bf16_t* __restrict__ B,
                                                          bf16_t* __restrict__ C, int M, int N, int K,
                                                          const int* __restrict__ valid, int tiles_m,
                                                          int tiles_n, int patched) {
-  constexpr int INST = BIG_BM / 8 / WAVES;   // 1 KB loads of A (and of B) a wave issues per stage
+  static_assert(KB == 64 || (KB == 32 && WAVES == 4), "k per stage: 64, or 32 with 4 waves");
+  constexpr int ROWB = KB * 2;               // bytes of a tile row in LDS
+  constexpr int CPR = KB / 8;                // its 16-byte chunks
+  constexpr int RPI = 1024 / ROWB;           // rows one 1 KB load covers
+  constexpr int A_BYTES = BIG_BM * ROWB, STAGE_BYTES = (BIG_BM + BIG_BN) * ROWB;
+  constexpr int STAGES = KB == 64 ? 2 : 4;   // 128 KB either way
+  constexpr int INST = BIG_BM / RPI / WAVES; // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int TN = 8 / WAVES * 2;          // 32-column MFMA tiles a wave owns along n (4 or 2)
-  constexpr int KSTEPS = BK / 16;
+  constexpr int KSTEPS = KB / 16;
   extern __shared__ __align__(16) char smem_big[];
   const int Mv = bound_or(valid, M);
 
@@ -563,27 +573,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / (WAVES / 2), wn = wave % (WAVES / 2);
-  // Loader: instruction i of a wave moves rows (wave*INST + i)*8 .. +7; lane -> (row, physical
+  // Loader: instruction i of a wave moves rows (wave*INST + i)*RPI .. ; lane -> (row, physical
   // chunk); the logical chunk it fetches is the physical one swizzled by the row.
-  const int lrow = lane >> 3, pch = lane & 7;
+  const int lrow = lane / CPR, pch = lane % CPR;
   unsigned ld_off[2];   // byte offset of this lane's 16 bytes within an even / odd instruction's rows
 #pragma unroll
   for (int par = 0; par < 2; ++par) {
-    const int r = par * 8 + lrow;
-    ld_off[par] = (unsigned)(((size_t)lrow * K + (pch ^ ((r >> 1) & 7)) * 8) * 2);
+    const int r = par * RPI + lrow;
+    ld_off[par] = (unsigned)(((size_t)lrow * K + (pch ^ ((r >> 1) & (CPR - 1))) * 8) * 2);
   }
-  const char* a_base = reinterpret_cast<const char*>(A + (size_t)(m0 + wave * INST * 8) * K);
-  const char* b_base = reinterpret_cast<const char*>(B + (size_t)(n0 + wave * INST * 8) * K);
-  const size_t inst_stride = (size_t)8 * K * 2;   // 8 rows
+  const char* a_base = reinterpret_cast<const char*>(A + (size_t)(m0 + wave * INST * RPI) * K);
+  const char* b_base = reinterpret_cast<const char*>(B + (size_t)(n0 + wave * INST * RPI) * K);
+  const size_t inst_stride = (size_t)RPI * K * 2;
   auto issue_one = [&](char* st, int kt, int idx) {
-    const size_t k_off = (size_t)kt * BK * 2;
+    const size_t k_off = (size_t)kt * KB * 2;
     if (idx < INST)
       __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_base + idx * inst_stride + k_off + ld_off[idx & 1]),
                                        IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16, 0, 0);
     else
       __builtin_amdgcn_global_load_lds(
           IRON_GLOBAL_PTR(b_base + (idx - INST) * inst_stride + k_off + ld_off[idx & 1]),
-          IRON_LDS_PTR(st + BIG_A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
+          IRON_LDS_PTR(st + A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
   };
 
   f32x16 acc[4][TN];
@@ -594,30 +604,34 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int nk = K / BK;
+  const int nk = K / KB;
+  // STAGES-1 stages in flight before the loop (short K repeats its last stage), one more each
+  // iteration: the wait count in the loop is exact from the first iteration.
 #pragma unroll
-  for (int idx = 0; idx < 2 * INST; ++idx) issue_one(smem_big, 0, idx);
+  for (int s = 0; s < STAGES - 1; ++s)
+#pragma unroll
+    for (int idx = 0; idx < 2 * INST; ++idx) issue_one(smem_big + s * STAGE_BYTES, min(s, nk - 1), idx);
 
   const int fr = lane & 31, kh = lane >> 5;
-  const int swz = (fr >> 1) & 7;   // tile rows are multiples of 32 apart: one swizzle for all
-  const int a_row = (wm * 128 + fr) * 128, b_row = BIG_A_BYTES + (wn * TN * 32 + fr) * 128;
+  const int swz = (fr >> 1) & (CPR - 1);   // tile rows are multiples of 32 apart: one swizzle for all
+  const int a_row = (wm * 128 + fr) * ROWB, b_row = A_BYTES + (wn * TN * 32 + fr) * ROWB;
   auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[4], bf16x8 (&bfr)[TN]) {
     const int c = ((ks * 2 + kh) ^ swz) << 4;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * 128 + c);
+    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * ROWB + c);
 #pragma unroll
-    for (int i = 0; i < TN; ++i) bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * 128 + c);
+    for (int i = 0; i < TN; ++i) bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * ROWB + c);
   };
 
   for (int kt = 0; kt < nk; ++kt) {
-    wait_vmcnt<0>();   // this wave's share of stage kt has landed
+    wait_vmcnt<(STAGES - 2) * 2 * INST>();   // this wave's share of stage kt has landed
     block_barrier();   // so has everyone's; and everyone is done reading stage kt-1
     // The next stage goes into the buffer stage kt-1 used.  The last iteration fetches its own
     // stage again (into the idle buffer) rather than branch: a branch would end the scheduling
     // region and undo the interleaving below.
-    const int kn = min(kt + 1, nk - 1);
-    char* nst = smem_big + ((kt + 1) & 1) * BIG_STAGE_BYTES;
-    const char* st = smem_big + (kt & 1) * BIG_STAGE_BYTES;
+    const int kn = min(kt + STAGES - 1, nk - 1);
+    char* nst = smem_big + ((kt + STAGES - 1) % STAGES) * STAGE_BYTES;
+    const char* st = smem_big + (kt % STAGES) * STAGE_BYTES;
     bf16x8 af[2][4], bfr[2][TN];
     read_frags(st, 0, af[0], bfr[0]);
 #pragma unroll
@@ -633,12 +647,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
           if (j == 0 && ks + 1 < KSTEPS)
-            af[nxt][i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * 128 + c);
+            af[nxt][i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * ROWB + c);
           if (j == 1 && ks + 1 < KSTEPS && i < TN)
-            bfr[nxt][i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * 128 + c);
+            bfr[nxt][i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * ROWB + c);
           // The whole next stage is requested during the first two k-steps, so that its latency
           // (about a microsecond when the lines come from beyond L2) hides under the other two.
-          if (ks < 2 && (j & 1)) issue_one(nst, kn, ks * INST + i * (TN / 2) + (j >> 1));
+          if (KB == 64 ? (ks < 2 && (j & 1)) : (j == 1))
+            issue_one(nst, kn, KB == 64 ? ks * INST + i * (TN / 2) + (j >> 1) : ks * INST + i);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -652,15 +667,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
   // which spreads both the 8-byte writes below and the 16-byte reads over all banks) and stores
   // whole 16-byte pieces, so a row of the tile leaves as one contiguous segment.
   // acc[i][j][e]: row fr of A tile i, column 8*(e/4) + 4*kh + e%4 of B tile j.
-  constexpr int ROWB = BIG_OUT_ROW_BYTES(TN);
-  char* ot = smem_big + wave * (128 * ROWB);
+  constexpr int OROWB = BIG_OUT_ROW_BYTES(TN);
+  char* ot = smem_big + wave * (128 * OROWB);
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<uint2*>(ot + (i * 32 + fr) * ROWB + (j * 32 + 8 * q + 4 * kh) * 2) =
+        *reinterpret_cast<uint2*>(ot + (i * 32 + fr) * OROWB + (j * 32 + 8 * q + 4 * kh) * 2) =
             make_uint2(pack_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
                        pack_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
   // The tile is private to the wave, whose LDS operations execute in order: no block barrier,
@@ -669,13 +684,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   constexpr int LPRW = TN * 4;        // lanes (16 bytes each) per tile row
-  constexpr int RPI = 64 / LPRW;      // rows per instruction
+  constexpr int ORPI = 64 / LPRW;     // rows per instruction
   const int lr = lane / LPRW, lc = lane % LPRW;
   bf16_t* cbase = C + (size_t)(m0 + wm * 128) * N + n0 + wn * TN * 32 + lc * 8;
 #pragma unroll 4
-  for (int r0 = 0; r0 < 128; r0 += RPI) {
+  for (int r0 = 0; r0 < 128; r0 += ORPI) {
     const int r = r0 + lr;
-    const uint4 v = *reinterpret_cast<const uint4*>(ot + r * ROWB + lc * 16);
+    const uint4 v = *reinterpret_cast<const uint4*>(ot + r * OROWB + lc * 16);
     if (m0 + wm * 128 + r < Mv) *reinterpret_cast<uint4*>(cbase + (size_t)r * N) = v;
   }
 }
@@ -687,13 +702,13 @@ static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M,
   const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt256_kernel<BIG_WAVES>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL(gemm_nt256_kernel<BIG_WAVES>, dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
+  hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
                      tiles_m, tiles_n, patched);
   IRON_LAUNCH_CHECK();
 }

@@ -268,3 +268,21 @@ def eval_words(words, exprs, n=None):
     _dev(exprs, "exprs", torch.int32)
     n = exprs.numel() // 7 if n is None else n
     check(lib().iron_eval_words(ptr(words), words.numel(), ptr(exprs), n, current_stream()), "iron_eval_words")
+
+
+PROBE_BLOCKS = 512
+
+
+def probe_mfma(operands, sink, iters):
+    """Launch the register-only MFMA loop (a measurement aid); returns the flops of the launch."""
+    if operands is not None:
+        _dev(operands, "operands", torch.bfloat16)
+    _dev(sink, "sink", torch.float32)
+    if sink.numel() < PROBE_BLOCKS * 256:
+        raise ValueError(f"sink: {sink.numel()} floats, {PROBE_BLOCKS * 256} needed")
+    check(
+        lib().iron_probe_mfma_bf16(ptr(operands), 0 if operands is None else operands.numel(), ptr(sink), iters,
+                                   current_stream()),
+        "iron_probe_mfma_bf16",
+    )
+    return lib().iron_probe_mfma_flops(iters)
