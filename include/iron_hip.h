@@ -97,6 +97,13 @@ int iron_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n, 
 int iron_silu_mul_bf16(const uint16_t* g, const uint16_t* u, uint16_t* y, int64_t n,
                        const int* valid, void* stream);
 
+/* y[r] = bf16(x[r] + row) (or x[r] * row if multiply) for r < *valid (or rows): one row met by
+ * every row, f32 math, one rounding.  x,y (rows, cols); row (cols).  cols % 8 == 0.
+ * Replaces RowwiseAdd (a projection's bias) / RowwiseMul: iron/operators/elementwise_add.py:18,
+ * elementwise_mul.py:18, iron/common/elementwise.py:797-867. */
+int iron_row_broadcast_bf16(const uint16_t* x, const uint16_t* row, uint16_t* y, int rows, int cols,
+                            int multiply, const int* valid, void* stream);
+
 /* Attention, many queries (prefill / prompt chunk).  Q,O: (seq, heads, d) if q_interleaved
  * else (heads, seq, d); K,V: (kv_len, kv_heads, d) if kv_interleaved else (kv_heads, kv_len, d).
  * The queries are the last rows of the keys: query i sits at position kv_tokens - q_tokens + i,

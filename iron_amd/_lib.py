@@ -31,6 +31,7 @@ SIGNATURES = {
     "iron_silu_bf16": (c_int, [_P, _P, c_int64, _P, _P]),
     "iron_mul_bf16": (c_int, [_P, _P, _P, c_int64, _P, _P]),
     "iron_add_bf16": (c_int, [_P, _P, _P, c_int64, _P, _P]),
+    "iron_row_broadcast_bf16": (c_int, [_P, _P, _P, c_int, c_int, c_int, _P, _P]),
     "iron_silu_mul_bf16": (c_int, [_P, _P, _P, c_int64, _P, _P]),
     "iron_mha_prefill_bf16": (
         c_int,

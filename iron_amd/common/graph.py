@@ -418,17 +418,26 @@ class Handle:
 
     # -- arithmetic ----------------------------------------------------------
     def _binary(self, other, op_name):
-        from ..operators.elementwise_add import ElementwiseAdd
-        from ..operators.elementwise_mul import ElementwiseMul
+        """``self`` met elementwise by an operand of its shape, or -- where ``self`` has two axes or
+        more -- by one row of its last axis (iron/common/graph/handle.py:652-676)."""
+        from ..operators.elementwise_add import ElementwiseAdd, RowwiseAdd
+        from ..operators.elementwise_mul import ElementwiseMul, RowwiseMul
 
         if isinstance(other, Resident):
             other = other._handle()
         if not isinstance(other, Handle):
             return NotImplemented
-        if other.elements != self.elements:
-            raise ValueError(f"{op_name}: {self.shape} and {other.shape} differ in size")
-        cls = ElementwiseAdd if op_name == "+" else ElementwiseMul
-        return cls.step(self, other).reshape(self.shape)
+        whole, rowwise = (ElementwiseAdd, RowwiseAdd) if op_name == "+" else (ElementwiseMul, RowwiseMul)
+        x, y = self, other
+        if len(x.shape) == 1 and len(y.shape) > 1:   # a row met by a matrix: commutative
+            x, y = y, x
+        if len(x.shape) > 1 and tuple(y.shape) == tuple(x.shape[-1:]):
+            rows = x.elements // x.shape[-1]
+            return rowwise.step(x.reshape(rows, x.shape[-1]), y).reshape(x.shape)
+        if y.elements != x.elements:
+            raise TypeError(f"{whole.__name__} of {x!r} takes an operand of its shape or a row of "
+                            f"{x.shape[-1] if x.shape else 1}, not {list(y.shape)}")
+        return whole.step(x, y).reshape(x.shape)
 
     def __add__(self, other):
         return self._binary(other, "+")

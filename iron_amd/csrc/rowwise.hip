@@ -185,6 +185,32 @@ static int launch_ew(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t 
   IRON_LAUNCH_CHECK();
 }
 
+
+// Every row of x (rows, cols) met elementwise by the one row `row` (cols): a projection's bias
+// (add) or a per-column scale (mul).  A thread takes 16-byte pieces; the piece of `row` it needs
+// stays in L1/L2.  `valid` bounds the rows.
+template <Ew OP>
+__global__ __launch_bounds__(256) void row_broadcast_kernel(const bf16_t* __restrict__ x,
+                                                            const bf16_t* __restrict__ row,
+                                                            bf16_t* __restrict__ y, int rows, int cols,
+                                                            const int* __restrict__ valid) {
+  rows = bound_or(valid, rows);
+  const int cpr = cols >> 3;                 // 16-byte pieces a row has
+  const long nchunk = (long)rows * cpr;
+  const long stride = (long)gridDim.x * 256;
+  const uint4* xv = reinterpret_cast<const uint4*>(x);
+  const uint4* rv = reinterpret_cast<const uint4*>(row);
+  uint4* yv = reinterpret_cast<uint4*>(y);
+  for (long c = (long)blockIdx.x * 256 + threadIdx.x; c < nchunk; c += stride) {
+    float fa[8], fb[8], fy[8];
+    unpack8(xv[c], fa);
+    unpack8(rv[c % cpr], fb);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) fy[i] = ew_apply<OP>(fa[i], fb[i]);
+    yv[c] = pack8(fy);
+  }
+}
+
 }  // namespace iron
 
 using namespace iron;
@@ -244,4 +270,23 @@ extern "C" int iron_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* y, 
 extern "C" int iron_silu_mul_bf16(const uint16_t* g, const uint16_t* u, uint16_t* y, int64_t n,
                                   const int* valid, void* stream) {
   return launch_ew<Ew::kSiluMul>(g, u, y, n, valid, stream, "silu_mul");
+}
+
+extern "C" int iron_row_broadcast_bf16(const uint16_t* x, const uint16_t* row, uint16_t* y, int rows,
+                                       int cols, int multiply, const int* valid, void* stream) {
+  IRON_REQUIRE(x && row && y, "row_broadcast: null operand");
+  IRON_REQUIRE(rows > 0 && cols > 0 && cols % 8 == 0,
+               "row_broadcast: rows (%d) positive, cols (%d) a positive multiple of 8", rows, cols);
+  IRON_REQUIRE((((uintptr_t)x | (uintptr_t)row | (uintptr_t)y) & 15) == 0,
+               "row_broadcast: operands must be 16-byte aligned");
+  long chunks = (long)rows * (cols >> 3);
+  long blocks = (chunks + 255) / 256;
+  if (blocks > 256L * 16) blocks = 256L * 16;
+  if (multiply)
+    hipLaunchKernelGGL((row_broadcast_kernel<Ew::kMul>), dim3((unsigned)blocks), dim3(256), 0,
+                       (hipStream_t)stream, x, row, y, rows, cols, valid);
+  else
+    hipLaunchKernelGGL((row_broadcast_kernel<Ew::kAdd>), dim3((unsigned)blocks), dim3(256), 0,
+                       (hipStream_t)stream, x, row, y, rows, cols, valid);
+  IRON_LAUNCH_CHECK();
 }

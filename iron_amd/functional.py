@@ -40,8 +40,9 @@ def linear(x, weight, bias=None, *, precision: Precision = Precision.HIGHEST, **
         y = GEMM.step(x, weight, b_col_maj=True, precision=precision)
     if bias is None:
         return y
+    # A row added to every row, also for GEMV's one-dimensional output.
     rows = math.prod(y.shape) // bias.shape[0]
-    raise NotImplementedError(f"linear(): a bias over {rows} rows (RowwiseAdd) is not built")
+    return (y.reshape(rows, bias.shape[0]) + bias).reshape(y.shape)
 
 
 def _last_axis(name: str, x, normalized_shape) -> None:

@@ -154,6 +154,18 @@ add = _binary("iron_add_bf16")
 silu_mul = _binary("iron_silu_mul_bf16")
 
 
+def row_broadcast(x, row, y, *, rows, cols, multiply=False, valid=None):
+    """``y[r] = x[r] + row`` (or ``* row``) for every row ``r`` under the bound."""
+    _numel(_dev(x, "x"), rows * cols, "x")
+    _numel(_dev(row, "row"), cols, "row")
+    _numel(_dev(y, "y"), rows * cols, "y")
+    check(
+        lib().iron_row_broadcast_bf16(ptr(x), ptr(row), ptr(y), rows, cols, int(bool(multiply)),
+                                      ptr(_word(valid, "valid")), current_stream()),
+        "iron_row_broadcast_bf16",
+    )
+
+
 def silu(x, y, *, n=None, valid=None):
     n = y.numel() if n is None else n
     _numel(_dev(x, "x"), n, "x")

@@ -63,8 +63,6 @@ class DecoderConfig:
             object.__setattr__(self, "head_dim", self.hidden_size // self.num_attention_heads)
         if self.prefill_chunk > self.max_seq_len:
             object.__setattr__(self, "prefill_chunk", self.max_seq_len)
-        if self.attention_bias or self.mlp_bias:
-            raise ValueError(f"{type(self).__name__}: biased projections are not built")
         if self.hidden_act != "silu":
             raise ValueError(f"{type(self).__name__}: hidden_act {self.hidden_act!r}: only silu is built")
 

@@ -138,6 +138,38 @@ class Rowwise(Elementwise):
         return self.rows * self.tile_size
 
 
+class RowBroadcast(Rowwise):
+    """``rows`` rows of ``tile_size`` elements, each met elementwise by the one ``row``
+    (iron/common/elementwise.py:797-867; the reference's cut of a wide row into ``segments``
+    lines is its cores' memory limit and does not change the sums)."""
+
+    multiply: ClassVar[bool] = False
+    tile_cap: ClassVar[int] = 4096
+    test = Testing([Sweep(rows=True), Case(dict(rows=64, tile_size=5120), id="wide_row"),
+                    Case(dict(rows=8, tile_size=12288), id="wider_row")])
+
+    segments: int = tunable()
+    line: int = tunable()
+    x = In(Rowwise.rows, Rowwise.tile_size)
+    row = In(Rowwise.tile_size, replicate=True)
+    y = Out(Rowwise.rows, Rowwise.tile_size)
+
+    def tolerance(self) -> Tolerance:
+        return Tolerance.exact(note="bf16(f32(x) op f32(row))")
+
+    def build(self):
+        from .. import kernels
+        from ..common.declare import Built
+
+        rows, cols, multiply = self.rows, self.tile_size, self.multiply
+
+        def launch(t, words):
+            kernels.row_broadcast(t["x"], t["row"], t["y"], rows=rows, cols=cols, multiply=multiply,
+                                  valid=words.get("valid"))
+
+        return Built("iron_row_broadcast_bf16", launch)
+
+
 class WeightedRowwise(Rowwise):
     """A ``Rowwise`` kernel's rows, optionally times a learned ``weight`` row, the row
     rounded to bf16 between the two (elementwise.py:676-682)."""

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 from ..common.declare import Built
 from ..common.verify import Tolerance
-from .elementwise import BinaryElementwise
+from .elementwise import BinaryElementwise, RowBroadcast
 
 
 class ElementwiseAdd(BinaryElementwise):
@@ -20,3 +20,9 @@ class ElementwiseAdd(BinaryElementwise):
             kernels.add(t["a"], t["b"], t["y"], n=n, valid=words.get("valid"))
 
         return Built("iron_add_bf16", launch)
+
+
+class RowwiseAdd(RowBroadcast):
+    """Each row plus one row, ``x + row``: a projection's bias (iron/operators/elementwise_add.py:18)."""
+
+    multiply = False

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 from ..common.declare import Built
 from ..common.verify import Tolerance
-from .elementwise import BinaryElementwise
+from .elementwise import BinaryElementwise, RowBroadcast
 
 
 class ElementwiseMul(BinaryElementwise):
@@ -20,3 +20,9 @@ class ElementwiseMul(BinaryElementwise):
             kernels.mul(t["a"], t["b"], t["y"], n=n, valid=words.get("valid"))
 
         return Built("iron_mul_bf16", launch)
+
+
+class RowwiseMul(RowBroadcast):
+    """Each row times one row, ``x * row`` (iron/operators/elementwise_mul.py:18)."""
+
+    multiply = True

@@ -39,6 +39,18 @@ def add(op, a, b):
     return ops.add(a, np.asarray(b).reshape(np.shape(a)))
 
 
+def rowwise_add(op, x, row):
+    """iron/common/elementwise.py:797-867 over eltwise.add_sized: every row plus the one row."""
+    x = np.asarray(x).reshape(op.rows, op.tile_size)
+    return ops.add(x, np.broadcast_to(np.asarray(row).reshape(1, -1), x.shape))
+
+
+def rowwise_mul(op, x, row):
+    """iron/common/elementwise.py:797-867 over eltwise.mul_sized."""
+    x = np.asarray(x).reshape(op.rows, op.tile_size)
+    return ops.mul(x, np.broadcast_to(np.asarray(row).reshape(1, -1), x.shape))
+
+
 def rope(op, x, angles):
     """iron/operators/rope.py:167-184."""
     return ops.rope(x, angles, two_halves=op.two_halves)
@@ -74,5 +86,5 @@ def install() -> None:
 
     REFERENCES.update(
         GEMM=gemm, GEMV=gemv, RMSNorm=rms_norm, SiLU=silu, ElementwiseMul=mul, ElementwiseAdd=add,
-        RoPE=rope, MHA=mha, Copy=copy, Sample=sample,
+        RoPE=rope, MHA=mha, Copy=copy, Sample=sample, RowwiseAdd=rowwise_add, RowwiseMul=rowwise_mul,
     )

@@ -9,6 +9,7 @@ in the oracle.  ``tests/golden/llama_small_hf_logits.npz`` is the reference's ow
 those weights, keyed by sha256(int64 tokens)[:16] (iron/lm/golden.py:88-92).
 """
 
+import dataclasses
 import hashlib
 from pathlib import Path
 
@@ -27,8 +28,30 @@ SCALED = LlamaConfig(
 )
 
 
+# The reference's second toy: the same shape with its RoPE table unscaled and a bias on each of
+# q, k, v and o (tests/applications/llama/reference/test.py:23-43; SMALL,
+# iron/tests/support/llama_model.py:56-68).  Its golden, tests/golden/llama_biased_hf_logits.npz,
+# is the reference's tests/applications/llama/reference/goldens/biased.npz; prompts are drawn at seed 1.
+BIASED = dataclasses.replace(SCALED, rope_scaling=None, attention_bias=True)
+BIASED_GOLDEN = Path(__file__).parent / "golden" / "llama_biased_hf_logits.npz"
+
+
+def biased_names(config=BIASED):
+    """The checkpoint's names in the order the reference's test draws them: Llama's, then each
+    layer's four biases."""
+    c = config
+    Q, KV = c.num_attention_heads * c.head_dim, c.num_key_value_heads * c.head_dim
+    out = dict(shapes(c))
+    for i in range(c.num_hidden_layers):
+        attention = f"model.layers.{i}.self_attn"
+        out |= {f"{attention}.q_proj.bias": (Q,), f"{attention}.k_proj.bias": (KV,),
+                f"{attention}.v_proj.bias": (KV,), f"{attention}.o_proj.bias": (c.hidden_size,)}
+    return out
+
+
 def weights(config=SCALED, seed=0):
-    return ops.filled(shapes(config), seed=seed)
+    named = biased_names(config) if config.attention_bias else shapes(config)
+    return ops.filled(named, seed=seed)
 
 
 class Golden:

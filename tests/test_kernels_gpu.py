@@ -157,6 +157,20 @@ def test_gemm_bounded_rows_and_k_do_not_read_the_poison(cuda, b_col_maj):
     assert np.all(got[rows:] == 5.0)
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 2048), (8, 512), (2048, 512), (64, 5120), (7, 12288)])
+@pytest.mark.parametrize("multiply", [False, True])
+def test_row_broadcast_exact(cuda, rows, cols, multiply):
+    rng = np.random.default_rng(70)
+    x, row = bf(rng, rows, cols), bf(rng, cols)
+    y = out_like((rows, cols), cuda, fill=3.0)
+    bound = max(1, rows - 3)
+    K.row_broadcast(dev(x, cuda), dev(row, cuda), y, rows=rows, cols=cols, multiply=multiply, valid=word(bound, cuda))
+    want = (ops.mul if multiply else ops.add)(x, np.broadcast_to(row, x.shape))
+    got = from_torch(y)
+    assert np.array_equal(got[:bound], want[:bound])
+    assert np.all(got[bound:] == 3.0)
+
+
 # --------------------------------------------------------------------- rowwise
 @pytest.mark.parametrize("rows,cols", [(1, 2048), (2048, 2048), (7, 64), (3, 8192), (2, 16640)])
 @pytest.mark.parametrize("weighted", [False, True])

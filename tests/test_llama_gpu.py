@@ -13,7 +13,7 @@ import pytest
 import oracle
 from iron_amd.applications.llama import LLAMA_3_2_1B, Llama
 from iron_amd.lm.causal import OnHost
-from tests.llama_support import SCALED, Golden, assert_close, kl, weights
+from tests.llama_support import BIASED, BIASED_GOLDEN, SCALED, Golden, assert_close, kl, weights
 
 pytestmark = pytest.mark.gpu
 oracle.install()
@@ -211,3 +211,29 @@ def test_fused_kernels_against_the_oracle_at_llama_1b_width(cuda):
         lg = torch.empty(rows, dtype=torch.bfloat16, device=cuda)
         K.gemv_fused(dev(Wh), dev(x), lg, M=rows, K=E, norm_w=dev(g), eps=1e-5, epilogue=0)
         close(lg, ops.gemv(Wh, n))
+
+
+def test_biased_projections_match_hugging_face_on_the_gpu(cuda):
+    """q, k, v and o with a bias (RowwiseAdd after each projection) against the reference's second
+    golden fixture: prompt, greedy decode under the HIP graph, and a prompt of several chunks."""
+    golden, w = Golden(BIASED_GOLDEN), weights(BIASED)
+    model = Llama(dataclasses.replace(BIASED, max_seq_len=4 * BIASED.prefill_chunk), w)
+    model.load_versions()
+    try:
+        names = [type(s.op).__name__ for s in model.decode_step.recording.steps]
+        assert names.count("RowwiseAdd") == 4 * BIASED.num_hidden_layers
+        prompt = np.random.default_rng(1).integers(0, BIASED.vocab_size, 8)
+        want = golden.logits(prompt)
+        got = model.logits(prompt)
+        assert_close(got, want)
+        tokens = prompt
+        for step in range(6):
+            tokens = np.append(tokens, want.argmax())
+            want = golden.logits(tokens)
+            got = model.logits(tokens)
+            assert_close(got, want, f"step {step}")
+            assert kl(want, got) < 1e-3
+        tokens = np.random.default_rng(3).integers(0, BIASED.vocab_size, BIASED.prefill_chunk + 150)
+        assert_close(model.logits(tokens), golden.logits(tokens))
+    finally:
+        model.release()

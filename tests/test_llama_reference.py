@@ -14,7 +14,7 @@ import pytest
 import oracle
 from iron_amd.applications.llama import Llama
 from iron_amd.lm.causal import OnHost
-from tests.llama_support import SCALED, Golden, assert_close, kl, weights
+from tests.llama_support import BIASED, BIASED_GOLDEN, SCALED, Golden, assert_close, kl, weights
 
 oracle.install()
 
@@ -39,8 +39,8 @@ def host(config, w):
     return model
 
 
-def greedy_case(golden):
-    prompt = np.random.default_rng(7).integers(0, SCALED.vocab_size, 8)
+def greedy_case(golden, seed=7):
+    prompt = np.random.default_rng(seed).integers(0, SCALED.vocab_size, 8)
     tokens, expected = prompt, []
     first = logits = golden.logits(tokens)
     for _ in range(6):
@@ -112,3 +112,40 @@ def test_a_model_runs_only_the_versions_it_loaded(w):
         model.logits([1, 2, 3])
     with pytest.raises(RuntimeError, match=r"load_versions\(\) first"):
         model(start=0, rows=1, rope_start=0, token=0, position=0)
+
+
+# ---- projections with a bias (RowwiseAdd), against the reference's second golden fixture
+def test_biased_projections_match_the_forward_prompt_then_decode():
+    golden, w = Golden(BIASED_GOLDEN), weights(BIASED)
+    prompt, first, expected = greedy_case(golden, seed=1)
+    model = host(BIASED, w)
+    got = model.logits(prompt)
+    assert_close(got, first)
+    assert kl(first, got) < 1e-3
+    tokens = prompt
+    for step, want in enumerate(expected):
+        tokens = np.append(tokens, got.argmax())
+        got = model.logits(tokens)
+        assert_close(got, want, f"step {step}")
+
+
+def test_biased_projections_match_the_forward_token_by_token_and_in_chunks():
+    golden, w = Golden(BIASED_GOLDEN), weights(BIASED)
+    prompt, first, _ = greedy_case(golden, seed=1)
+    model = host(BIASED, w)
+    for n in range(1, len(prompt) + 1):
+        last = model.logits(prompt[:n])
+    assert_close(last, first)
+    C = BIASED.prefill_chunk
+    model = host(dataclasses.replace(BIASED, max_seq_len=4 * C), w)
+    tokens = np.random.default_rng(3).integers(0, BIASED.vocab_size, C + 150)
+    assert_close(model.logits(tokens), golden.logits(tokens))
+
+
+def test_a_bias_changes_the_logits():
+    """The biased toy's weights with the biases dropped no longer match its golden: the bias is used."""
+    golden, w = Golden(BIASED_GOLDEN), weights(BIASED)
+    prompt, first, _ = greedy_case(golden, seed=1)
+    zeroed = {n: (np.zeros_like(a) if n.endswith("bias") else a) for n, a in w.items()}
+    got = host(BIASED, zeroed).logits(prompt)
+    assert np.abs(np.asarray(got, np.float32).reshape(-1) - first).max() > 0.05 * np.abs(first).max()
