@@ -46,6 +46,21 @@ class LlamaConfig(DecoderConfig):
     rope_scaling: Llama3RopeScaling | None = None
     precision: Precision = Precision.MEDIUM
 
+    @classmethod
+    def convert(cls, name: str, value):
+        if name == "rope_scaling":
+            return Llama3RopeScaling.from_dict(value)
+        return super().convert(name, value)
+
+    @classmethod
+    def from_json(cls, data: dict, source="config.json") -> "LlamaConfig":
+        """As ``DecoderConfig.from_json``, at ``Precision.HIGH`` from 3B's width up (the reference's
+        choice for its device; every precision runs the same f32-accumulating kernels here)."""
+        config = super().from_json(data, source)
+        if config.hidden_size < 3072:
+            return config
+        return dataclasses.replace(config, precision=Precision.HIGH)
+
 
 #: Llama 3.2 1B's shape.
 LLAMA_3_2_1B = LlamaConfig(

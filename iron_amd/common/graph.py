@@ -868,7 +868,12 @@ class Recording:
                 out[:n] = table[ids[:n]]
                 return out.reshape(h.shape)
             s = start_of(h)
-            return flat[s : s + h.elements].reshape(h.shape)
+            got = flat[s : s + h.elements]
+            if got.size < h.elements:
+                # A fixed-width window from a per-call start may run past its buffer; its bound (checked
+                # before dispatch) keeps every row that is read inside.  The rest read as zeros here.
+                got = np.concatenate([got, np.zeros(h.elements - got.size, flat.dtype)])
+            return got.reshape(h.shape)
 
         def write(h: Handle, value: np.ndarray, rows: int | None) -> None:
             flat = array_of(h.buffer)

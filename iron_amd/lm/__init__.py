@@ -1,7 +1,9 @@
 """A decoder-only language model wired from the hot-path operators."""
 
 from .causal import Call, CausalLM, Decoder, Stats
+from .checkpoint import Checkpoint, weights_file, write_safetensors
 from .config import DecoderConfig, rope_angles
 from .session import Session
 
-__all__ = ["Call", "CausalLM", "Decoder", "DecoderConfig", "Session", "Stats", "rope_angles"]
+__all__ = ["Call", "CausalLM", "Checkpoint", "Decoder", "DecoderConfig", "Session", "Stats", "rope_angles",
+           "weights_file", "write_safetensors"]

@@ -9,8 +9,11 @@ in a HIP graph that carries its own values, so a run of decode steps is a run of
 from __future__ import annotations
 
 import dataclasses
+import functools
+import json
 import time
 from collections.abc import Iterator
+from pathlib import Path
 from typing import Any
 
 import numpy as np
@@ -64,6 +67,74 @@ class CausalLM(iron.Graph):
 
     decoder_class = Decoder
     layer_class = DecoderLayer
+    #: The config class ``from_checkpoint`` builds from a checkpoint's ``config.json``.
+    config_class = DecoderConfig
+    checkpoint = None
+    tokenizer = None
+
+    @classmethod
+    def from_checkpoint(cls, path, *, max_seq_len: int | None = None, **changes):
+        """The model of a checkpoint directory's files (``config.json``, ``model.safetensors`` or its
+        sharded index, ``tokenizer.json``), not yet loaded (iron/lm/model.py:321-388).
+
+        Args:
+            path: the directory (nothing is downloaded here).
+            max_seq_len: the longest context served, at most the checkpoint's own.
+            changes: other config fields replaced (``prefill_chunk=...``).
+
+        Raises:
+            ValueError: ``max_seq_len`` is past the checkpoint's own.
+        """
+        from .checkpoint import Checkpoint, weights_file
+        from .tokenizer import Tokenizer, TokenizerJson
+
+        directory = Path(path)
+        if not directory.is_dir():
+            raise FileNotFoundError(f"{directory} is not a checkpoint directory (repositories are not downloaded)")
+        config = cls.config_class.from_checkpoint(directory)
+        if max_seq_len is not None:
+            if max_seq_len > config.max_seq_len:
+                raise ValueError(f"max_seq_len {max_seq_len} is past the model's {config.max_seq_len}")
+            changes["max_seq_len"] = max_seq_len
+        if changes:
+            config = dataclasses.replace(config, **changes)
+        checkpoint = Checkpoint(weights_file(directory))
+        # On the device a bf16 tensor goes up as the file holds it; the host stand-in computes on arrays.
+        weights = checkpoint.state_dict(as_torch=not issubclass(cls, OnHost))
+        if config.tie_word_embeddings:
+            weights.pop("lm_head.weight", None)  # some exports repeat the tied matrix
+        model = cls(config, weights)
+        model.checkpoint = checkpoint
+        if (directory / "tokenizer.json").exists():
+            settings, jinja = directory / "tokenizer_config.json", directory / "chat_template.jinja"
+            found = json.loads(settings.read_text()) if settings.exists() else {}
+            template = jinja.read_text() if jinja.exists() else found.get("chat_template")
+            b = found.get("bos_token")
+            bos_token = (b["content"] if isinstance(b, dict) else b) or ""
+            model.tokenizer = Tokenizer(TokenizerJson(directory / "tokenizer.json"), template, bos_token)
+        return model
+
+    @classmethod
+    def load(cls, path, *, max_seq_len: int | None = None, capture: bool = True, **changes):
+        """``from_checkpoint``'s model compiled and loaded, its weights uploaded."""
+        model = cls.from_checkpoint(path, max_seq_len=max_seq_len, **changes)
+        model.load_versions(capture=capture)
+        return model
+
+    @functools.cached_property
+    def eos(self) -> set[int]:
+        """The tokens generation stops at: the checkpoint's ``eos_token_id``, one or a list, from its
+        ``generation_config.json`` or else its ``config.json``; none without either."""
+        if self.checkpoint is None:
+            return set()
+        directory = Path(self.checkpoint.path).parent
+        for name in ("generation_config.json", "config.json"):
+            file = directory / name
+            if file.exists():
+                eos = json.loads(file.read_text()).get("eos_token_id")
+                if eos is not None:
+                    return set(eos) if isinstance(eos, list) else {eos}
+        return set()
 
     def __init__(self, config: DecoderConfig, weights):
         self.config = config
@@ -170,11 +241,24 @@ class CausalLM(iron.Graph):
         """The logits after the last of ``tokens``, the whole history (``Session.logits``)."""
         return self.session.logits(tokens)
 
-    def generate(self, tokens, max_tokens: int) -> list[int]:
-        """Greedy: ``max_tokens`` tokens drawn on the device after ``tokens``; fills ``stats``."""
-        return list(self.stream(tokens, max_tokens))
+    def generate(self, prompt, max_tokens: int):
+        """Greedy: up to ``max_tokens`` tokens drawn on the device after ``prompt``, stopping after an
+        end-of-sequence token; fills ``stats``.  Token ids in, token ids out; a text (or a chat's
+        list of messages) in, the text drawn out (needs the checkpoint's tokenizer)."""
+        if _is_text(prompt):
+            drawn = [t for t in self.stream(prompt, max_tokens) if t not in self.eos]
+            return self.tokenizer.decode(drawn)
+        return list(self.stream(prompt, max_tokens))
 
-    def stream(self, tokens, max_tokens: int) -> Iterator[int]:
+    def _ids(self, prompt):
+        if not _is_text(prompt):
+            return prompt
+        if self.tokenizer is None:
+            raise ValueError(f"{type(self).__name__}: a text prompt takes the checkpoint's tokenizer; none is loaded")
+        return self.tokenizer(prompt) if isinstance(prompt, str) else self.tokenizer.chat(prompt)
+
+    def stream(self, prompt, max_tokens: int) -> Iterator[int]:
+        tokens = self._ids(prompt)
         t0 = time.perf_counter()
         first = None
         n = 0
@@ -183,9 +267,16 @@ class CausalLM(iron.Graph):
             if first is None:
                 first = time.perf_counter()
             yield token
+            if token in self.eos:
+                break
         end = time.perf_counter()
         self.stats = Stats(ttft=(first or end) - t0,
                            tokens_per_s=(n - 1) / (end - first) if n > 1 and end > first else 0.0, tokens=n)
+
+
+def _is_text(prompt) -> bool:
+    """A string, or a chat: a list of ``{"role": ..., "content": ...}`` messages."""
+    return isinstance(prompt, str) or (isinstance(prompt, list) and bool(prompt) and isinstance(prompt[0], dict))
 
 
 class _HostOutput:

@@ -7,7 +7,9 @@ Field names are a Hugging Face checkpoint's ``config.json``'s where it has one
 from __future__ import annotations
 
 import dataclasses
+import json
 from collections.abc import Callable
+from pathlib import Path
 
 import numpy as np
 
@@ -57,6 +59,67 @@ class DecoderConfig:
     attention_bias: bool = False
     mlp_bias: bool = False
     sliding_window: int | None = None
+
+    # Where a checkpoint's config.json holds a field, where that is not the field's own name; None:
+    # nowhere -- a choice of this package, kept at its default by ``from_checkpoint`` and left out
+    # by ``to_json`` (iron/lm/config.py:68-183).
+    JSON = {"eps": "rms_norm_eps", "max_seq_len": "max_position_embeddings", "precision": None,
+            "prefill_chunk": None}
+
+    @classmethod
+    def from_checkpoint(cls, path):
+        """The fields read from ``path``'s ``config.json``: ``path`` is that file, or a checkpoint's
+        directory or one of its files.
+
+        Raises:
+            FileNotFoundError: no ``config.json`` is there.
+            ValueError: the file lacks a field that has no default.
+        """
+        path = Path(path)
+        if path.name != "config.json":
+            path = (path if path.is_dir() else path.parent) / "config.json"
+        return cls.from_json(json.loads(path.read_text()), path)
+
+    @classmethod
+    def from_json(cls, data: dict, source="config.json"):
+        """``from_checkpoint`` on ``data``, a ``config.json`` already parsed; ``source`` names it in an error."""
+        kwargs, missing = {}, []
+        for f in dataclasses.fields(cls):
+            key = cls.JSON.get(f.name, f.name)
+            if key is None:
+                continue
+            value = data.get(key)
+            if value is None:  # absent, or Hugging Face's null for an unset option
+                if f.default is dataclasses.MISSING and f.default_factory is dataclasses.MISSING:
+                    missing.append(key)
+                continue
+            kwargs[f.name] = cls.convert(f.name, value)
+        if missing:
+            raise ValueError(f"{source} lacks {missing}")
+        return cls(**kwargs)
+
+    @classmethod
+    def convert(cls, name: str, value):
+        """A ``config.json`` value as the field holds it."""
+        if name == "rope_scaling":
+            kind = value.get("rope_type", value.get("type"))
+            if kind != "default":
+                raise ValueError(f"rope_scaling {value}: no RoPE table here builds it")
+            return None
+        return value
+
+    def to_json(self) -> dict:
+        """The fields as ``config.json`` names them: ``from_json``'s inverse."""
+        out = {}
+        for f in dataclasses.fields(self):
+            key = self.JSON.get(f.name, f.name)
+            value = getattr(self, f.name)
+            if dataclasses.is_dataclass(value) and not isinstance(value, type):
+                value = dataclasses.asdict(value)
+            if key is None or not isinstance(value, (bool, int, float, str, tuple, dict)):
+                continue
+            out[key] = list(value) if isinstance(value, tuple) else value
+        return out
 
     def __post_init__(self):
         if self.head_dim is None:

@@ -237,3 +237,17 @@ def test_biased_projections_match_hugging_face_on_the_gpu(cuda):
         assert_close(model.logits(tokens), golden.logits(tokens))
     finally:
         model.release()
+
+
+def test_a_checkpoint_directory_loads_onto_the_gpu_and_generates_text(cuda, tmp_path, golden):
+    """config.json + model.safetensors (bf16 as stored, uploaded without widening) + tokenizer.json."""
+    from tests.test_checkpoint import toy_directory
+
+    model = Llama.load(toy_directory(tmp_path))
+    try:
+        prompt = np.random.default_rng(7).integers(0, SCALED.vocab_size, 8)
+        assert_close(model.logits(prompt), golden.logits(prompt))
+        ids = model.generate(model.tokenizer("w5 w9"), 5)
+        assert model.generate("w5 w9", 5) == model.tokenizer.decode([t for t in ids if t not in model.eos])
+    finally:
+        model.release()
