@@ -533,7 +533,7 @@ constexpr int BIG_WAVES = IRON_BIG_WAVES;
 #endif
 constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stages of half-line rows) measured 13 % slower
 #define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
-constexpr int BIG_A_BYTES = BIG_BM * BK * 2, BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
+constexpr int BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
 
 template <int WAVES, int KB>
 __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
