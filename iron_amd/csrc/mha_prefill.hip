@@ -2,7 +2,7 @@
 // flash-style, causal / windowed, grouped-query, the queries being the last rows
 // of the keys.
 //
-// grid = (ceil(seq/128), heads); a block of 4 waves takes 128 query rows of one
+// grid = ceil(seq/128) * heads; a block of 4 waves takes 128 query rows of one
 // head, a wave 32 of them.  Keys and values stream through LDS in tiles of 64
 // rows.  The wave computes the TRANSPOSED score tile S^T = K Q^T (M = keys,
 // N = queries): a lane then owns one query column, so the row max / row sum of
@@ -30,7 +30,7 @@ constexpr int BKV = 64;   // key rows per tile
 template <int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
-    bf16_t* __restrict__ O, int group, int seq, int seq_len, int kv_len, float scale_log2,
+    bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
     long kv_head_stride, const int* __restrict__ valid, const int* __restrict__ kv_valid) {
   constexpr int ROWB = D * 2;            // bytes of a tile row
@@ -46,9 +46,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, g = lane >> 5;
-  const int head = blockIdx.y, kvh = head / group;
-  // Heaviest (last) query blocks first under a causal mask.
-  const int qb = gridDim.x - 1 - blockIdx.x;
+  // Blocks are dispatched in id order, so the id runs over the query blocks from the last (under a
+  // causal mask the heaviest: it sees the most keys) to the first, all heads of one query block
+  // together: the long blocks start first and the short ones fill the tail.  Within a query block
+  // the heads are dealt so that an XCD (block id mod 8) serves the heads of one KV group, whose
+  // K and V it then reads from its own L2.
+  const int j = blockIdx.x % heads;
+  const int head = (heads % 8 == 0) ? (j % 8) * (heads / 8) + j / 8 : j;
+  const int kvh = head / group;
+  const int qb = (int)(gridDim.x / heads) - 1 - (int)(blockIdx.x / heads);
   const int q0 = qb * BQ;
 
   const int q_tokens = valid ? bound_or(valid, seq) : seq_len;
@@ -295,14 +301,14 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   const long kv_row = kv_interleaved ? (long)kv_heads * d : d;
   const long kv_head = kv_interleaved ? d : (long)kv_len * d;
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid((seq + BQ - 1) / BQ, heads), block(256);
+  dim3 grid(((seq + BQ - 1) / BQ) * heads), block(256);
   hipStream_t s = (hipStream_t)stream;
   if (d == 64)
-    hipLaunchKernelGGL((mha_prefill_kernel<64>), grid, block, 0, s, Q, K, V, O, heads / kv_heads, seq,
+    hipLaunchKernelGGL((mha_prefill_kernel<64>), grid, block, 0, s, Q, K, V, O, heads, heads / kv_heads, seq,
                        seq_len, kv_len, scale_log2, causal, window, q_row, q_head, kv_row, kv_head,
                        valid, kv_valid);
   else
-    hipLaunchKernelGGL((mha_prefill_kernel<128>), grid, block, 0, s, Q, K, V, O, heads / kv_heads,
+    hipLaunchKernelGGL((mha_prefill_kernel<128>), grid, block, 0, s, Q, K, V, O, heads, heads / kv_heads,
                        seq, seq_len, kv_len, scale_log2, causal, window, q_row, q_head, kv_row,
                        kv_head, valid, kv_valid);
   IRON_LAUNCH_CHECK();
