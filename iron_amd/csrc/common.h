@@ -152,6 +152,14 @@ __device__ __forceinline__ short4v lds_read_tr16(unsigned lds_addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(lds_addr));
   return v;
 }
+// The same with a compile-time byte offset in the instruction's offset field (no address arithmetic).
+template <int OFFSET>
+__device__ __forceinline__ short4v lds_read_tr16_at(unsigned lds_addr) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "the offset field holds 16 bits");
+  short4v v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFFSET));
+  return v;
+}
 struct TrFrag {   // the two halves of a fragment, as the reads deliver them
   short4v lo, hi;
 };

@@ -13,6 +13,8 @@
 #include "../../include/iron_hip.h"
 #include "common.h"
 
+#include <type_traits>
+
 namespace iron {
 
 constexpr int BQ = 128;   // query rows per block
@@ -234,18 +236,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
         }
 
-        // O^T += V^T P^T, two (t, h) steps at a time so one wait covers a batch of reads.
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        // O^T += V^T P^T, a 32-key half at a time so one wait covers a batch of reads; the key
+        // offsets ride in the reads' offset fields.
+        auto pv_half = [&](auto half) {
+          constexpr int t = decltype(half)::value;
           TrFrag vf[DT][2];
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-              const unsigned a = vt + (32 * t + 16 * h) * ROWB + v_frag[dt];
-              vf[dt][h].lo = lds_read_tr16(a);
-              vf[dt][h].hi = lds_read_tr16(a + 8 * ROWB);
-            }
+          for (int dt = 0; dt < DT; ++dt) {
+            const unsigned a = vt + v_frag[dt];
+            vf[dt][0].lo = lds_read_tr16_at<(32 * t) * ROWB>(a);
+            vf[dt][0].hi = lds_read_tr16_at<(32 * t + 8) * ROWB>(a);
+            vf[dt][1].lo = lds_read_tr16_at<(32 * t + 16) * ROWB>(a);
+            vf[dt][1].hi = lds_read_tr16_at<(32 * t + 24) * ROWB>(a);
+          }
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
             lds_tr_wait(vf[dt][0], vf[dt][1]);
@@ -253,7 +256,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             for (int h = 0; h < 2; ++h)
               oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_join(vf[dt][h]), pf[t][h], oacc[dt], 0, 0, 0);
           }
-        }
+        };
+        pv_half(std::integral_constant<int, 0>{});
+        pv_half(std::integral_constant<int, 1>{});
       }
     }
     wait_vmcnt<0>();   // the idle fetches of the last iterations land before the block's LDS is released
