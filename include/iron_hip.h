@@ -68,6 +68,18 @@ int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, float eps, c
                          uint16_t* q_out, uint16_t* keys, uint16_t* values, int hidden, int heads,
                          int kv_heads, int d, int cache_rows, const int* position, void* stream);
 
+/* A prompt chunk's three projections and the rotation of q and k in one launch (no single
+ * counterpart in the reference: replaces 3 GEMM and 2 RoPE steps, iron/lm/blocks.py:617-648, and
+ * rounds where those steps round): q = x Wq^T, k = x Wk^T, v = x Wv^T, each rounded to bf16; q and k
+ * then turned by RoPE (two halves) with row r's angles `angles[r]` (rows, 64; cos and sin interleaved)
+ * and rounded again.  x (rows, hidden); Wq (heads*d, hidden), Wk, Wv (kv_heads*d, hidden);
+ * q_out (rows, heads*d), k_out, v_out (rows, kv_heads*d).  d == 64; heads, kv_heads even;
+ * hidden % 64 == 0; rows >= 64.  valid: rows computed. */
+int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
+                          const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
+                          uint16_t* k_out, uint16_t* v_out, int rows, int hidden, int heads,
+                          int kv_heads, int d, const int* valid, void* stream);
+
 /* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; w NULL = unweighted (one rounding).
  * x,y (rows, cols); w (cols).  cols % 8 == 0.  valid: rows computed.
  * Replaces norm.rms_norm_eps + eltwise.mul_sized: iron/operators/rms_norm.py:10,

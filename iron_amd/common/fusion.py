@@ -11,6 +11,10 @@ round:
   GEMV, ElementwiseAdd (the residual)                    => iron_gemv_fused_bf16 (epilogue 1)
   RMSNorm, GEMV (the head)                               => iron_gemv_fused_bf16 (epilogue 0)
 
+and, in a prompt chunk's version (several rows, 64-wide heads),
+
+  GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
+
 A run is fused only if every intermediate it hides is read by nothing else.
 """
 
@@ -59,6 +63,12 @@ def _name(step) -> str:
 def _same(a, b) -> bool:
     """Two handles that are the same elements of the same buffer."""
     return a.buffer is b.buffer and a.offset == b.offset and a.elements == b.elements and _plain(a) and _plain(b)
+
+
+def _same_view(a, b) -> bool:
+    """The same elements of the same buffer, whatever bound each carries."""
+    return (a.buffer is b.buffer and a.offset == b.offset and a.elements == b.elements
+            and a.index is None and a.ids is None and b.index is None and b.ids is None)
 
 
 def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) -> list[Fused]:
@@ -156,6 +166,37 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                             norm_w=tensor(s.inputs["weight"]).reshape(-1), y=tensor(g0.outputs["C"]).reshape(-1))
                 kw = dict(M=g0.op.M, K=g0.op.K, eps=float(s.op.epsilon), epilogue=0)
                 got = Fused("norm_gemv", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+        elif (_name(s) == "GEMM" and len(steps) - i >= 5
+              and [_name(t) for t in steps[i + 1 : i + 5]] == ["GEMM", "GEMM", "RoPE", "RoPE"]):
+            # a prompt chunk's projections and rotations
+            gq, gk, gv, rq, rk = steps[i : i + 5]
+            a = gq.inputs["A"]
+
+            def rows_gemm(g):
+                return (g.op.b_col_maj and not g.op.c_col_maj and "valid_k" not in g.values
+                        and _same_view(g.inputs["A"], a) and g.op.M == gq.op.M and g.op.K == gq.op.K
+                        and all(h.index is None and h.ids is None for h in (*g.inputs.values(), *g.outputs.values())))
+
+            q, k, v = (g.outputs["C"] for g in (gq, gk, gv))
+            M, d = gq.op.M, 64
+            ok = (
+                all(rows_gemm(g) for g in (gq, gk, gv)) and once(q) and once(k)
+                and M >= 64 and gq.op.K % 64 == 0 and gq.op.N % 128 == 0 and gk.op.N % 128 == 0
+                and gk.op.N == gv.op.N
+                and _same_view(rq.inputs["x"], q) and _same_view(rk.inputs["x"], k)
+                and all(r.op.two_halves and r.op.cols == d and r.op.angle_rows == M for r in (rq, rk))
+                and rq.op.rows * d == M * gq.op.N and rk.op.rows * d == M * gk.op.N
+                and rq.inputs["angles"].buffer is rk.inputs["angles"].buffer
+                and _same_view(rq.inputs["angles"], rk.inputs["angles"])
+                and all(h.index is None and h.ids is None for h in (rq.outputs["y"], rk.outputs["y"]))
+            )
+            if ok:
+                args = dict(x=tensor(a), Wq=tensor(gq.inputs["B"]), Wk=tensor(gk.inputs["B"]), Wv=tensor(gv.inputs["B"]),
+                            angles=tensor(rq.inputs["angles"]), q_out=tensor(rq.outputs["y"]),
+                            k_out=tensor(rk.outputs["y"]), v_out=tensor(v))
+                kw = dict(rows=M, hidden=gq.op.K, heads=gq.op.N // d, kv_heads=gk.op.N // d, d=d,
+                          valid=word(gq.values.get("valid")))
+                got = Fused("prefill_qkv", i, 5, lambda a=args, kw=kw: kernels.prefill_qkv(**a, **kw))
         elif gemv_row(s) and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseAdd":
             ad = steps[i + 1]
             c = s.outputs["C"]

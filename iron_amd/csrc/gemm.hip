@@ -289,12 +289,28 @@ constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK
 // instruction moves 4 k-rows x 256 B, chunks swizzled by 2*(k & 7)), and the fragments are
 // fetched with the transposing LDS read (ds_read_b64_tr_b16): within 16 lanes, lane i points
 // at 4 consecutive n of row k0 + i/4 and receives k0..k0+3 of column n0 + i%16.
-template <bool B_KN>
+// QKV: one launch for a prompt chunk's three projections and the rotation of two of them.  B, C and
+// N then stand for q's weight (N,K), output and width; `qkv` brings k's and v's (each kv_n wide,
+// widths multiples of the 128-column tile) and the chunk's angle rows (M, 64; cos and sin
+// interleaved).  A block's tile column picks its matrix.  With 64-wide heads a wave's 64 columns are
+// one head whose two halves are its two accumulator tiles, so q and k are rotated in registers:
+// rounded to bf16 as the projection would store them, turned (two halves), rounded again.
+struct QkvTail {
+  const bf16_t* Bk;
+  const bf16_t* Bv;
+  bf16_t* Ck;
+  bf16_t* Cv;
+  const bf16_t* angles;
+  int kv_n;
+};
+
+template <bool B_KN, bool QKV>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
-                                                      const bf16_t* __restrict__ B,
-                                                      bf16_t* __restrict__ C, int M, int N, int K,
+                                                      const bf16_t* __restrict__ B_,
+                                                      bf16_t* __restrict__ C_, int M, int N_, int K,
                                                       const int* __restrict__ valid, int tiles_m,
-                                                      int tiles_n, int patched) {
+                                                      int tiles_n, int patched, QkvTail qkv) {
+  static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int LOADS = 2 * INST;
   extern __shared__ __align__(16) char smem_nt[];
@@ -315,8 +331,22 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     tm = first + in_band % height;
     tn = in_band / height;
   }
-  const int m0 = tm * NT_BM, n0 = tn * NT_BN;
+  const int m0 = tm * NT_BM;
   if (m0 >= Mv) return;
+  const bf16_t* B = B_;
+  bf16_t* C = C_;
+  int N = N_, which = 0;
+  if constexpr (QKV) {
+    const int q_tiles = N_ / NT_BN, kv_tiles = qkv.kv_n / NT_BN;
+    if (tn >= q_tiles) {
+      which = tn < q_tiles + kv_tiles ? 1 : 2;
+      tn -= q_tiles + (which - 1) * kv_tiles;
+      B = which == 1 ? qkv.Bk : qkv.Bv;
+      C = which == 1 ? qkv.Ck : qkv.Cv;
+      N = qkv.kv_n;
+    }
+  }
+  const int n0 = tn * NT_BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -449,6 +479,29 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
   }
 
   wait_vmcnt<0>();  // the idle fetches of the last iterations land before the block's LDS is released
+  if constexpr (QKV) {
+    if (which < 2) {
+      // acc[i][0][e] and acc[i][1][e] are columns c and c + 32 of the wave's head, c = 8 (e/4) + 4 kh + e%4,
+      // of row m = fr of tile i: the pair RoPE turns by the angle row's (cos, sin) number c.
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int m = min(m0 + wm * 64 + i * 32 + fr, M - 1);
+        const bf16_t* ang = qkv.angles + (size_t)m * 64 + 8 * kh;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float cs[8];
+          unpack8(*reinterpret_cast<const uint4*>(ang + 16 * q), cs);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float x1 = round_bf16(acc[i][0][4 * q + e]), x2 = round_bf16(acc[i][1][4 * q + e]);
+            const float c = cs[2 * e], sn = cs[2 * e + 1];
+            acc[i][0][4 * q + e] = x1 * c - x2 * sn;
+            acc[i][1][4 * q + e] = x2 * c + x1 * sn;
+          }
+        }
+      }
+    }
+  }
   const int hi = kh * 4;
   const bool vec = (N & 3) == 0;
 #pragma unroll
@@ -471,21 +524,22 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     }
 }
 
-template <bool B_KN>
+template <bool B_KN, bool QKV = false>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
-                          const int* valid, hipStream_t s) {
-  const int tiles_m = (M + NT_BM - 1) / NT_BM, tiles_n = (N + NT_BN - 1) / NT_BN;
+                          const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}) {
+  const int tiles_m = (M + NT_BM - 1) / NT_BM;
+  const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / NT_BN : (N + NT_BN - 1) / NT_BN;
   const size_t lds = (size_t)NT_STAGES * NT_STAGE_BYTES;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nt_kernel<B_KN>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL(gemm_nt_kernel<B_KN>, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
-                     valid, tiles_m, tiles_n, patched);
+  hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
+                     valid, tiles_m, tiles_n, patched, qkv);
   IRON_LAUNCH_CHECK();
 }
 
@@ -742,4 +796,21 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   if (tiles128 >= 128 || (M >= 128 && N >= 128))
     return launch_gemm<128, 128, 2, 2>(A, B, C, M, N, K, b_col_maj, c_col_maj, valid, valid_k, s);
   return launch_gemm<64, 64, 2, 2>(A, B, C, M, N, K, b_col_maj, c_col_maj, valid, valid_k, s);
+}
+
+extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
+                                     const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
+                                     uint16_t* k_out, uint16_t* v_out, int rows, int hidden, int heads,
+                                     int kv_heads, int d, const int* valid, void* stream) {
+  IRON_REQUIRE(x && Wq && Wk && Wv && angles && q_out && k_out && v_out, "prefill_qkv: null operand");
+  IRON_REQUIRE(d == 64, "prefill_qkv: d (%d) must be 64 (a wave's 64 output columns are one head)", d);
+  IRON_REQUIRE(rows >= 64 && heads > 0 && kv_heads > 0 && heads % 2 == 0 && kv_heads % 2 == 0,
+               "prefill_qkv: rows (%d) at least 64; heads (%d) and kv_heads (%d) positive and even "
+               "(whole 128-column tiles)", rows, heads, kv_heads);
+  IRON_REQUIRE(hidden > 0 && hidden % BK == 0, "prefill_qkv: hidden (%d) must be a positive multiple of %d", hidden, BK);
+  IRON_REQUIRE((((uintptr_t)x | (uintptr_t)Wq | (uintptr_t)Wk | (uintptr_t)Wv | (uintptr_t)angles |
+                 (uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)v_out) & 15) == 0,
+               "prefill_qkv: operands must be 16-byte aligned");
+  QkvTail tail{Wk, Wv, k_out, v_out, angles, kv_heads * d};
+  return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, (hipStream_t)stream, tail);
 }

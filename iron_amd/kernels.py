@@ -107,6 +107,24 @@ def decode_qkv(x, norm_w, Wq, Wk, Wv, angles, q_out, keys, values, *, eps, hidde
     )
 
 
+def prefill_qkv(x, Wq, Wk, Wv, angles, q_out, k_out, v_out, *, rows, hidden, heads, kv_heads, d, valid=None):
+    """A prompt chunk's q/k/v projections with q and k turned by RoPE, one launch."""
+    _numel(_dev(x, "x"), rows * hidden, "x")
+    _numel(_dev(Wq, "Wq"), heads * d * hidden, "Wq")
+    _numel(_dev(Wk, "Wk"), kv_heads * d * hidden, "Wk")
+    _numel(_dev(Wv, "Wv"), kv_heads * d * hidden, "Wv")
+    _numel(_dev(angles, "angles"), rows * d, "angles")
+    _numel(_dev(q_out, "q_out"), rows * heads * d, "q_out")
+    _numel(_dev(k_out, "k_out"), rows * kv_heads * d, "k_out")
+    _numel(_dev(v_out, "v_out"), rows * kv_heads * d, "v_out")
+    check(
+        lib().iron_prefill_qkv_bf16(ptr(x), ptr(Wq), ptr(Wk), ptr(Wv), ptr(angles), ptr(q_out), ptr(k_out),
+                                    ptr(v_out), rows, hidden, heads, kv_heads, d, ptr(_word(valid, "valid")),
+                                    current_stream()),
+        "iron_prefill_qkv_bf16",
+    )
+
+
 def rmsnorm(x, w, y, *, rows, cols, eps, valid=None):
     _numel(_dev(x, "x"), rows * cols, "x")
     _numel(_dev(y, "y"), rows * cols, "y")

@@ -140,6 +140,29 @@ def test_gemm_weight_layout_fast_paths(cuda, M, Kdim, N, rows):
     assert np.all(got[lim:] == 5.0)
 
 
+@pytest.mark.parametrize("rows,bound,H,G", [(2048, None, 32, 8), (256, 150, 16, 4), (128, None, 2, 2)])
+def test_prefill_qkv_equals_three_projections_then_rope(cuda, rows, bound, H, G):
+    """The fused launch against the oracle's separate steps: project and round, rotate and round."""
+    rng = np.random.default_rng(91)
+    E, D = 512, 64
+    x = bf(rng, rows, E)
+    Wq, Wk, Wv = bf(rng, H * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05)
+    table = round_bf16(ops.rope_angles(D, rows + 5, 500000.0))[5:]
+    lim = rows if bound is None else bound
+    q, k, v = (ops.gemm(x, W, b_col_maj=True) for W in (Wq, Wk, Wv))
+    want_q = ops.rope(q.reshape(rows * H, D), table).reshape(rows, H * D)
+    want_k = ops.rope(k.reshape(rows * G, D), table).reshape(rows, G * D)
+    if bound is not None:
+        x[bound:] = np.nan
+    outs = [out_like((rows, n), cuda, fill=7.0) for n in (H * D, G * D, G * D)]
+    K.prefill_qkv(dev(x, cuda), dev(Wq, cuda), dev(Wk, cuda), dev(Wv, cuda), dev(table, cuda), *outs, rows=rows,
+                  hidden=E, heads=H, kv_heads=G, d=D, valid=None if bound is None else word(bound, cuda))
+    for got, want in zip(outs, (want_q, want_k, v)):
+        got = from_torch(got)
+        close(got[:lim], want[:lim], rtol=1e-2, atol=1e-2)
+        assert np.all(got[lim:] == 7.0)
+
+
 @pytest.mark.parametrize("b_col_maj", [False, True])
 def test_gemm_bounded_rows_and_k_do_not_read_the_poison(cuda, b_col_maj):
     """NaN past the bounds must not reach the output (test_gemm_bounded_k.py)."""
