@@ -18,6 +18,8 @@
 #include "../../include/iron_hip.h"
 #include "common.h"
 
+#include <climits>
+
 namespace iron {
 
 constexpr int BK = 64;
@@ -309,12 +311,15 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       const bf16_t* __restrict__ B_,
                                                       bf16_t* __restrict__ C_, int M, int N_, int K,
                                                       const int* __restrict__ valid, int tiles_m,
-                                                      int tiles_n, int patched, QkvTail qkv) {
+                                                      int tiles_n, int patched, int run_above,
+                                                      int run_upto, QkvTail qkv) {
   static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int LOADS = 2 * INST;
   extern __shared__ __align__(16) char smem_nt[];
   const int Mv = bound_or(valid, M);
+  // Two launches may share one problem, each taking a range of the row bound (see iron_gemm_bf16).
+  if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
   const int bid = blockIdx.x;
@@ -526,7 +531,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
 
 template <bool B_KN, bool QKV = false>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
-                          const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}) {
+                          const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}, int run_above = -1,
+                          int run_upto = INT_MAX) {
   const int tiles_m = (M + NT_BM - 1) / NT_BM;
   const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / NT_BN : (N + NT_BN - 1) / NT_BN;
   const size_t lds = (size_t)NT_STAGES * NT_STAGE_BYTES;
@@ -539,7 +545,7 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
-                     valid, tiles_m, tiles_n, patched, qkv);
+                     valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
   IRON_LAUNCH_CHECK();
 }
 
@@ -594,7 +600,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
                                                          const bf16_t* __restrict__ B,
                                                          bf16_t* __restrict__ C, int M, int N, int K,
                                                          const int* __restrict__ valid, int tiles_m,
-                                                         int tiles_n, int patched) {
+                                                         int tiles_n, int patched, int run_above,
+                                                         int run_upto) {
   static_assert(KB == 64 || (KB == 32 && WAVES == 4), "k per stage: 64, or 32 with 4 waves");
   constexpr int ROWB = KB * 2;               // bytes of a tile row in LDS
   constexpr int CPR = KB / 8;                // its 16-byte chunks
@@ -606,6 +613,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
   constexpr int KSTEPS = KB / 16;
   extern __shared__ __align__(16) char smem_big[];
   const int Mv = bound_or(valid, M);
+  if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
   const int bid = blockIdx.x;
@@ -750,7 +758,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
 }
 
 static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
-                             const int* valid, hipStream_t s) {
+                             const int* valid, hipStream_t s, int run_above = -1, int run_upto = INT_MAX) {
   const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
   constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
   const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
@@ -763,7 +771,7 @@ static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M,
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
-                     tiles_m, tiles_n, patched);
+                     tiles_m, tiles_n, patched, run_above, run_upto);
   IRON_LAUNCH_CHECK();
 }
 
@@ -785,8 +793,17 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   if (!c_col_maj && valid_k == nullptr && K % BK == 0 && M >= 64 && N >= 64) {
     // Enough whole 256x256 tiles to fill the chip: the large-tile kernel (offsets are 32-bit).
     if (b_col_maj && M % BIG_BM == 0 && N % BIG_BN == 0 && (long)(M / BIG_BM) * (N / BIG_BN) >= 192 &&
-        K <= (1 << 24))
-      return launch_gemm_nt256(A, B, C, M, N, K, valid, s);
+        K <= (1 << 24)) {
+      // Under a row bound read on the device the large tiles may cover too few rows to fill the
+      // chip (512 valid rows of 2048 leave 64 of 256 tiles).  Both kernels are launched, each
+      // running only for its range of the bound, decided where the bound is known: on the device.
+      const int tiles_n256 = N / BIG_BN;
+      const int few = tiles_n256 >= 128 ? 0 : BIG_BM * (128 / tiles_n256);   // rows up to which 128x128 tiles win
+      if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt256(A, B, C, M, N, K, valid, s);
+      const int rc = launch_gemm_nt256(A, B, C, M, N, K, valid, s, few, INT_MAX);
+      if (rc != 0) return rc;
+      return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, QkvTail{}, -1, few);
+    }
     if (b_col_maj) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s);
     // (K,N) B is read in whole 128-column tiles straight into LDS: N must be whole tiles.
     if (N % NT_BN == 0) return launch_gemm_nt<true>(A, B, C, M, N, K, valid, s);
