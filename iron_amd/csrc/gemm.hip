@@ -284,8 +284,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A,
 // the prefetch; each wave instead waits until only the two youngest stages are in flight.
 // Blocks are ordered so each XCD (block id mod 8) owns 8x4-tile patches and re-reads its
 // A/B panels from its own L2.
-constexpr int NT_BM = 128, NT_BN = 128, NT_STAGES = 4;
-constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
+constexpr int NT_STAGES = 4;
 
 // B_KN: B is (K,N) row-major.  Its tile lands in LDS as stored, [64 k][128 n] (a wave
 // instruction moves 4 k-rows x 256 B, chunks swizzled by 2*(k & 7)), and the fragments are
@@ -306,7 +305,7 @@ struct QkvTail {
   int kv_n;
 };
 
-template <bool B_KN, bool QKV>
+template <bool B_KN, bool QKV, int T>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
                                                       const bf16_t* __restrict__ B_,
                                                       bf16_t* __restrict__ C_, int M, int N_, int K,
@@ -314,6 +313,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       int tiles_n, int patched, int run_above,
                                                       int run_upto, QkvTail qkv) {
   static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
+  static_assert(T == 2 || (T == 1 && !B_KN && !QKV), "64x64 tiles: B (N,K), plain output");
+  // T = 32x32 MFMA tiles a wave owns along each of m and n: 128x128 block tiles (T = 2), or 64x64
+  // (T = 1) for problems -- or row bounds -- whose 128x128 tiles would leave CUs idle.
+  constexpr int NT_BM = 64 * T, NT_BN = 64 * T;
+  constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int LOADS = 2 * INST;
   extern __shared__ __align__(16) char smem_nt[];
@@ -385,11 +389,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                        IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + i) * 1024), 16, 0, 0);
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[T][T];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < T; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < T; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
@@ -400,18 +404,18 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
   for (int s = 0; s < NT_STAGES - 1; ++s) issue(min(s, nk - 1), s);
 
   const int fr = lane & 31, kh = lane >> 5;
-  int a_off[2], a_swz[2], b_off[2], b_swz[2];
+  int a_off[T], a_swz[T], b_off[T], b_swz[T];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int ra = wm * 64 + i * 32 + fr, rb = wn * 64 + i * 32 + fr;
+  for (int i = 0; i < T; ++i) {
+    const int ra = wm * 32 * T + i * 32 + fr, rb = wn * 32 * T + i * 32 + fr;
     a_off[i] = ra * 128; a_swz[i] = (ra >> 1) & 7;
     b_off[i] = NT_A_BYTES + rb * 128; b_swz[i] = (rb >> 1) & 7;
   }
   // (K,N) B: this lane's row within a 16-k step and its 8-byte piece of the row.
   const int tr_k = (kh << 3) + ((lane & 15) >> 2);
-  int tr_n[2];
+  int tr_n[T];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) tr_n[i] = wn * 64 + i * 32 + (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  for (int i = 0; i < T; ++i) tr_n[i] = wn * 64 + i * 32 + (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
 
   // One load of the 2*INST a wave issues per stage (A's first, then B's).
   auto issue_one = [&](char* st, int kt, int idx) {
@@ -439,9 +443,9 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
       t.hi = lds_read_tr16(base + (k + 4) * 256 + c1);
     }
   };
-  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[2], bf16x8 (&bfr)[2], TrFrag (&tf)[2]) {
+  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[T], bf16x8 (&bfr)[T], TrFrag (&tf)[T]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) read_frag_pair(st, ks, i, af[i], bfr[i], tf[i]);
+    for (int i = 0; i < T; ++i) read_frag_pair(st, ks, i, af[i], bfr[i], tf[i]);
   };
   // A wave is alone on its SIMD, so nothing overlaps unless its own instruction stream interleaves:
   // each k-step's four MFMAs are issued with the next step's fragment reads and a quarter of the
@@ -456,28 +460,30 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     const int kn = min(kt + NT_STAGES - 1, nk - 1);
     char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
     const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
-    bf16x8 af[2][2], bfr[2][2];
-    TrFrag tf[2][2];
+    bf16x8 af[2][T], bfr[2][T];
+    TrFrag tf[2][T];
     read_frags(st, 0, af[0], bfr[0], tf[0]);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
       if constexpr (B_KN) {
-        lds_tr_wait(tf[cur][0], tf[cur][1]);
+        lds_tr_wait(tf[cur][0], tf[cur][T - 1]);
         bfr[cur][0] = tr_join(tf[cur][0]);
-        bfr[cur][1] = tr_join(tf[cur][1]);
+        bfr[cur][T - 1] = tr_join(tf[cur][T - 1]);
       }
       // Source order is issue order (nothing crosses a sched_barrier): while an MFMA runs, half of
       // the next k-step's fragment reads or one prefetch load goes out.
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < T; ++i) {
         acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][i], acc[i][0], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (ks + 1 < BK / 16) read_frag_pair(st, ks + 1, i, af[nxt][i], bfr[nxt][i], tf[nxt][i]);
         __builtin_amdgcn_sched_barrier(0);
-        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][1], af[cur][i], acc[i][1], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        issue_one(nst, kn, ks * 2 + i);
+        if constexpr (T == 2) {
+          acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][1], af[cur][i], acc[i][1], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        issue_one(nst, kn, ks * T + i);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -510,10 +516,10 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
   const int hi = kh * 4;
   const bool vec = (N & 3) == 0;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < T; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int m = m0 + wm * 64 + i * 32 + fr, nb = n0 + wn * 64 + j * 32;
+    for (int j = 0; j < T; ++j) {
+      const int m = m0 + wm * 32 * T + i * 32 + fr, nb = n0 + wn * 32 * T + j * 32;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = nb + 8 * q + hi;
@@ -529,22 +535,23 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     }
 }
 
-template <bool B_KN, bool QKV = false>
+template <bool B_KN, bool QKV = false, int T = 2>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                           const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}, int run_above = -1,
                           int run_upto = INT_MAX) {
-  const int tiles_m = (M + NT_BM - 1) / NT_BM;
-  const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / NT_BN : (N + NT_BN - 1) / NT_BN;
-  const size_t lds = (size_t)NT_STAGES * NT_STAGE_BYTES;
+  constexpr int BM = 64 * T, BN = 64 * T;
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / BN : (N + BN - 1) / BN;
+  const size_t lds = (size_t)NT_STAGES * (BM + BN) * BK * 2;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV, T>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
+  hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV, T>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
                      valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
   IRON_LAUNCH_CHECK();
 }
@@ -804,9 +811,20 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
       if (rc != 0) return rc;
       return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, QkvTail{}, -1, few);
     }
-    if (b_col_maj) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s);
+    if (b_col_maj) {
+      // 128x128 tiles that would occupy under half the CUs give way to 64x64 ones: always, where
+      // the shape says so; under a row bound, by a second launch for the low range of the bound.
+      const int tiles_n128 = (N + 127) / 128;
+      const long tiles128 = (long)((M + 127) / 128) * tiles_n128;
+      if (tiles128 < 128) return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s);
+      const int few = tiles_n128 >= 128 ? 0 : 128 * (127 / tiles_n128);   // rows up to which 64x64 tiles win
+      if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s);
+      const int rc = launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, QkvTail{}, few, INT_MAX);
+      if (rc != 0) return rc;
+      return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, QkvTail{}, -1, few);
+    }
     // (K,N) B is read in whole 128-column tiles straight into LDS: N must be whole tiles.
-    if (N % NT_BN == 0) return launch_gemm_nt<true>(A, B, C, M, N, K, valid, s);
+    if (N % 128 == 0) return launch_gemm_nt<true>(A, B, C, M, N, K, valid, s);
   }
   // 128x128 tiles fill the 256 CUs once at 2048x2048; narrower problems take 64-wide tiles.
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);

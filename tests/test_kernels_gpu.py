@@ -121,7 +121,7 @@ def test_gemm_ragged_shapes(cuda, M, Kdim, N, b_col_maj):
     close(C, ops.gemm(A, B, b_col_maj=b_col_maj), rtol=1e-2, atol=2e-2)
 
 
-@pytest.mark.parametrize("M,Kdim,N,rows", [(2048, 512, 8192, None), (2048, 64, 6144, None), (4096, 192, 4096, 1000), (4096, 192, 4096, 3000),
+@pytest.mark.parametrize("M,Kdim,N,rows", [(2048, 512, 8192, None), (2048, 64, 6144, None), (4096, 192, 4096, 1000), (4096, 192, 4096, 3000), (2048, 128, 2048, 512), (2048, 128, 2048, 1500), (2048, 192, 512, 700),
                                            (128, 64, 128, None), (256, 128, 192, None)])
 def test_gemm_weight_layout_fast_paths(cuda, M, Kdim, N, rows):
     """B (N,K): the 256x256-tile kernel (>= 192 whole tiles) and the 128x128 one, down to a single
