@@ -155,10 +155,12 @@ int iron_copy_rows(const void* src, void* dst, int rows, int64_t row_bytes, int6
                    const int* dst_row, const int* valid, void* stream);
 
 /* Greedy draw: *token = index of the first largest logit among logits[0..n); when record is
- * not NULL also record[*at] = token (at NULL = 0; skipped if outside [0, record_len)).
+ * not NULL also record[*at] = token (at NULL = 0; skipped if outside [0, record_len)), and when
+ * token_copy is not NULL *token_copy = token (the carried `token` word of a decode loop: the draw
+ * feeds the next step without a copy kernel between).
  * Replaces Sample with an all-zero draw row: iron/operators/sample.py:72-79,106,324-333. */
 int iron_argmax_bf16(const uint16_t* logits, int n, int* token, int* record, int record_len,
-                     const int* at, void* stream);
+                     const int* at, int* token_copy, void* stream);
 
 /* Evaluate n per-call word expressions in order, on the device, in one thread:
  *   words[e.dst] = clamp(((words[e.src] * e.mul + e.add) >> e.shift), e.lo, e.hi)

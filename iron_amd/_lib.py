@@ -46,7 +46,7 @@ SIGNATURES = {
     "iron_mha_decode_workspace_bytes": (c_int64, [c_int, c_int]),
     "iron_gather_rows": (c_int, [_P, _P, _P, c_int, c_int, c_int64, _P, _P]),
     "iron_copy_rows": (c_int, [_P, _P, c_int, c_int64, c_int64, c_int64, c_int, c_int, _P, _P, _P, _P]),
-    "iron_argmax_bf16": (c_int, [_P, c_int, _P, _P, c_int, _P, _P]),
+    "iron_argmax_bf16": (c_int, [_P, c_int, _P, _P, c_int, _P, _P, _P]),
     "iron_eval_words": (c_int, [_P, c_int, _P, c_int, _P]),
     "iron_probe_mfma_bf16": (c_int, [_P, c_int64, _P, c_int, _P]),
     "iron_probe_mfma_flops": (c_int64, [c_int]),

@@ -1155,9 +1155,23 @@ class CompiledGraph:
             else:
                 rows.append([self.slots[k], 0, 0, int(v), 0, -big - 1, big])
         self.n_exprs = len(rows)
+        # A replay ends by carrying its values and re-deriving the words the next replay reads, in
+        # one launch: the carried rows are followed by a second copy of the derived ones.
+        self.n_tail = 0
+        if self.n_exprs > self.n_derived and self.n_exprs + self.n_derived <= WORD_SLOTS:
+            rows = rows + rows[: self.n_derived]
+            self.n_tail = self.n_exprs
         if rows:
             table = torch.tensor(rows, dtype=torch.int32).reshape(-1)
             self.expr_table[: table.numel()].copy_(table)
+        # A value carried from the draw's own output is written into its word by the draw itself.
+        self._carry_by_draw: dict[int, int] = {}
+        last = self.recording.steps[-1] if self.recording.steps else None
+        if last is not None and type(last.op).__name__ == "Sample":
+            for slot, h in list(self.carry_copies):
+                if h.buffer is last.outputs["token"].buffer and h.offset == last.outputs["token"].offset:
+                    self._carry_by_draw[len(self.recording.steps) - 1] = slot
+                    self.carry_copies.remove((slot, h))
         self._launches = [self._bind(step) for step in self.recording.steps]
         self._fused = {}
         if self.fuse:
@@ -1186,6 +1200,9 @@ class CompiledGraph:
                 )
         if views:
             words = {**words, "__views__": views}
+        slot = self._carry_by_draw.get(self.recording.steps.index(step)) if self._carry_by_draw else None
+        if slot is not None:
+            words = {**words, "__carry_token__": self.words[slot : slot + 1]}
         return built.launch, tensors, words
 
     def _run_steps(self) -> None:
@@ -1218,8 +1235,11 @@ class CompiledGraph:
         for slot, h in self.carry_copies:
             kernels.copy_rows(self._tensor(h).view(-1)[:1], self.words[slot : slot + 1], rows=1, row_elems=1,
                               src_rows=1, dst_rows=1)
-        if self.n_exprs > self.n_derived:
+        if self.n_tail:
+            kernels.eval_words(self.words, self.expr_table[7 * self.n_derived :], self.n_tail)
+        elif self.n_exprs > self.n_derived:
             kernels.eval_words(self.words, self.expr_table[7 * self.n_derived :], self.n_exprs - self.n_derived)
+            self._derive()
 
     def _capture(self) -> None:
         import torch
@@ -1235,7 +1255,8 @@ class CompiledGraph:
             stream.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
-                self._derive()
+                # The host wrote every word, derived ones included, before the first replay; each
+                # replay re-derives them for the next as it carries.
                 self._run_steps()
                 self._carry_on_device()
             stream.synchronize()

@@ -64,7 +64,8 @@ __device__ __forceinline__ Best better(Best a, Best b) {
 __global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* __restrict__ logits, int n,
                                                       int* __restrict__ token,
                                                       int* __restrict__ record, int record_len,
-                                                      const int* __restrict__ at) {
+                                                      const int* __restrict__ at,
+                                                      int* __restrict__ token_copy) {
   Best best{-INFINITY, 0x7fffffff};
   const int nchunk = n >> 3;
   const uint4* lv = reinterpret_cast<const uint4*>(logits);
@@ -94,6 +95,7 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* __restrict__
     // Every logit NaN or -inf: index 0, as a scan from the left would leave it.
     int tok = b.i == 0x7fffffff ? 0 : b.i;
     *token = tok;
+    if (token_copy != nullptr) *token_copy = tok;
     if (record != nullptr) {
       int where = at ? *at : 0;
       if (where >= 0 && where < record_len) record[where] = tok;
@@ -153,12 +155,12 @@ extern "C" int iron_copy_rows(const void* src, void* dst, int rows, int64_t row_
 }
 
 extern "C" int iron_argmax_bf16(const uint16_t* logits, int n, int* token, int* record,
-                                int record_len, const int* at, void* stream) {
+                                int record_len, const int* at, int* token_copy, void* stream) {
   IRON_REQUIRE(logits && token, "argmax: null operand");
   IRON_REQUIRE(n > 0, "argmax: n (%d) must be positive", n);
   IRON_REQUIRE(((uintptr_t)logits & 15) == 0, "argmax: logits must be 16-byte aligned");
   hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits, n, token,
-                     record, record_len, at);
+                     record, record_len, at, token_copy);
   IRON_LAUNCH_CHECK();
 }
 

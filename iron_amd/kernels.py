@@ -278,7 +278,7 @@ def copy_rows(src, dst, *, rows, row_elems, src_rows, dst_rows, src_stride=None,
     )
 
 
-def argmax(logits, token, *, n=None, record=None, at=None):
+def argmax(logits, token, *, n=None, record=None, at=None, token_copy=None):
     n = logits.numel() if n is None else n
     _dev(logits, "logits")
     _dev(token, "token", torch.int32)
@@ -287,7 +287,7 @@ def argmax(logits, token, *, n=None, record=None, at=None):
     check(
         lib().iron_argmax_bf16(
             ptr(logits), n, ptr(token), ptr(record), 0 if record is None else record.numel(),
-            ptr(_word(at, "at")), current_stream(),
+            ptr(_word(at, "at")), ptr(_word(token_copy, "token_copy")), current_stream(),
         ),
         "iron_argmax_bf16",
     )

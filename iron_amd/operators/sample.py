@@ -59,7 +59,9 @@ class Sample(Operator):
         drawable = self.drawable
 
         def launch(t, words):
+            # "__carry_token__": the scratchpad word a compiled loop carries the draw in, if it does.
             kernels.argmax(t["logits"].reshape(-1), t["token"].reshape(-1), n=drawable,
-                           record=t["tokens"].reshape(-1), at=words.get("at"))
+                           record=t["tokens"].reshape(-1), at=words.get("at"),
+                           token_copy=words.get("__carry_token__"))
 
         return Built("iron_argmax_bf16", launch)
