@@ -19,7 +19,9 @@ constexpr int kSingleMaxKeys = 2048;  // caches up to this many rows take the on
 // One wave's pass over key rows base + u*RW + rg for base = lo, lo + stride, ... while < hi, for
 // the G query heads q0.. of one KV head, then the merge of the wave's lane groups: on return every
 // lane holds the wave's (m, l) per head and acc = its 8 columns sub*8.. of the weighted V sum.
-template <int D, int G, int U>
+// STREAM: rows are read with streaming (non-temporal) loads -- right for a long cache read once per
+// step; a short cache is better left to the caches, where the next step finds much of it again.
+template <int D, int G, int U, bool STREAM>
 __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const bf16_t* __restrict__ Kh,
                                             const bf16_t* __restrict__ Vh, int q0, int lo, int hi,
                                             int stride, long row_stride, float scale_log2,
@@ -55,8 +57,8 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
       const int r = base + u * RW + rg;
       live[u] = r < hi;
       const size_t off = (size_t)(live[u] ? r : (hi - 1)) * row_stride;
-      kv[u] = load_stream(reinterpret_cast<const uint4*>(Kh + off));
-      vv[u] = load_stream(reinterpret_cast<const uint4*>(Vh + off));
+      kv[u] = STREAM ? load_stream(reinterpret_cast<const uint4*>(Kh + off)) : *reinterpret_cast<const uint4*>(Kh + off);
+      vv[u] = STREAM ? load_stream(reinterpret_cast<const uint4*>(Vh + off)) : *reinterpret_cast<const uint4*>(Vh + off);
     }
     float s[U][G];
 #pragma unroll
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
   const int whi = min(min(wlo + chunk / 4, blo + chunk), kv_tokens);
 
   float m[G], l[G], acc[G][8];
-  decode_scan<D, G, 4>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, kvh * G, wlo, whi,
+  decode_scan<D, G, 4, true>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, kvh * G, wlo, whi,
                     4 * RW, row_stride, scale_log2, m, l, acc);
 
   // Merge the 4 waves through LDS; wave 0 writes the block's partial.
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(1024) void mha_decode_single_kernel(
   const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
 
   float m[1], l[1], acc[1][8];
-  decode_scan<D, 1, U>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, head,
+  decode_scan<D, 1, U, false>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, head,
                     first + wave * U * RW, kv_tokens, WAVES * U * RW, row_stride, scale_log2, m, l, acc);
 
   __shared__ float sm[WAVES];
