@@ -171,15 +171,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
         const unsigned vt = lds_base + buf * STAGE + TILE;
         // S^T = K Q^T for the two 32-key halves of the tile.
         f32x16 sacc[2];
+        // A half's K fragments are all requested before its MFMAs (one wait, not one a fragment),
+        // and the second half's while the first half's MFMAs run.
+        bf16x8 kf[2][KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+          kf[0][s] = *reinterpret_cast<const bf16x8*>(kt + k_frag + (((2 * s + g) ^ k_swz) << 4));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+          kf[1][s] = *reinterpret_cast<const bf16x8*>(kt + 32 * ROWB + k_frag + (((2 * s + g) ^ k_swz) << 4));
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
 #pragma unroll
-          for (int s = 0; s < KS; ++s) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kt + t * 32 * ROWB + k_frag + (((2 * s + g) ^ k_swz) << 4));
-            sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[t], 0, 0, 0);
-          }
+          for (int s = 0; s < KS; ++s)
+            sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t][s], qf[s], sacc[t], 0, 0, 0);
         }
         // The prefetch goes out while the score MFMAs run (its buffer, tile - 1's, is free since
         // the barrier above).
