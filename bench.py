@@ -141,6 +141,24 @@ def bench_attention(torch, K, dev, n, rng):
     return out
 
 
+def bench_sample(torch, K, dev, n, rng):
+    """The draw over 128256 logits N(0, 3): greedy (an all-zero draw row) and at temperature 0.7 over the
+    top 50; a latency, launched back to back in a replayed graph."""
+    from iron_amd.bf16 import round_bf16, to_torch
+    from iron_amd.operators.sample import draw_row
+
+    vocab = 128256
+    logits = to_torch(round_bf16(rng.normal(0, 3, vocab).astype(np.float32))).to(dev)
+    token = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws = K.sample_workspace(vocab, dev)
+    out = {"vocab": vocab}
+    for name, (t, k) in (("greedy_us", (0.0, 1)), ("top50_t0.7_us", (0.7, 50))):
+        row = torch.from_numpy(np.ascontiguousarray(draw_row(t, k, 1234567890123))).to(dev)
+        launches = [lambda row=row: K.sample(logits, row, token, workspace=ws)] * 20
+        out[name] = round(graph_time_us(torch, launches, max(1, n // 20)), 2)
+    return out
+
+
 def bench_pre_attention(torch, K, dev, n):
     """The pre-attention block at sequence 2048, hidden 2048: RMSNorm, the Q/K/V projections (32 q / 8 kv heads,
     d 64) and RoPE on q and k, as the prompt chunk runs them (five operator steps)."""
@@ -400,6 +418,7 @@ def main():
     for g in gemm:
         g["frac_sustained"] = round(g["TFLOPs"] / mfma_ceiling["random"], 4)
     pre_attention = bench_pre_attention(torch, K, dev, n)
+    sample = bench_sample(torch, K, dev, n, rng)
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     decoder, cpu = bench_decoder(torch, dev, args.steps, args.warmup, not args.no_cpu)
@@ -436,6 +455,7 @@ def main():
         "mfma_sustained_TFLOPs": mfma_ceiling,
         "attention": attention,
         "pre_attention_block": pre_attention,
+        "sample": sample,
         "bench_wall_s": round(wall, 1),
     }
     if cpu is not None:

@@ -162,6 +162,23 @@ int iron_copy_rows(const void* src, void* dst, int rows, int64_t row_bytes, int6
 int iron_argmax_bf16(const uint16_t* logits, int n, int* token, int* record, int record_len,
                      const int* at, int* token_copy, void* stream);
 
+/* The draw of one draw row: draws[*row .. *row+4) = {temperature as float32 bits, top-k, the low
+ * and the high word of a 53-bit number} (row NULL = 0; draws NULL, a row outside
+ * [0, draws_words) or a temperature that is not positive = the greedy draw above).  With a
+ * temperature the candidates are the min(top-k, k_max) largest of logits[0..n), equals to the
+ * lower index; candidate i weighs exp((l_i - l_0) / temperature) in float64 and the token is the
+ * first whose running weight exceeds number * 2^-53 * total.  token, record, at, token_copy as
+ * iron_argmax_bf16.  1 <= k_max <= 64; n <= 524288.  workspace: iron_sample_workspace_bytes(n)
+ * bytes, 8-byte aligned, any contents (NULL allowed for n <= 2048).  One launch; launches on one
+ * device must not overlap (they count their blocks in one device-wide word).
+ * Replaces Sample: iron/operators/sample.py:72-79,106-336 (its sample_ref is out of the
+ * reference's tree; the arithmetic above is this library's own, fixed so a host computes the
+ * same token bit for bit). */
+int64_t iron_sample_workspace_bytes(int n);
+int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,
+                     const int* row, int k_max, void* workspace, int* token, int* record,
+                     int record_len, const int* at, int* token_copy, void* stream);
+
 /* Evaluate n per-call word expressions in order, on the device, in one thread:
  *   words[e.dst] = clamp(((words[e.src] * e.mul + e.add) >> e.shift), e.lo, e.hi)
  * exprs is n records of 7 int32 {dst, src, mul, add, shift, lo, hi} in device memory.

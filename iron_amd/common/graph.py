@@ -1377,7 +1377,8 @@ class CompiledGraph:
             tol = op.tolerance()
             if not plain or tol is None:
                 continue
-            written = {n: from_torch(tensors[n]).reshape(h.shape) for n, h in step.outputs.items()}
+            declared = {b.name for b in op.outputs}  # scratch memory is written and not judged
+            written = {n: from_torch(tensors[n]).reshape(h.shape) for n, h in step.outputs.items() if n in declared}
             values = {k: e.evaluate(full) for k, e in step.values.items()}
             extents = {k: v for k, v in values.items()
                        if next(m for m in op.declaration.per_calls if m.name == k).bounds is not None}

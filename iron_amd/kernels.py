@@ -293,6 +293,35 @@ def argmax(logits, token, *, n=None, record=None, at=None, token_copy=None):
     )
 
 
+def sample_workspace(n, device="cuda"):
+    return torch.empty(lib().iron_sample_workspace_bytes(n) // 8, dtype=torch.int64, device=device)
+
+
+def sample(logits, draws, token, *, n=None, row=None, k_max=64, workspace=None, record=None, at=None,
+           token_copy=None):
+    """The draw of ``draws``' row at word ``row`` (a device word, or None for the first row)."""
+    n = logits.numel() if n is None else n
+    _dev(logits, "logits")
+    _dev(token, "token", torch.int32)
+    if draws is not None:
+        _dev(draws, "draws", torch.int32)
+    if record is not None:
+        _dev(record, "record", torch.int32)
+    if workspace is None:
+        workspace = sample_workspace(n, logits.device)
+    need = lib().iron_sample_workspace_bytes(n)
+    if workspace.numel() * workspace.element_size() < need:
+        raise ValueError(f"workspace: {workspace.numel() * workspace.element_size()} bytes, need {need}")
+    check(
+        lib().iron_sample_bf16(
+            ptr(logits), n, ptr(draws), 0 if draws is None else draws.numel(), ptr(_word(row, "row")), k_max,
+            ptr(workspace), ptr(token), ptr(record), 0 if record is None else record.numel(),
+            ptr(_word(at, "at")), ptr(_word(token_copy, "token_copy")), current_stream(),
+        ),
+        "iron_sample_bf16",
+    )
+
+
 def eval_words(words, exprs, n=None):
     _dev(words, "words", torch.int32)
     _dev(exprs, "exprs", torch.int32)

@@ -136,12 +136,16 @@ class CausalLM(iron.Graph):
                     return set(eos) if isinstance(eos, list) else {eos}
         return set()
 
+    #: The most candidates a draw on the device weighs (``Sampler.rows`` refuses a larger top-k).
+    k_max = 64
+
     def __init__(self, config: DecoderConfig, weights):
         self.config = config
         self.rotary_emb = None if config.rope_theta is None else Rope(config)
         # Zero until the host writes draws: a row of zeros is greedy.
         self.draws = iron.state((config.max_seq_len, ROW_WORDS), np.int32)
         self.drawn = iron.state((config.max_seq_len,), np.int32)
+        self.sampled = False  # the draw rows hold a sampler's, not zeros
         self.prompt_chunk = None
         self.decode_step = None
         self.holder = None
@@ -195,7 +199,8 @@ class CausalLM(iron.Graph):
         """``logits`` and the token drawn from them on the device, carried with the next position."""
         c = self.config
         _, drawn = Sample.step(logits.reshape(c.vocab_size), self.draws, self.drawn,
-                               row=call.position * ROW_WORDS, at=call.position, drawable=c.vocab_size)
+                               row=call.position * ROW_WORDS, at=call.position, drawable=c.vocab_size,
+                               k_max=self.k_max)
         return logits, iron.carry(token=drawn, position=call.position + 1)
 
     # -- versions ------------------------------------------------------------
@@ -241,14 +246,15 @@ class CausalLM(iron.Graph):
         """The logits after the last of ``tokens``, the whole history (``Session.logits``)."""
         return self.session.logits(tokens)
 
-    def generate(self, prompt, max_tokens: int):
-        """Greedy: up to ``max_tokens`` tokens drawn on the device after ``prompt``, stopping after an
+    def generate(self, prompt, max_tokens: int, sampler=None):
+        """Up to ``max_tokens`` tokens drawn on the device after ``prompt``, stopping after an
         end-of-sequence token; fills ``stats``.  Token ids in, token ids out; a text (or a chat's
-        list of messages) in, the text drawn out (needs the checkpoint's tokenizer)."""
+        list of messages) in, the text drawn out (needs the checkpoint's tokenizer).  ``sampler``:
+        how each is drawn (``generation.Sampler``); None is greedy (iron/lm/model.py:506-545)."""
         if _is_text(prompt):
-            drawn = [t for t in self.stream(prompt, max_tokens) if t not in self.eos]
+            drawn = [t for t in self.stream(prompt, max_tokens, sampler) if t not in self.eos]
             return self.tokenizer.decode(drawn)
-        return list(self.stream(prompt, max_tokens))
+        return list(self.stream(prompt, max_tokens, sampler))
 
     def _ids(self, prompt):
         if not _is_text(prompt):
@@ -257,12 +263,12 @@ class CausalLM(iron.Graph):
             raise ValueError(f"{type(self).__name__}: a text prompt takes the checkpoint's tokenizer; none is loaded")
         return self.tokenizer(prompt) if isinstance(prompt, str) else self.tokenizer.chat(prompt)
 
-    def stream(self, prompt, max_tokens: int) -> Iterator[int]:
+    def stream(self, prompt, max_tokens: int, sampler=None) -> Iterator[int]:
         tokens = self._ids(prompt)
         t0 = time.perf_counter()
         first = None
         n = 0
-        for token in self.session.draw(tokens, max_tokens):
+        for token in self.session.draw(tokens, max_tokens, sampler):
             n += 1
             if first is None:
                 first = time.perf_counter()
@@ -298,6 +304,13 @@ class _HostVersion:
     def __call__(self, *tensors, **values):
         outs, carried = iron.Graph.reference(self.graph, *tensors, **values)
         return (*(_HostOutput(o) for o in outs), iron.Carry(carried))
+
+    def write(self, resident, array) -> None:
+        resident.host = np.array(array).reshape(-1)
+
+    def read(self, resident) -> np.ndarray:
+        host = getattr(resident, "host", None)
+        return np.zeros(resident.shape, np.int32) if host is None else host.reshape(resident.shape)
 
 
 class OnHost:

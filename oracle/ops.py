@@ -19,12 +19,20 @@ Pinned by (see tests/test_oracle.py):
   copy/gather exact                                              copy.py:839-902
   argmax      np.argmax of f32 logits (first of ties)            sample.py:72-79
   rope_angles closed forms                                       test_rope_angles.py:20-107
+  sample_ref  (temperature > 0) against what the mathematics fixes: exp_det
+              against math.exp, the draw's distribution against softmax
+              of the top-k logits / T, the cumulative walk against exact
+              rationals, top_k = 1 / n53 = 0 = greedy
 Parity unpinned (arithmetic lives in mlir-aie 1.4.6.dev15, absent here; textbook
 formula used, bounded by the stated bf16 tolerance and the model-level goldens):
-  rms_norm inner summation order / rsqrt, silu (LUT kernel), mul.
+  rms_norm inner summation order / rsqrt, silu (LUT kernel), mul;
+  sample_ref with temperature > 0 (aie.iron.kernels.sample.sample_ref): which token
+  a given 53-bit number draws is this build's own definition, stated at sample_ref.
 """
 
 from __future__ import annotations
+
+import math
 
 import numpy as np
 
@@ -209,6 +217,89 @@ def gather_rows(table, ids):
 def argmax(logits) -> int:
     """Greedy draw: the first largest float32 logit (sample.py:72-79, test_lm_host.py:554-557)."""
     return int(np.argmax(_f32(logits).reshape(-1)))
+
+
+# ------------------------------------------------------------------ sampling
+
+LOG2E = 1.4426950408889634
+LN2_HI = 6.93147180369123816490e-01   # ln 2 with its low 32 bits zero: n * LN2_HI is exact for |n| < 2**20
+LN2_LO = 1.90821492927058770002e-10
+EXP_FLOOR = -690.0                    # below it a weight is 0.0
+EXP_COEFFS = [1.0 / math.factorial(i) for i in range(14)]
+
+
+def exp_det(z: float) -> float:
+    """``exp(z)`` for ``z <= 0`` from IEEE double +, -, * alone (no fused multiply-add, no library
+    exp), so that any machine computes the same bits: n = rint(z * log2 e), r = z - n ln 2 in two
+    steps, a degree-13 Taylor polynomial by Horner, an exact scaling by 2**n."""
+    if not z >= EXP_FLOOR:   # also NaN
+        return 0.0
+    n = float(round(z * LOG2E))   # round(): half to even, as rint
+    r = (z - n * LN2_HI) - n * LN2_LO
+    p = EXP_COEFFS[13]
+    for c in EXP_COEFFS[12::-1]:
+        p = p * r + c
+    return math.ldexp(p, int(n))
+
+
+def sample_order(logits) -> np.ndarray:
+    """The indices of ``logits`` from the best: larger first, of equals the lower index, NaN last."""
+    x = _f32(logits).reshape(-1)
+    key = np.where(np.isnan(x), -np.inf, x).astype(np.float64)
+    nan = np.isnan(x)
+    # lexsort: the last key is the primary one.
+    return np.lexsort((np.arange(x.size), -key, nan))
+
+
+def sample_weights(logits, temperature, top_k, k_max=None):
+    """``(candidates, weights)``: the ``top_k`` best tokens (at most ``k_max``) in ``sample_order``
+    and each one's weight ``exp_det((logit - best) / temperature)`` in float64, 0.0 for a NaN logit."""
+    x = _f32(logits).reshape(-1)
+    k = min(max(int(top_k), 1), x.size if k_max is None else min(int(k_max), x.size))
+    cand = sample_order(x)[:k]
+    top, t = float(x[cand[0]]), float(np.float32(temperature))
+    weights = np.array([0.0 if math.isnan(float(x[i])) else exp_det((float(x[i]) - top) / t) for i in cand])
+    return cand, weights
+
+
+def sample_ref(logits, temperature, top_k, n53, k_max=None) -> int:
+    """The token a draw row draws from a row of bf16 logits (iron/operators/sample.py:72-79's
+    ``sample.sample_ref``, whose arithmetic is not in the reference's tree: this is the
+    definition this build's device kernel follows, bit for bit).
+
+    A temperature that is not positive is greedy: the first largest logit.  Otherwise the candidates are the
+    ``top_k`` (1..``k_max``) best logits, ties to the lower index; candidate i weighs
+    ``exp_det((l_i - l_0) / T)`` in float64 (T the float32 temperature); with ``total`` the
+    weights summed in candidate order and ``threshold = (n53 * 2**-53) * total``, the draw
+    is the first candidate whose running sum exceeds the threshold (the last of non-zero
+    weight if rounding leaves none).  A best logit that is not finite draws itself.
+    """
+    x = _f32(logits).reshape(-1)
+    if not float(np.float32(temperature)) > 0.0:
+        return int(sample_order(x)[0])
+    cand, weights = sample_weights(x, temperature, top_k, k_max)
+    if not math.isfinite(float(x[cand[0]])):
+        return int(cand[0])
+    total = 0.0
+    for w in weights:
+        total += float(w)
+    threshold = (float(int(n53)) * 2.0 ** -53) * total
+    running, last = 0.0, 0
+    for i, w in enumerate(weights):
+        running += float(w)
+        if running > threshold:
+            return int(cand[i])
+        if w > 0.0:
+            last = i
+    return int(cand[last])
+
+
+def draw_words(draw_row):
+    """``(temperature, top_k, n53)`` of a four-word draw row (iron/operators/sample.py:72-79)."""
+    words = np.asarray(draw_row, dtype=np.int32).reshape(-1)
+    row = words.view(np.uint32)
+    temperature = row[0:1].view(np.float32)[0]
+    return temperature, max(int(words[1]), 1), (int(row[2]) | int(row[3]) << 32) & ((1 << 53) - 1)
 
 
 # --------------------------------------------------------------- RoPE tables

@@ -71,11 +71,10 @@ def copy(op, src):
 
 
 def sample(op, logits, draws, tokens, *, row=0, at=0):
-    """iron/operators/sample.py:324-333; only the greedy draw (an all-zero row) is restated."""
+    """iron/operators/sample.py:72-79,324-333: the draw at ``draws`` word ``row``, recorded at ``at``."""
     words = np.asarray(draws).reshape(-1)[row : row + 4]
-    if np.any(words != 0):
-        raise NotImplementedError("the oracle restates the greedy draw only (an all-zero draw row)")
-    token = ops.argmax(np.asarray(logits).reshape(-1)[: op.drawable])
+    temperature, top_k, n53 = ops.draw_words(words)
+    token = ops.sample_ref(np.asarray(logits).reshape(-1)[: op.drawable], temperature, top_k, n53, op.k_max)
     tokens = np.array(tokens, dtype=np.int32).reshape(-1)
     tokens[at] = token
     return tokens, np.array([token], dtype=np.int32)
@@ -87,4 +86,6 @@ def install() -> None:
     REFERENCES.update(
         GEMM=gemm, GEMV=gemv, RMSNorm=rms_norm, SiLU=silu, ElementwiseMul=mul, ElementwiseAdd=add,
         RoPE=rope, MHA=mha, Copy=copy, Sample=sample, RowwiseAdd=rowwise_add, RowwiseMul=rowwise_mul,
+        # The host's draw, for iron_amd.lm.generation.Sampler's checks.
+        sample_ref=ops.sample_ref, sample_weights=ops.sample_weights,
     )

@@ -436,6 +436,89 @@ def test_argmax_first_of_ties_and_record(cuda):
     assert int(tok.item()) == ops.argmax(odd)
 
 
+def _draw_rows(rng, count, temperatures=(0.0, 0.05, 0.7, 1.0, 5.0), k_hi=65):
+    from iron_amd.operators.sample import draw_row
+
+    return np.stack([draw_row(rng.choice(temperatures), int(rng.integers(1, k_hi)), int(rng.integers(0, 1 << 53)))
+                     for _ in range(count)])
+
+
+def _host_draw(logits, row, k_max=64):
+    return ops.sample_ref(logits, *ops.draw_words(row), k_max)
+
+
+def _sample_rows(cuda, logits, rows, n=None, k_max=64):
+    """The device's draw for each of ``rows`` (picked by a device word), recorded one per slot."""
+    steps = len(rows)
+    tok = torch.full((1,), -1, dtype=torch.int32, device=cuda)
+    rec = torch.full((steps,), -1, dtype=torch.int32, device=cuda)
+    lg, dr = dev(logits, cuda), torch.from_numpy(np.ascontiguousarray(rows)).to(cuda)
+    for i in range(steps):
+        K.sample(lg, dr, tok, n=n, row=word(4 * i, cuda), k_max=k_max, record=rec, at=word(i, cuda))
+        assert int(tok.item()) == int(rec[i].item())
+    return rec.cpu().tolist()
+
+
+@pytest.mark.parametrize("vocab,drawable", [(4096, 4096), (128256, 128256), (51866, 51866), (151670, 151669),
+                                            (1003, 1003), (100, 100)])
+def test_sample_draws_the_host_token(cuda, vocab, drawable):
+    rng = np.random.default_rng(vocab)
+    logits = round_bf16(rng.normal(0, 3, vocab))
+    logits[rng.choice(drawable, 8, replace=False)] = logits[:drawable].max()
+    logits[drawable:] = logits.max() + 1   # padding no draw may take
+    rows = _draw_rows(rng, 48)
+    got = _sample_rows(cuda, logits, rows, n=drawable)
+    want = [_host_draw(logits[:drawable], r) for r in rows]
+    assert got == want
+    assert len(set(got)) > 4   # the draws spread over candidates
+
+
+def test_sample_ties_at_the_cut_go_to_the_lower_index(cuda):
+    # Few distinct values: the top-k cut falls inside a run of equal logits, and the k kept are
+    # those of the lowest index.
+    rng = np.random.default_rng(21)
+    logits = round_bf16(rng.integers(-3, 4, 128256).astype(np.float32) * 0.5)
+    rows = _draw_rows(rng, 32, temperatures=(0.7, 1.0, 5.0))
+    assert _sample_rows(cuda, logits, rows) == [_host_draw(logits, r) for r in rows]
+    # All equal: more logits at the floor than the list holds (the slow path), uniform over the first k.
+    flat = np.full(40000, 1.5, np.float32)
+    got = _sample_rows(cuda, flat, rows)
+    assert got == [_host_draw(flat, r) for r in rows] and max(got) < 64
+    # The best first in memory, falling: every thread's maximum is its first logit.
+    falling = round_bf16(np.linspace(8, -8, 20000, dtype=np.float32))
+    assert _sample_rows(cuda, falling, rows) == [_host_draw(falling, r) for r in rows]
+
+
+def test_sample_special_values_and_row_bounds(cuda):
+    from iron_amd.operators.sample import draw_row
+
+    rng = np.random.default_rng(22)
+    logits = round_bf16(rng.normal(0, 1, 5000))
+    logits[[7, 1200]] = np.nan
+    logits[[9, 4000]] = -np.inf
+    logits[[100, 101]] = [-0.0, 0.0]
+    rows = np.concatenate([_draw_rows(rng, 16), [draw_row(0.7, 50, 0), draw_row(0.7, 50, (1 << 53) - 1),
+                                                 draw_row(1e-3, 64, 1 << 52), draw_row(np.nan, 5, 77),
+                                                 draw_row(-1.0, 5, 77)]])
+    assert _sample_rows(cuda, logits, rows) == [_host_draw(logits, r) for r in rows]
+    infinite = logits.copy()
+    infinite[3000] = np.inf
+    assert _sample_rows(cuda, infinite, rows[:8]) == [3000] * 8
+    hollow = np.full(3000, -np.inf, np.float32)
+    hollow[[5, 2500]] = [np.nan, 2.0]
+    assert _sample_rows(cuda, hollow, rows[16:18]) == [2500, 2500]
+    # A k_max under the row's top-k caps it.
+    assert _sample_rows(cuda, logits, rows[:16], k_max=3) == [_host_draw(logits, r, 3) for r in rows[:16]]
+    # No draw rows, or a row outside them: greedy.
+    tok = torch.full((1,), -1, dtype=torch.int32, device=cuda)
+    dr = torch.from_numpy(np.ascontiguousarray(rows[:2])).to(cuda)
+    for kw in (dict(draws=None), dict(draws=dr, row=word(8, cuda)), dict(draws=dr, row=word(-4, cuda))):
+        K.sample(dev(logits, cuda), kw.pop("draws"), tok, **kw)
+        assert int(tok.item()) == ops.sample_ref(logits, 0.0, 1, 0)
+    with pytest.raises(Exception, match="k_max"):
+        K.sample(dev(logits, cuda), dr, tok, k_max=65)
+
+
 def test_eval_words_advances_a_decode_step(cuda):
     words = torch.tensor([11, 40, 0, 0, 0, 0, 0, 0], dtype=torch.int32, device=cuda)
     # position += 1; kv_valid = position + 1; rope_row = min(position, 5); half = position >> 1

@@ -100,6 +100,21 @@ def test_generate_replays_the_captured_step_and_matches_stepwise_decode(toy):
     assert list(host.session.draw(prompt, 6, each=True)) == replayed[:6]
 
 
+def test_sampled_tokens_are_the_host_s_token_for_token(toy):
+    """Drawn on the device from the sampler's rows (one replayed HIP graph), then drawn again on the
+    host from each step's logits at the same seed: the same tokens (iron/lm/testing.py:169-179)."""
+    from iron_amd.lm.generation import Sampler, generate_on_host
+
+    prompt = np.random.default_rng(13).integers(0, SCALED.vocab_size, 40)
+    drawn = toy.generate(prompt, 24, Sampler(1.5, 50, seed=4))
+    assert drawn == list(toy.session.draw(prompt, 24, Sampler(1.5, 50, seed=4), each=True))
+    assert drawn == generate_on_host(toy, prompt, 24, Sampler(1.5, 50, seed=4))
+    assert drawn != toy.generate(prompt, 24, Sampler(1.5, 50, seed=5))
+    # A greedy run after a sampled one finds its rows zero again.
+    greedy = toy.generate(prompt, 24)
+    assert greedy == generate_on_host(toy, prompt, 24, Sampler(0.0)) and greedy != drawn
+
+
 def test_check_mode_judges_every_step_against_its_reference(cuda):
     model = Llama(SCALED, weights())
     model.load_versions(check=True)

@@ -149,3 +149,18 @@ def test_a_bias_changes_the_logits():
     zeroed = {n: (np.zeros_like(a) if n.endswith("bias") else a) for n, a in w.items()}
     got = host(BIASED, zeroed).logits(prompt)
     assert np.abs(np.asarray(got, np.float32).reshape(-1) - first).max() > 0.05 * np.abs(first).max()
+
+
+def test_a_sampler_s_rows_draw_on_the_graph_what_the_sampler_draws_on_the_host(w):
+    """``generate`` with a sampler writes one draw row per position ahead of time and the graph's
+    Sample draws from them; the same sampler called on each step's logits draws the same tokens
+    (iron/lm/testing.py:169-179)."""
+    from iron_amd.lm.generation import Sampler, generate_on_host
+
+    prompt = np.random.default_rng(12).integers(0, SCALED.vocab_size, 8)
+    model = host(SCALED, w)
+    drawn = model.generate(prompt, 5, Sampler(1.5, 50, seed=2))
+    assert drawn == generate_on_host(model, prompt, 5, Sampler(1.5, 50, seed=2))
+    greedy = model.generate(prompt, 5)
+    assert greedy == generate_on_host(model, prompt, 5, Sampler(0.0))
+    assert drawn != greedy   # at this temperature the toy's flat logits do not keep to the top token

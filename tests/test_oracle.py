@@ -231,6 +231,103 @@ def test_gather_and_argmax():
     assert ops.argmax(logits) == 1  # first of the ties
 
 
+# -------------------------------------------------------------------- sampling
+# The draw with a temperature is this build's own definition (the reference's sample_ref is not
+# in its tree), so it is pinned to what the mathematics fixes: exp, softmax, an exact cumulative walk.
+def test_exp_det_is_exp_to_an_ulp():
+    rng = np.random.default_rng(0)
+    zs = np.concatenate([-rng.random(5000) * 40, -rng.random(500) * 690, [0.0, -0.0, -1e-300, -690.0, -0.34657359]])
+    worst = max(abs(ops.exp_det(float(z)) - math.exp(z)) / math.exp(z) for z in zs)
+    assert worst < 4e-16
+    assert ops.exp_det(0.0) == 1.0
+    assert ops.exp_det(-690.1) == 0.0 and ops.exp_det(-math.inf) == 0.0 and ops.exp_det(math.nan) == 0.0
+
+
+def test_sample_order_and_greedy():
+    x = np.array([1.0, 5.0, np.nan, 5.0, -np.inf, -0.0, 0.0, 7.0, 7.0], np.float32)
+    # Larger first, of equals the lower index (-0 equals +0), NaN last.
+    assert ops.sample_order(x).tolist() == [7, 8, 1, 3, 0, 5, 6, 4, 2]
+    assert ops.sample_ref(x, 0.0, 50, 12345) == 7
+    assert ops.sample_ref(x, 0.7, 1, (1 << 53) - 1) == 7          # top-1 is greedy whatever the number
+    assert ops.sample_ref(x, 0.7, 50, 0) == 7                     # the number 0 draws the best
+    assert ops.sample_ref(x, 1e-3, 50, (1 << 52) - 1) == 7        # u just under 1/2, two equal bests
+    assert ops.sample_ref(x, 1e-3, 50, 1 << 52) == 8              # u = 1/2: the second of them
+    # A best logit that is not finite draws itself; NaN and -inf candidates weigh nothing.
+    assert ops.sample_ref(np.array([1.0, np.inf, 3.0], np.float32), 0.7, 3, 1 << 52) == 1
+    assert ops.sample_ref(np.array([np.nan, -np.inf, 3.0], np.float32), 0.7, 3, (1 << 53) - 1) == 2
+
+
+def test_sample_weights_are_the_top_k_softmax():
+    from scipy.special import softmax
+
+    rng = np.random.default_rng(5)
+    x = round_bf16(rng.normal(0, 3, 2000))
+    for t, k in [(0.7, 50), (1.0, 7), (0.05, 64), (5.0, 33)]:
+        cand, w = ops.sample_weights(x, t, k)
+        assert cand.tolist() == sorted(range(x.size), key=lambda i: (-x[i], i))[:k]
+        want = softmax(x[cand].astype(np.float64) / float(np.float32(t)))
+        assert np.allclose(w / w.sum(), want, rtol=1e-13, atol=0)
+    # k_max caps top_k; a top_k past the row keeps the row.
+    assert ops.sample_weights(x, 0.7, 500, k_max=64)[0].size == 64
+    assert ops.sample_weights(x[:10], 0.7, 50)[0].size == 10
+
+
+def test_sample_ref_walks_the_cumulative_weights():
+    from fractions import Fraction
+
+    rng = np.random.default_rng(6)
+    x = round_bf16(rng.normal(0, 2, 512))
+    x[[3, 77, 78]] = x.max()   # ties at the top, in index order
+    for t, k in [(0.7, 50), (1.5, 64), (0.3, 5)]:
+        cand, w = ops.sample_weights(x, t, k)
+        cum = np.cumsum([Fraction(float(v)) for v in w])
+        seen = set()
+        for n53 in rng.integers(0, 1 << 53, 400):
+            u = Fraction(int(n53), 1 << 53)
+            want = next(i for i, c in enumerate(cum) if c > u * cum[-1])
+            got = ops.sample_ref(x, t, k, int(n53))
+            assert got == cand[want]
+            seen.add(want)
+        assert len(seen) > 1
+        # Either side of the first boundary: the number just under w0/total draws the best, the
+        # next but one draws its neighbour.
+        edge = int(Fraction(float(w[0])) / cum[-1] * (1 << 53))
+        assert ops.sample_ref(x, t, k, edge - 1) == cand[0]
+        assert ops.sample_ref(x, t, k, edge + 1) == cand[1]
+
+
+def test_draw_row_words_round_trip():
+    from iron_amd.operators.sample import draw_row
+
+    row = draw_row(0.7, 50, (1 << 53) - 12345)
+    assert row.dtype == np.int32 and row.shape == (4,)
+    t, k, n = ops.draw_words(row)
+    assert t == np.float32(0.7) and k == 50 and n == (1 << 53) - 12345
+    assert ops.draw_words(np.zeros(4, np.int32)) == (0.0, 1, 0)
+    with pytest.raises(ValueError, match="53-bit"):
+        draw_row(0.7, 50, 1 << 53)
+
+
+def test_sampler_draws_what_its_rows_draw():
+    import oracle
+    from iron_amd.lm.generation import Sampler
+
+    oracle.install()
+    rng = np.random.default_rng(8)
+    x = round_bf16(rng.normal(0, 3, 4096))
+    host, device = Sampler(0.7, 50, seed=3), Sampler(0.7, 50, seed=3)
+    rows = device.rows(20, 64)
+    for r in rows:
+        assert host(x) == ops.sample_ref(x, *ops.draw_words(r), 64)
+    probs = Sampler(0.7, 50).probabilities(x)
+    assert abs(probs.sum() - 1) < 1e-12 and np.count_nonzero(probs) == 50
+    assert Sampler(0.0, 50).probabilities(x).argmax() == x.argmax()
+    with pytest.raises(ValueError, match="not one the device draws"):
+        Sampler(0.7, None).rows(1, 64)
+    with pytest.raises(ValueError, match="negative"):
+        Sampler(-1.0)
+
+
 # ----------------------------------------------------------------- RoPE tables
 def test_rope_angles_closed_forms():
     t = ops.rope_angles(64, 128, 500000.0)
