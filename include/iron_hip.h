@@ -116,6 +116,40 @@ int iron_silu_mul_bf16(const uint16_t* g, const uint16_t* u, uint16_t* y, int64_
 int iron_row_broadcast_bf16(const uint16_t* x, const uint16_t* row, uint16_t* y, int rows, int cols,
                             int multiply, const int* valid, void* stream);
 
+/* y[i] = bf16(f(x[i])) for i < *valid (or n), f32 math, one rounding; kind names f:
+ * GELU by its tanh approximation or exact (x Phi(x)), ReLU, sigmoid, tanh, or the clamp to
+ * [p0, p1] (p0, p1 are read by the clamp alone; the caller rounds them to bf16).
+ * Replaces GELU / ReLU / Sigmoid / Tanh / Clamp: iron/operators/gelu.py:13, relu.py:11,
+ * sigmoid.py:9, tanh.py:9, clamp.py:14 (each a UnaryElementwise, iron/common/elementwise.py:494). */
+#define IRON_UNARY_GELU_TANH 0
+#define IRON_UNARY_GELU_ERF 1
+#define IRON_UNARY_RELU 2
+#define IRON_UNARY_SIGMOID 3
+#define IRON_UNARY_TANH 4
+#define IRON_UNARY_CLAMP 5
+int iron_unary_bf16(const uint16_t* x, uint16_t* y, int64_t n, int kind, float p0, float p1,
+                    const int* valid, void* stream);
+
+/* out[i] = bf16(a * x[i] + y[i]) for i < *valid (or n): one fused multiply-add in f32.
+ * Replaces AXPY: iron/operators/axpy.py:13. */
+int iron_axpy_bf16(const uint16_t* x, const uint16_t* y, uint16_t* out, int64_t n, float a,
+                   const int* valid, void* stream);
+
+/* y[r] = bf16((x[r] - mean) / sqrt(var + eps)) per row r < *valid (or rows), mean and the
+ * variance about it in f32 (beta 0); with w, that row times w rounded again, as RMSNorm.
+ * x,y (rows, cols); w (cols) or NULL.  cols % 8 == 0.
+ * Replaces LayerNorm: iron/operators/layer_norm.py:10 over iron/common/elementwise.py:676-682. */
+int iron_layernorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int rows, int cols,
+                        float eps, const int* valid, void* stream);
+
+/* y[r, c] = softmax over the first *length (or cols) columns of row r, 0 in the columns past them:
+ * z = x + addend (addend float32 or NULL), capped as soft_cap * tanh(z / soft_cap) when
+ * soft_cap > 0, exp(z - max) / sum in f32, one rounding.  x (rows, cols) bf16, or float32 when
+ * x_is_f32; y (rows, cols) bf16.  cols % 8 == 0.
+ * Replaces Softmax without its band (window, period): iron/operators/softmax.py:62,523-545. */
+int iron_softmax_bf16(const void* x, int x_is_f32, const float* addend, uint16_t* y, int rows,
+                      int cols, float soft_cap, const int* length, void* stream);
+
 /* Attention, many queries (prefill / prompt chunk).  Q,O: (seq, heads, d) if q_interleaved
  * else (heads, seq, d); K,V: (kv_len, kv_heads, d) if kv_interleaved else (kv_heads, kv_len, d).
  * The queries are the last rows of the keys: query i sits at position kv_tokens - q_tokens + i,

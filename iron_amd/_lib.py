@@ -47,6 +47,10 @@ SIGNATURES = {
     "iron_gather_rows": (c_int, [_P, _P, _P, c_int, c_int, c_int64, _P, _P]),
     "iron_copy_rows": (c_int, [_P, _P, c_int, c_int64, c_int64, c_int64, c_int, c_int, _P, _P, _P, _P]),
     "iron_argmax_bf16": (c_int, [_P, c_int, _P, _P, c_int, _P, _P, _P]),
+    "iron_unary_bf16": (c_int, [_P, _P, c_int64, c_int, c_float, c_float, _P, _P]),
+    "iron_axpy_bf16": (c_int, [_P, _P, _P, c_int64, c_float, _P, _P]),
+    "iron_layernorm_bf16": (c_int, [_P, _P, _P, c_int, c_int, c_float, _P, _P]),
+    "iron_softmax_bf16": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_float, _P, _P]),
     "iron_sample_workspace_bytes": (c_int64, [c_int]),
     "iron_sample_bf16": (c_int, [_P, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P]),
     "iron_eval_words": (c_int, [_P, c_int, _P, c_int, _P]),

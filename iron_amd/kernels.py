@@ -191,6 +191,47 @@ def silu(x, y, *, n=None, valid=None):
     check(lib().iron_silu_bf16(ptr(x), ptr(y), n, ptr(_word(valid, "valid")), current_stream()), "iron_silu_bf16")
 
 
+UNARY = {"gelu_tanh": 0, "gelu_erf": 1, "relu": 2, "sigmoid": 3, "tanh": 4, "clamp": 5}
+
+
+def unary(x, y, kind, *, n=None, low=0.0, high=0.0, valid=None):
+    """``y = f(x)``, ``kind`` one of ``UNARY``; ``low`` and ``high`` are the clamp's bounds."""
+    n = y.numel() if n is None else n
+    _numel(_dev(x, "x"), n, "x")
+    _numel(_dev(y, "y"), n, "y")
+    check(lib().iron_unary_bf16(ptr(x), ptr(y), n, UNARY[kind], float(low), float(high), ptr(_word(valid, "valid")),
+                                current_stream()), "iron_unary_bf16")
+
+
+def axpy(x, y, out, *, a, n=None, valid=None):
+    n = out.numel() if n is None else n
+    _numel(_dev(x, "x"), n, "x")
+    _numel(_dev(y, "y"), n, "y")
+    _numel(_dev(out, "out"), n, "out")
+    check(lib().iron_axpy_bf16(ptr(x), ptr(y), ptr(out), n, float(a), ptr(_word(valid, "valid")), current_stream()),
+          "iron_axpy_bf16")
+
+
+def layernorm(x, w, y, *, rows, cols, eps, valid=None):
+    _numel(_dev(x, "x"), rows * cols, "x")
+    _numel(_dev(y, "y"), rows * cols, "y")
+    if w is not None:
+        _numel(_dev(w, "weight"), cols, "weight")
+    check(lib().iron_layernorm_bf16(ptr(x), ptr(w), ptr(y), rows, cols, float(eps), ptr(_word(valid, "valid")),
+                                    current_stream()), "iron_layernorm_bf16")
+
+
+def softmax(x, y, *, rows, cols, addend=None, soft_cap=None, length=None):
+    """Softmax of each row of ``x`` (bf16 or float32) over its first ``length`` columns (a device word)."""
+    f32 = x.dtype == torch.float32
+    _numel(_dev(x, "x", torch.float32 if f32 else torch.bfloat16), rows * cols, "x")
+    _numel(_dev(y, "y"), rows * cols, "y")
+    if addend is not None:
+        _numel(_dev(addend, "addend", torch.float32), rows * cols, "addend")
+    check(lib().iron_softmax_bf16(ptr(x), int(f32), ptr(addend), ptr(y), rows, cols, float(soft_cap or 0.0),
+                                  ptr(_word(length, "length")), current_stream()), "iron_softmax_bf16")
+
+
 def mha_prefill(
     Q, K, V, O, *, heads, kv_heads, d, seq, seq_len=None, kv_len, scale=None, causal=True,
     window=None, q_interleaved=False, kv_interleaved=False, valid=None, kv_valid=None,

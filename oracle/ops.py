@@ -25,7 +25,8 @@ Pinned by (see tests/test_oracle.py):
               rationals, top_k = 1 / n53 = 0 = greedy
 Parity unpinned (arithmetic lives in mlir-aie 1.4.6.dev15, absent here; textbook
 formula used, bounded by the stated bf16 tolerance and the model-level goldens):
-  rms_norm inner summation order / rsqrt, silu (LUT kernel), mul;
+  rms_norm inner summation order / rsqrt, silu (LUT kernel), mul; gelu, sigmoid, tanh (table
+  kernels), axpy, layer_norm, softmax -- each checked against a float64 library routine instead;
   sample_ref with temperature > 0 (aie.iron.kernels.sample.sample_ref): which token
   a given 53-bit number draws is this build's own definition, stated at sample_ref.
 """
@@ -99,6 +100,78 @@ def silu(x):
     """``x * sigmoid(x)`` in float32, rounded once (silu.py:12; LUT kernel -- parity unpinned)."""
     x = _f32(x)
     return round_bf16(x / (np.float32(1.0) + np.exp(-x)))
+
+
+def gelu(x, approximate="tanh"):
+    """GELU in float32, rounded once: ``0.5 x (1 + tanh(sqrt(2/pi)(x + 0.044715 x^3)))``, or exact
+    ``x Phi(x)`` (gelu.py:13-40, torch's ``approximate``; the reference's kernels are a table and an
+    erf of mlir-aie -- parity unpinned)."""
+    x = _f32(x)
+    if approximate == "none":
+        from scipy.special import erf
+
+        return round_bf16(np.float32(0.5) * x * (np.float32(1.0) + erf(x * np.float32(0.7071067811865476)).astype(np.float32)))
+    inner = np.float32(0.7978845608028654) * (x + np.float32(0.044715) * x * x * x)
+    return round_bf16(np.float32(0.5) * x * (np.float32(1.0) + np.tanh(inner)))
+
+
+def relu(x):
+    """``max(x, 0)`` (relu.py:11; pinned bit-exact with an add by test_elementwise.py:125-132)."""
+    return np.maximum(_f32(x), np.float32(0.0))
+
+
+def sigmoid(x):
+    """``1 / (1 + exp(-x))`` in float32, rounded once (sigmoid.py:9; table kernel -- parity unpinned)."""
+    return round_bf16(np.float32(1.0) / (np.float32(1.0) + np.exp(-_f32(x))))
+
+
+def tanh(x):
+    """``tanh(x)`` in float32, rounded once (tanh.py:9; table kernel -- parity unpinned)."""
+    return round_bf16(np.tanh(_f32(x)))
+
+
+def clamp(x, low, high):
+    """``x`` clamped to ``[low, high]``, the bounds rounded to bf16 (clamp.py:14-63): exact."""
+    lo, hi = round_bf16(np.array([low, high], np.float32))
+    return np.minimum(np.maximum(_f32(x), lo), hi)
+
+
+def axpy(a, x, y):
+    """``a x + y``: the product exact in float64, the sum rounded to float32 (a fused multiply-add),
+    then to bf16 (axpy.py:13-31 over datamovement.axpy -- parity unpinned)."""
+    fused = (np.float64(np.float32(a)) * _f32(x).astype(np.float64) + _f32(y).astype(np.float64)).astype(np.float32)
+    return round_bf16(fused)
+
+
+def layer_norm(x, weight=None, *, epsilon=1e-5):
+    """Each row less its mean over its standard deviation (beta 0), rounded to bf16; then times
+    ``weight``, rounded again (layer_norm.py:10-20; structure from elementwise.py:676-682; the row
+    formula is the textbook one, torch's -- parity unpinned)."""
+    x = _f32(x)
+    mean = np.mean(x, axis=-1, keepdims=True, dtype=np.float32)
+    centred = x - mean
+    var = np.mean(centred * centred, axis=-1, keepdims=True, dtype=np.float32)
+    normed = round_bf16(centred * (np.float32(1.0) / np.sqrt(var + np.float32(epsilon))).astype(np.float32))
+    if weight is None:
+        return normed
+    return round_bf16(normed * _f32(weight).reshape(-1))
+
+
+def softmax(x, addend=None, *, soft_cap=None, length=None):
+    """Softmax of each row over its first ``length`` columns, the rest zero (softmax.py:523-545 over
+    activation.softmax_ref -- parity unpinned): ``z = x + addend``, capped as ``cap tanh(z / cap)``,
+    ``exp(z - max) / sum`` in float32, one rounding."""
+    x = np.asarray(x, dtype=np.float32)
+    n = x.shape[-1] if length is None else int(length)
+    z = x[..., :n]
+    if addend is not None:
+        z = z + np.asarray(addend, dtype=np.float32)[..., :n]
+    if soft_cap is not None:
+        z = np.float32(soft_cap) * np.tanh(z / np.float32(soft_cap))
+    e = np.exp(z - z.max(axis=-1, keepdims=True))
+    out = np.zeros(x.shape, np.float32)
+    out[..., :n] = round_bf16(e / e.sum(axis=-1, keepdims=True, dtype=np.float32))
+    return out
 
 
 def mul(a, b):

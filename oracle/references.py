@@ -39,6 +39,46 @@ def add(op, a, b):
     return ops.add(a, np.asarray(b).reshape(np.shape(a)))
 
 
+def gelu(op, x):
+    """iron/operators/gelu.py:13-40."""
+    return ops.gelu(x, op.approximate)
+
+
+def relu(op, x):
+    return ops.relu(x)
+
+
+def sigmoid(op, x):
+    return ops.sigmoid(x)
+
+
+def tanh(op, x):
+    return ops.tanh(x)
+
+
+def clamp(op, x):
+    """iron/operators/clamp.py:14-63."""
+    return ops.clamp(x, op.low, op.high)
+
+
+def axpy(op, a, b):
+    """iron/operators/axpy.py:13-31: ``scalar_factor * a + b``."""
+    return ops.axpy(op.scalar_factor, a, np.asarray(b).reshape(np.shape(a)))
+
+
+def layer_norm(op, x, weight=None):
+    """iron/common/elementwise.py:676-682 over norm.layer_norm_eps."""
+    return ops.layer_norm(np.asarray(x).reshape(op.rows, op.tile_size), weight, epsilon=op.epsilon)
+
+
+def softmax(op, x, addend=None):
+    """iron/operators/softmax.py:523-545; a bounded call's ``length`` read off the operator."""
+    length = vars(op).get("_extents", {}).get("length")
+    return ops.softmax(np.asarray(x).reshape(op.rows, op.cols),
+                       None if addend is None else np.asarray(addend).reshape(op.rows, op.cols),
+                       soft_cap=op.soft_cap, length=length)
+
+
 def rowwise_add(op, x, row):
     """iron/common/elementwise.py:797-867 over eltwise.add_sized: every row plus the one row."""
     x = np.asarray(x).reshape(op.rows, op.tile_size)
@@ -86,6 +126,8 @@ def install() -> None:
     REFERENCES.update(
         GEMM=gemm, GEMV=gemv, RMSNorm=rms_norm, SiLU=silu, ElementwiseMul=mul, ElementwiseAdd=add,
         RoPE=rope, MHA=mha, Copy=copy, Sample=sample, RowwiseAdd=rowwise_add, RowwiseMul=rowwise_mul,
+        GELU=gelu, ReLU=relu, Sigmoid=sigmoid, Tanh=tanh, Clamp=clamp, AXPY=axpy, LayerNorm=layer_norm,
+        Softmax=softmax,
         # The host's draw, for iron_amd.lm.generation.Sampler's checks.
         sample_ref=ops.sample_ref, sample_weights=ops.sample_weights,
     )

@@ -436,6 +436,81 @@ def test_argmax_first_of_ties_and_record(cuda):
     assert int(tok.item()) == ops.argmax(odd)
 
 
+# ---------------------------------------------- the sibling decoders' operators
+@pytest.mark.parametrize("kind,ref,exact", [
+    ("gelu_tanh", lambda x: ops.gelu(x), False), ("gelu_erf", lambda x: ops.gelu(x, "none"), False),
+    ("relu", ops.relu, True), ("sigmoid", ops.sigmoid, False), ("tanh", ops.tanh, False),
+    ("clamp", lambda x: ops.clamp(x, -0.75, 1.25), True)])
+def test_unary_kinds_and_their_bound(cuda, kind, ref, exact):
+    rng = np.random.default_rng(50)
+    x = bf(rng, 10007, scale=3.0)   # odd: a tail short of a 16-byte piece
+    y = out_like((10007,), cuda, fill=7.0)
+    K.unary(dev(x, cuda), y, kind, low=-0.75, high=1.25)
+    if exact:
+        assert np.array_equal(from_torch(y), ref(x))
+    else:
+        close(y, ref(x), rtol=2.0**-7, atol=1e-5)
+    # A bound read on the device leaves the rest as it was.
+    y.fill_(7.0)
+    K.unary(dev(x, cuda), y, kind, low=-0.75, high=1.25, valid=word(4001, cuda))
+    got = from_torch(y)
+    close(got[:4001], ref(x)[:4001], rtol=2.0**-7, atol=1e-5)
+    assert np.all(got[4001:] == 7.0)
+
+
+def test_axpy_and_its_bound(cuda):
+    rng = np.random.default_rng(51)
+    x, y = bf(rng, 70001, scale=4.0), bf(rng, 70001, scale=4.0)
+    out = out_like((70001,), cuda, fill=7.0)
+    for a in (3.0, 1.003, -0.5):
+        K.axpy(dev(x, cuda), dev(y, cuda), out, a=a)
+        assert np.array_equal(from_torch(out), ops.axpy(a, x, y))   # one fma, one rounding: exact
+    out.fill_(7.0)
+    K.axpy(dev(x, cuda), dev(y, cuda), out, a=3.0, valid=word(13, cuda))
+    got = from_torch(out)
+    assert np.array_equal(got[:13], ops.axpy(3.0, x, y)[:13]) and np.all(got[13:] == 7.0)
+
+
+@pytest.mark.parametrize("rows,cols,weighted", [(1, 2048, True), (33, 1024, False), (16, 4096, True), (5, 8192, True),
+                                                (3, 12288, True), (64, 768, True)])
+def test_layernorm_rows(cuda, rows, cols, weighted):
+    rng = np.random.default_rng(cols + rows)
+    x = round_bf16(bf(rng, rows, cols, scale=2.0) + np.float32(1.5))
+    w = round_bf16(rng.uniform(0.9, 1.1, cols).astype(np.float32)) if weighted else None
+    y = out_like((rows, cols), cuda, fill=7.0)
+    K.layernorm(dev(x, cuda), None if w is None else dev(w, cuda), y, rows=rows, cols=cols, eps=1e-5)
+    close(y, ops.layer_norm(x, w))
+    if rows > 2:
+        y.fill_(7.0)
+        K.layernorm(dev(x, cuda), None if w is None else dev(w, cuda), y, rows=rows, cols=cols, eps=1e-5,
+                    valid=word(2, cuda))
+        got = from_torch(y)
+        close(got[:2], ops.layer_norm(x, w)[:2])
+        assert np.all(got[2:] == 7.0)
+
+
+@pytest.mark.parametrize("rows,cols,f32,addend,cap", [(32, 1024, False, False, None), (16, 4608, False, False, None),
+                                                      (4, 32768, False, False, None), (32, 1024, True, False, None),
+                                                      (64, 1536, True, True, 50.0), (16, 80, True, True, None)])
+def test_softmax_rows_cap_addend_and_length(cuda, rows, cols, f32, addend, cap):
+    rng = np.random.default_rng(cols)
+    x = rng.normal(0, 4, (rows, cols)).astype(np.float32)
+    x = x if f32 else round_bf16(x)
+    add = rng.normal(0, 1, (rows, cols)).astype(np.float32) if addend else None
+    xd = torch.from_numpy(x).to(cuda) if f32 else dev(x, cuda)
+    ad = None if add is None else torch.from_numpy(add).to(cuda)
+    y = out_like((rows, cols), cuda, fill=7.0)
+    K.softmax(xd, y, rows=rows, cols=cols, addend=ad, soft_cap=cap)
+    close(y, ops.softmax(x, add, soft_cap=cap), rtol=1e-2, atol=1e-4)
+    assert abs(float(from_torch(y).sum(axis=-1).mean()) - 1.0) < 5e-3
+    # A length read on the device: the first columns' softmax, zeros after them.
+    n = cols // 3
+    K.softmax(xd, y, rows=rows, cols=cols, addend=ad, soft_cap=cap, length=word(n, cuda))
+    got = from_torch(y)
+    close(got, ops.softmax(x, add, soft_cap=cap, length=n), rtol=1e-2, atol=1e-4)
+    assert not got[:, n:].any()
+
+
 def _draw_rows(rng, count, temperatures=(0.0, 0.05, 0.7, 1.0, 5.0), k_hi=65):
     from iron_amd.operators.sample import draw_row
 

@@ -231,6 +231,78 @@ def test_gather_and_argmax():
     assert ops.argmax(logits) == 1  # first of the ties
 
 
+# ------------------------------------------------------- the sibling decoders' operators
+# Their kernels' references live in mlir-aie (parity unpinned there); each restatement is held to a
+# float64 library routine of the same function, within one rounding to bf16.
+def _within_a_bf16_step(got, want64, atol=2.0**-126):
+    """``atol``: what float32's own rounding leaves of a result that cancels (1 + erf(x) far in the tail)."""
+    want = round_bf16(want64.astype(np.float32))
+    step = np.maximum(np.abs(want) * 2.0**-7, atol)
+    assert np.all(np.abs(got - want) <= step), np.abs(got - want).max()
+    assert is_bf16_valued(got)
+
+
+def test_activations_match_float64_library_routines():
+    import torch
+
+    rng = np.random.default_rng(30)
+    x = bf(rng, 4096, scale=3.0)
+    x64 = torch.from_numpy(x.astype(np.float64))
+    _within_a_bf16_step(ops.gelu(x), torch.nn.functional.gelu(x64, approximate="tanh").numpy(), atol=1e-5)
+    _within_a_bf16_step(ops.gelu(x, "none"), torch.nn.functional.gelu(x64).numpy(), atol=1e-5)
+    _within_a_bf16_step(ops.sigmoid(x), torch.sigmoid(x64).numpy())
+    _within_a_bf16_step(ops.tanh(x), np.tanh(x.astype(np.float64)))
+    assert np.array_equal(ops.relu(x), np.where(x > 0, x, 0))
+    # The clamp's bounds are rounded to bf16 first: 1.003 is 1.0 there.
+    assert np.array_equal(ops.clamp(x, -0.75, 1.003), np.clip(x, -0.75, 1.0))
+    # GELU's two forms differ where the approximation does (about 1e-3 near |x| = 2), not elsewhere.
+    assert 1e-4 < np.abs(ops.gelu(x) - ops.gelu(x, "none")).max() < 2e-2
+
+
+def test_axpy_is_one_fused_multiply_add():
+    rng = np.random.default_rng(31)
+    x, y = bf(rng, 2048, scale=4.0), bf(rng, 2048, scale=4.0)
+    for a in (3.0, 1.003, -0.5):
+        want = np.float32(a).astype(np.float64) * x.astype(np.float64) + y.astype(np.float64)
+        _within_a_bf16_step(ops.axpy(a, x, y), want)
+    # The scalar stays float32: 1.003 is not 1.0 (it would be, rounded to bf16).
+    assert not np.array_equal(ops.axpy(1.003, x, y), ops.axpy(1.0, x, y))
+    assert np.array_equal(ops.axpy(1.0, x, y), ops.add(x, y))
+
+
+def test_layer_norm_matches_torch_in_float64():
+    import torch
+
+    rng = np.random.default_rng(32)
+    x = bf(rng, 6, 1024, scale=2.0) + np.float32(1.5)   # a mean to take away
+    x = round_bf16(x)
+    w = round_bf16(rng.uniform(0.9, 1.1, 1024).astype(np.float32))
+    x64 = torch.from_numpy(x.astype(np.float64))
+    plain = torch.nn.functional.layer_norm(x64, (1024,), eps=1e-5).numpy()
+    _within_a_bf16_step(ops.layer_norm(x), plain)
+    # Weighted: the normalised row is rounded before the multiply (two roundings).
+    assert np.array_equal(ops.layer_norm(x, w), round_bf16(ops.layer_norm(x) * w))
+    # Not RMSNorm: a constant added to a row changes nothing.
+    assert np.array_equal(ops.layer_norm(round_bf16(x[:1])), ops.layer_norm(x)[:1])
+    shifted = ops.layer_norm(x + np.float32(8.0))
+    assert np.abs(shifted - ops.layer_norm(x)).max() < 0.05 and np.abs(ops.rms_norm(x + np.float32(8.0)) - ops.rms_norm(x)).max() > 0.2
+
+
+def test_softmax_matches_scipy_with_its_cap_addend_and_length():
+    from scipy.special import softmax
+
+    rng = np.random.default_rng(33)
+    x = rng.normal(0, 4, (16, 512)).astype(np.float32)
+    addend = rng.normal(0, 1, (16, 512)).astype(np.float32)
+    _within_a_bf16_step(ops.softmax(x), softmax(x.astype(np.float64), axis=-1))
+    capped = 30.0 * np.tanh((x.astype(np.float64) + addend) / 30.0)
+    _within_a_bf16_step(ops.softmax(x, addend, soft_cap=30.0), softmax(capped, axis=-1))
+    short = ops.softmax(x, length=100)
+    _within_a_bf16_step(short[:, :100], softmax(x[:, :100].astype(np.float64), axis=-1))
+    assert not short[:, 100:].any()
+    assert np.allclose(ops.softmax(x).sum(axis=-1), 1.0, atol=5e-3)
+
+
 # -------------------------------------------------------------------- sampling
 # The draw with a temperature is this build's own definition (the reference's sample_ref is not
 # in its tree), so it is pinned to what the mathematics fixes: exp, softmax, an exact cumulative walk.
