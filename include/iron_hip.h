@@ -51,12 +51,13 @@ int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16_t* y, int 
 /* One-row fusions of a decoder layer (no single counterpart in the reference: each replaces a run
  * of its steps, iron/lm/blocks.py:627-648,697-699,723-733, and rounds where those steps round).
  *   y = E(W @ N(x)):  N = RMSNorm(x, eps) * norm_w when norm_w is not NULL (else x itself);
- *   epilogue 0: y = bf16(W N(x));  1: y = bf16(bf16(W N(x)) + residual);
+ *   epilogue 0: y = bf16(W N(x));  1: y = bf16(residual_scale * bf16(W N(x)) + residual), one fused
+ *   multiply-add (a scale of 1 is the plain sum; another is AXPY's, iron/lm/blocks.py:386-391);
  *   2: y = bf16(bf16(silu(bf16(W N(x)))) * bf16(W2 N(x)))   (gate, up -> SiLU -> Mul).
  * W, W2 (M,K); x, norm_w (K); residual, y (M).  K % 8 == 0. */
 int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const uint16_t* x,
-                         const uint16_t* norm_w, float eps, const uint16_t* residual, uint16_t* y,
-                         int M, int K, int epilogue, void* stream);
+                         const uint16_t* norm_w, float eps, const uint16_t* residual,
+                         float residual_scale, uint16_t* y, int M, int K, int epilogue, void* stream);
 
 /* Attention's first half for one token: n = RMSNorm(x) * norm_w; q = Wq n, k = Wk n, v = Wv n
  * (each rounded to bf16); q and k rotated by the RoPE row `angles` (d bf16, cos/sin interleaved,

@@ -197,16 +197,19 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 kw = dict(rows=M, hidden=gq.op.K, heads=gq.op.N // d, kv_heads=gk.op.N // d, d=d,
                           valid=word(gq.values.get("valid")))
                 got = Fused("prefill_qkv", i, 5, lambda a=args, kw=kw: kernels.prefill_qkv(**a, **kw))
-        elif gemv_row(s) and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseAdd":
+        elif gemv_row(s) and i + 1 < len(steps) and _name(steps[i + 1]) in ("ElementwiseAdd", "AXPY"):
             ad = steps[i + 1]
             c = s.outputs["C"]
             a, b = ad.inputs["a"], ad.inputs["b"]
-            other = a if _same(b, c) else (b if _same(a, c) else None)
+            if _name(ad) == "AXPY":   # scalar_factor * a + b: the GEMV's row is the one scaled
+                other, scale = (b if _same(a, c) else None), float(ad.op.scalar_factor)
+            else:
+                other, scale = (a if _same(b, c) else (b if _same(a, c) else None)), 1.0
             if other is not None and once(c) and _plain(other) and not ad.values and _plain(ad.outputs["y"]) \
                     and other.elements == c.elements:
                 args = dict(W=tensor(s.inputs["A"]), x=tensor(s.inputs["B"]).reshape(-1),
                             residual=tensor(other).reshape(-1), y=tensor(ad.outputs["y"]).reshape(-1))
-                kw = dict(M=s.op.M, K=s.op.K, epilogue=1)
+                kw = dict(M=s.op.M, K=s.op.K, epilogue=1, residual_scale=scale)
                 got = Fused("gemv_add", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
         if got is not None:
             fused.append(got)

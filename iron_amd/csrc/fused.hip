@@ -99,7 +99,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
                                                          const bf16_t* __restrict__ x,
                                                          const bf16_t* __restrict__ nw, float eps,
                                                          const bf16_t* __restrict__ res,
-                                                         bf16_t* __restrict__ y, int M, int K) {
+                                                         float res_scale, bf16_t* __restrict__ y,
+                                                         int M, int K) {
   constexpr int MATS = EPI == EPI_SILU_MUL ? 2 : 1;
   __shared__ float scratch4[4];
   __shared__ float part[4][MATS][RPW];
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
     const int r = threadIdx.x, row = row0 + r;
     if (row < M) {
       float v = round_bf16(part[0][0][r] + part[1][0][r] + part[2][0][r] + part[3][0][r]);  // the GEMV's own rounding
-      if (EPI == EPI_ADD) v = v + bf16_to_f32(res[row]);
+      if (EPI == EPI_ADD) v = fmaf(res_scale, v, bf16_to_f32(res[row]));   // scale 1: the plain sum
       if (EPI == EPI_SILU_MUL) {
         const float u = round_bf16(part[0][MATS - 1][r] + part[1][MATS - 1][r] + part[2][MATS - 1][r] +
                                    part[3][MATS - 1][r]);
@@ -198,7 +199,8 @@ using namespace iron;
 
 extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const uint16_t* x,
                                     const uint16_t* norm_w, float eps, const uint16_t* residual,
-                                    uint16_t* y, int M, int K, int epilogue, void* stream) {
+                                    float residual_scale, uint16_t* y, int M, int K, int epilogue,
+                                    void* stream) {
   IRON_REQUIRE(W && x && y, "gemv_fused: null operand");
   IRON_REQUIRE(M > 0 && K > 0 && K % 8 == 0, "gemv_fused: M (%d) positive, K (%d) a positive multiple of 8", M, K);
   IRON_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemv_fused: epilogue (%d) is 0, 1 or 2", epilogue);
@@ -216,7 +218,7 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
 #define IRON_FUSED(R, C, NRM, E)                                                                   \
   if (rpw == R && ch == C && norm == NRM && epilogue == E) {                                       \
     hipLaunchKernelGGL((gemv_fused_kernel<R, C, NRM, E>), dim3(blocks), dim3(256), 0, s, W, W2, x, \
-                       norm_w, eps, residual, y, M, K);                                            \
+                       norm_w, eps, residual, residual_scale, y, M, K);                            \
     IRON_LAUNCH_CHECK();                                                                           \
   }
 #define IRON_FUSED_NE(R, C)                                                                        \

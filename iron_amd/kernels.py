@@ -69,7 +69,7 @@ def gemv(W, x, y, *, M, K, batches=1, repeat=1, valid=None, rows_per_wave=0, k_s
     )
 
 
-def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, epilogue=0):
+def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, residual_scale=1.0, epilogue=0):
     """One-row fusion: ``[RMSNorm ->] GEMV [-> + residual | gate/up -> SiLU -> Mul]``."""
     _numel(_dev(W, "W"), M * K, "W")
     _numel(_dev(x, "x"), K, "x")
@@ -81,8 +81,8 @@ def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, e
     if residual is not None:
         _numel(_dev(residual, "residual"), M, "residual")
     check(
-        lib().iron_gemv_fused_bf16(ptr(W), ptr(W2), ptr(x), ptr(norm_w), float(eps), ptr(residual), ptr(y),
-                                   M, K, int(epilogue), current_stream()),
+        lib().iron_gemv_fused_bf16(ptr(W), ptr(W2), ptr(x), ptr(norm_w), float(eps), ptr(residual),
+                                   float(residual_scale), ptr(y), M, K, int(epilogue), current_stream()),
         "iron_gemv_fused_bf16",
     )
 

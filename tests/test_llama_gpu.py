@@ -231,6 +231,9 @@ def test_fused_kernels_against_the_oracle_at_llama_1b_width(cuda):
     y = torch.empty(E, dtype=torch.bfloat16, device=cuda)
     K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, residual=dev(x), epilogue=1)
     close(y, ops.add(x, ops.gemv(Wd, want_m)))
+    # ... and with the residual's multiplier (AXPY's one fused multiply-add)
+    K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, residual=dev(x), residual_scale=0.22, epilogue=1)
+    close(y, ops.axpy(0.22, ops.gemv(Wd, want_m), x))
     # the head: norm then projection
     for rows in (4096, 10000, 128256):  # one, two and four rows a wave
         Wh = bf(rows, E, scale=0.02)
