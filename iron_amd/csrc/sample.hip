@@ -42,6 +42,16 @@ __device__ __forceinline__ uint64_t shfl_xor64(uint64_t v, int o) {
   return ((uint64_t)hi << 32) | lo;
 }
 
+// The blocks' lists cross from one XCD's block to another's through device-scope atomic stores and
+// loads (written through and read past the XCD's own L2), which costs less than a fence's
+// write-back and invalidation of the whole L2 on either side of the ticket.
+__device__ __forceinline__ void publish(uint64_t* where, uint64_t e) {
+  __hip_atomic_store(where, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t collect(const uint64_t* where) {
+  return __hip_atomic_load(where, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 struct SampleShared {
   __align__(16) uint64_t best[SAMPLE_THREADS];   // each thread's best entry
   __align__(16) uint64_t list[SAMPLE_LIST];
@@ -192,7 +202,7 @@ __device__ double exp_det(double z) {
 // lists: gridDim.x lists of SAMPLE_K_MAX entries, from each block's best, 0 past its last.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const bf16_t* __restrict__ logits, int n, const int* __restrict__ draws, int draws_words,
-    const int* __restrict__ row, int k_max, uint64_t* __restrict__ lists, int* __restrict__ token,
+    const int* __restrict__ row, int k_max, uint64_t* lists, int* __restrict__ token,
     int* __restrict__ record, int record_len, const int* __restrict__ at,
     int* __restrict__ token_copy) {
   __shared__ SampleShared sh;
@@ -242,24 +252,26 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     own([&](uint64_t e) { best = e > best ? e : best; });
     best = block_max(best, sh);
     if (threadIdx.x == 0) sh.cand[0] = best;
-    if (blocks > 1 && threadIdx.x == 0) lists[(size_t)blockIdx.x * SAMPLE_K_MAX] = best;
+    if (blocks > 1 && threadIdx.x == 0) publish(&lists[(size_t)blockIdx.x * SAMPLE_K_MAX], best);
   } else {
     select_best(k, sh, own);
     if (blocks > 1 && threadIdx.x < SAMPLE_K_MAX)
-      lists[(size_t)blockIdx.x * SAMPLE_K_MAX + threadIdx.x] = sh.cand[threadIdx.x];
+      publish(&lists[(size_t)blockIdx.x * SAMPLE_K_MAX + threadIdx.x], sh.cand[threadIdx.x]);
   }
   if (blocks > 1) {
-    // The lists are out; the block whose ticket is the last goes on with all of them.
-    __threadfence();
+    // The lists are out (each thread has waited for its own stores); the block whose ticket is
+    // the last goes on with all of them.
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (threadIdx.x == 0) sh.last_block = atomicAdd(&sample_ticket, 1u) == (unsigned)blocks - 1;
+    if (threadIdx.x == 0)
+      sh.last_block = __hip_atomic_fetch_add(&sample_ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                      (unsigned)blocks - 1;
     __syncthreads();
     if (!sh.last_block) return;
-    __threadfence();
     if (k == 1) {
       uint64_t best = 0;
       for (int b = threadIdx.x; b < blocks; b += SAMPLE_THREADS) {
-        const uint64_t e = lists[(size_t)b * SAMPLE_K_MAX];
+        const uint64_t e = collect(&lists[(size_t)b * SAMPLE_K_MAX]);
         best = e > best ? e : best;
       }
       best = block_max(best, sh);
@@ -275,7 +287,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       for (int i = 0; i < HOLD; ++i) {
         const int slot = threadIdx.x + SAMPLE_THREADS * i;
         const int b = slot / stride, r = slot - b * stride;
-        held[i] = (slot < slots && r < k) ? lists[(size_t)b * SAMPLE_K_MAX + r] : 0;
+        held[i] = (slot < slots && r < k) ? collect(&lists[(size_t)b * SAMPLE_K_MAX + r]) : 0;
       }
       select_best(k, sh, [&](auto&& f) {
 #pragma unroll
@@ -283,7 +295,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
           if (held[i] != 0) f(held[i]);
         for (int slot = threadIdx.x + SAMPLE_THREADS * HOLD; slot < slots; slot += SAMPLE_THREADS) {
           const int b = slot / stride, r = slot - b * stride;
-          const uint64_t e = r < k ? lists[(size_t)b * SAMPLE_K_MAX + r] : 0;
+          const uint64_t e = r < k ? collect(&lists[(size_t)b * SAMPLE_K_MAX + r]) : 0;
           if (e != 0) f(e);
         }
       });
