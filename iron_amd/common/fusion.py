@@ -14,6 +14,7 @@ round:
 and, in a prompt chunk's version (several rows, 64-wide heads),
 
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
+  SiLU, ElementwiseMul (the gated feed-forward)          => iron_silu_mul_bf16
 
 A run is fused only if every intermediate it hides is read by nothing else.
 """
@@ -197,6 +198,19 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 kw = dict(rows=M, hidden=gq.op.K, heads=gq.op.N // d, kv_heads=gk.op.N // d, d=d,
                           valid=word(gq.values.get("valid")))
                 got = Fused("prefill_qkv", i, 5, lambda a=args, kw=kw: kernels.prefill_qkv(**a, **kw))
+        elif _name(s) == "SiLU" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseMul":
+            # a gated feed-forward's activation and gate over many rows: one pass instead of two
+            m = steps[i + 1]
+            act = s.outputs["y"]
+            a, b = m.inputs["a"], m.inputs["b"]
+            other = b if _same_view(a, act) else (a if _same_view(b, act) else None)
+            flat = all(h.index is None and h.ids is None for h in (s.inputs["x"], act, a, b, m.outputs["y"]))
+            if (other is not None and flat and once(act) and s.op.size == m.op.size
+                    and s.values.get("valid") == m.values.get("valid") and other.elements == act.elements):
+                args = dict(a=tensor(s.inputs["x"]).reshape(-1), b=tensor(other).reshape(-1),
+                            y=tensor(m.outputs["y"]).reshape(-1))
+                kw = dict(n=s.op.size, valid=word(m.values.get("valid")))
+                got = Fused("silu_mul", i, 2, lambda a=args, kw=kw: kernels.silu_mul(**a, **kw))
         elif gemv_row(s) and i + 1 < len(steps) and _name(steps[i + 1]) in ("ElementwiseAdd", "AXPY"):
             ad = steps[i + 1]
             c = s.outputs["C"]
