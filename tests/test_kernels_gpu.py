@@ -100,6 +100,21 @@ def test_gemm_layouts(cuda, b_col_maj, c_col_maj):
     assert np.all(np.abs(from_torch(C) - want) <= bound)
 
 
+@pytest.mark.parametrize("n", [4096, 8192])
+def test_gemm_large_squares_on_sampled_rows(cuda, n):
+    """The 256 x 256-tile kernel at the benchmark's large squares: a sample of rows (tile edges and
+    random ones) of the product against float64 dot products, and nothing left unwritten."""
+    rng = np.random.default_rng(n)
+    A, B = bf(rng, n, n, scale=0.02), bf(rng, n, n, scale=0.02)   # B is (N, K)
+    C = out_like((n, n), cuda, fill=float("nan"))
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=n, N=n, K=n, b_col_maj=True)
+    got = from_torch(C)
+    assert not np.isnan(got).any()
+    rows = sorted({0, 1, 127, 128, 255, 256, 257, n // 2 - 1, n // 2, n - 256, n - 1, *rng.integers(0, n, 21).tolist()})
+    want = round_bf16((A[rows].astype(np.float64) @ B.astype(np.float64).T).astype(np.float32))
+    close(got[rows], want, rtol=1e-2, atol=1e-3)
+
+
 def test_gemm_headline_shape(cuda):
     rng = np.random.default_rng(4)
     A, B = bf(rng, 2048, 2048, scale=0.02), bf(rng, 2048, 2048, scale=0.02)
@@ -287,6 +302,26 @@ def run_prefill(cuda, Q, Kc, Vc, *, H, G, d, seq, seq_len, kv_len, causal=True, 
                    causal=causal, window=window, scale=scale, heads_interleaved=interleaved,
                    kv_interleaved=interleaved, valid=valid, kv_valid=kv_valid)
     return from_torch(O), want
+
+
+def test_mha_prefill_longest_shape_on_sampled_queries(cuda):
+    """S = 8192 (the longest of the benchmark's shapes): the whole output would take the oracle
+    minutes, so every head of a sample of queries -- tile edges, both ends, random rows -- is
+    checked against the oracle's attention of that one query over its keys."""
+    rng = np.random.default_rng(12)
+    S, H, G, d = 8192, 32, 8, 64
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    O = out_like(Q.shape, cuda, fill=float("nan"))
+    K.mha_prefill(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, seq=S, seq_len=S,
+                  kv_len=S, scale=0.125, causal=True, q_interleaved=True, kv_interleaved=True)
+    got = from_torch(O)
+    assert not np.isnan(got).any()
+    rows = sorted({0, 1, 63, 64, 127, 128, 129, 4095, 4096, 8063, 8064, 8191, *rng.integers(0, S, 12).tolist()})
+    for r in rows:
+        # The query at position r attends keys 0..r: the one-query form of the same operator.
+        want = ops.mha(Q[r : r + 1], Kc[: r + 1], Vc[: r + 1], num_heads=H, num_KV_heads=G, seq_len=1, kv_len=r + 1,
+                       d=d, causal=True, scale=0.125, heads_interleaved=True, kv_interleaved=True)
+        close(got[r : r + 1], want)
 
 
 @pytest.mark.parametrize("S", [512, 2048])
