@@ -86,6 +86,34 @@ def bench_gemm(torch, K, dev, steps, rng, b_col_maj, M=2048, N=2048, Kd=2048):
             "TFLOPs": round(flops / us / 1e6, 1), "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
+def bench_library_reference(torch, dev, n, rng):
+    """The vendor libraries on the same shapes and data, for scale (not this build's path, and
+    nothing here is compared for parity): ``torch.matmul`` (hipBLASLt / rocBLAS) on the GEMM shapes
+    with B as (N, K), and ``scaled_dot_product_attention`` on the prefill shapes."""
+    import torch.nn.functional as F
+
+    out = {"what": "torch.matmul and torch SDPA (vendor libraries), same shapes and data; for scale only",
+           "gemm_b_col_maj": [], "attention_prefill": []}
+    for M, N, Kd in ((2048, 2048, 2048), (2048, 8192, 2048), (4096, 4096, 4096), (8192, 8192, 8192)):
+        A = (torch.randn(M, Kd, device=dev) * 0.02).bfloat16()
+        B = (torch.randn(N, Kd, device=dev) * 0.02).bfloat16()
+        C = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+        us = graph_time_us(torch, [lambda: torch.matmul(A, B.t(), out=C)] * 10, max(1, n // 40))
+        out["gemm_b_col_maj"].append({"M": M, "N": N, "K": Kd, "us": round(us, 2),
+                                      "TFLOPs": round(2.0 * M * N * Kd / us / 1e6, 1)})
+    for S in (512, 2048, 8192):
+        q = torch.randn(1, 32, S, 64, device=dev).bfloat16()
+        k, v = (torch.randn(1, 8, S, 64, device=dev).bfloat16() for _ in range(2))
+        try:
+            us = graph_time_us(torch, [lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)] * 5,
+                               max(1, n // 40))
+            out["attention_prefill"].append({"S": S, "us": round(us, 2),
+                                             "TFLOPs": round(4.0 * 32 * 64 * S * (S + 1) / 2 / us / 1e6, 1)})
+        except Exception as e:  # a library without this shape is no failure of the bench
+            out["attention_prefill"].append({"S": S, "error": str(e)[:80]})
+    return out
+
+
 def bench_mfma_ceiling(torch, K, dev, rng):
     """What the MFMA units sustain from registers alone: with constant operands, and with operands
     drawn like the GEMM's (N(0,1)*0.02) -- under the power cap the clock depends on the data."""
@@ -419,6 +447,7 @@ def main():
         g["frac_sustained"] = round(g["TFLOPs"] / mfma_ceiling["random"], 4)
     pre_attention = bench_pre_attention(torch, K, dev, n)
     sample = bench_sample(torch, K, dev, n, rng)
+    library = bench_library_reference(torch, dev, n, rng)
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     decoder, cpu = bench_decoder(torch, dev, args.steps, args.warmup, not args.no_cpu)
@@ -456,6 +485,7 @@ def main():
         "attention": attention,
         "pre_attention_block": pre_attention,
         "sample": sample,
+        "library_reference": library,
         "bench_wall_s": round(wall, 1),
     }
     if cpu is not None:

@@ -449,23 +449,34 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
   };
   // A wave is alone on its SIMD, so nothing overlaps unless its own instruction stream interleaves:
   // each k-step's four MFMAs are issued with the next step's fragment reads and a quarter of the
-  // stage being prefetched between them.
+  // stage being prefetched between them.  The one barrier a stage needs sits before its LAST k-step,
+  // whose fragments are in registers by then: after it every wave's share of the next stage has
+  // landed and nobody reads this stage any more, so the next stage's first fragments are read under
+  // the last k-step's MFMAs (no read latency is exposed where a stage begins) and the buffer of the
+  // stage before is free for the prefetch.
+  wait_vmcnt<(NT_STAGES - 2) * LOADS>();   // stage 0 has landed once only the two younger ones are out
+  block_barrier();
+  bf16x8 af[2][T], bfr[2][T];
+  TrFrag tf[2][T];
+  read_frags(smem_nt, 0, af[0], bfr[0], tf[0]);
   for (int kt = 0; kt < nk; ++kt) {
-    // Stage kt has landed once at most the two younger stages' loads are outstanding.
-    wait_vmcnt<(NT_STAGES - 2) * LOADS>();
-    block_barrier();  // everyone's loads of stage kt are in; everyone is done reading stage kt-1
     // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
     // (into buffers nobody reads any more) rather than branch: every iteration issues the same
-    // loads, which keeps the wait count above exact and the scheduling region whole.
+    // loads, which keeps the wait counts exact and the scheduling region whole.
     const int kn = min(kt + NT_STAGES - 1, nk - 1);
     char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
     const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
-    bf16x8 af[2][T], bfr[2][T];
-    TrFrag tf[2][T];
-    read_frags(st, 0, af[0], bfr[0], tf[0]);
+    const char* st1 = smem_nt + ((kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks == BK / 16 - 1) {
+        // This wave has every fragment of stage kt; of the loads in flight the oldest LOADS are
+        // stage kt+1's (then stage kt+2's, and the 3 T issued so far for stage kt+3).
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_vmcnt<LOADS + 3 * T>();
+        block_barrier();
+      }
       if constexpr (B_KN) {
         lds_tr_wait(tf[cur][0], tf[cur][T - 1]);
         bfr[cur][0] = tr_join(tf[cur][0]);
@@ -478,6 +489,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
         acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][i], acc[i][0], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (ks + 1 < BK / 16) read_frag_pair(st, ks + 1, i, af[nxt][i], bfr[nxt][i], tf[nxt][i]);
+        else read_frag_pair(st1, 0, i, af[nxt][i], bfr[nxt][i], tf[nxt][i]);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (T == 2) {
           acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][1], af[cur][i], acc[i][1], 0, 0, 0);
@@ -609,7 +621,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
                                                          const int* __restrict__ valid, int tiles_m,
                                                          int tiles_n, int patched, int run_above,
                                                          int run_upto) {
-  static_assert(KB == 64 || (KB == 32 && WAVES == 4), "k per stage: 64, or 32 with 4 waves");
+  static_assert(KB == 64, "k per stage: 64 (32 with four stages of half-line rows measured 13 % slower)");
   constexpr int ROWB = KB * 2;               // bytes of a tile row in LDS
   constexpr int CPR = KB / 8;                // its 16-byte chunks
   constexpr int RPI = 1024 / ROWB;           // rows one 1 KB load covers
@@ -674,12 +686,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int nk = K / KB;
-  // STAGES-1 stages in flight before the loop (short K repeats its last stage), one more each
-  // iteration: the wait count in the loop is exact from the first iteration.
+  static_assert(KB == 64, "the loop below is written for two 64-wide stages");
+  // A stage's 2 INST loads go out in two halves of INST: the first under the last k-step of the
+  // stage two before it (right after that stage's barrier freed the buffer), the second under the
+  // first k-step of the stage before it; two k-steps later, at that stage's barrier, all have landed.
+  auto issue_half = [&](char* st, int kt, int half, int slot) { issue_one(st, kt, half * INST + slot); };
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s)
+  for (int idx = 0; idx < 2 * INST; ++idx) issue_one(smem_big, 0, idx);
 #pragma unroll
-    for (int idx = 0; idx < 2 * INST; ++idx) issue_one(smem_big + s * STAGE_BYTES, min(s, nk - 1), idx);
+  for (int slot = 0; slot < INST; ++slot) issue_half(smem_big + STAGE_BYTES, min(1, nk - 1), 0, slot);
 
   const int fr = lane & 31, kh = lane >> 5;
   const int swz = (fr >> 1) & (CPR - 1);   // tile rows are multiples of 32 apart: one swizzle for all
@@ -692,37 +707,43 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
     for (int i = 0; i < TN; ++i) bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * ROWB + c);
   };
 
+  wait_vmcnt<INST>();   // stage 0 has landed once only stage 1's first half is out
+  block_barrier();
+  bf16x8 af[2][4], bfr[2][TN];
+  read_frags(smem_big, 0, af[0], bfr[0]);
   for (int kt = 0; kt < nk; ++kt) {
-    wait_vmcnt<(STAGES - 2) * 2 * INST>();   // this wave's share of stage kt has landed
-    block_barrier();   // so has everyone's; and everyone is done reading stage kt-1
-    // The next stage goes into the buffer stage kt-1 used.  The last iteration fetches its own
-    // stage again (into the idle buffer) rather than branch: a branch would end the scheduling
-    // region and undo the interleaving below.
-    const int kn = min(kt + STAGES - 1, nk - 1);
-    char* nst = smem_big + ((kt + STAGES - 1) % STAGES) * STAGE_BYTES;
-    const char* st = smem_big + (kt % STAGES) * STAGE_BYTES;
-    bf16x8 af[2][4], bfr[2][TN];
-    read_frags(st, 0, af[0], bfr[0]);
+    // Past the end the last stage is fetched again (into buffers nobody reads any more) rather than
+    // branch: a branch would end the scheduling region and undo the interleaving below.
+    const int k1 = min(kt + 1, nk - 1), k2 = min(kt + 2, nk - 1);
+    char* st = smem_big + (kt % STAGES) * STAGE_BYTES;          // this stage; then stage kt+2's buffer
+    char* nst = smem_big + ((kt + 1) % STAGES) * STAGE_BYTES;   // stage kt+1's
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-      const int c = (((ks + 1) * 2 + kh) ^ swz) << 4;
+      const bool last = ks + 1 == KSTEPS;
+      if (last) {
+        // The one barrier of the stage, before its last k-step (whose fragments are in registers):
+        // after it every wave's loads of stage kt+1 have landed and nobody reads stage kt any more.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_vmcnt<0>();
+        block_barrier();
+      }
+      const char* from = last ? nst : st;
+      const int c = (((last ? 0 : ks + 1) * 2 + kh) ^ swz) << 4;
       // Source order is issue order (nothing crosses a sched_barrier): after each MFMA one of the
-      // next k-step's fragment reads or one load of the next stage goes out while it runs.
+      // next k-step's fragment reads (the next stage's first, under the last k-step) or one load goes out.
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
-          if (j == 0 && ks + 1 < KSTEPS)
-            af[nxt][i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * ROWB + c);
-          if (j == 1 && ks + 1 < KSTEPS && i < TN)
-            bfr[nxt][i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * ROWB + c);
-          // The whole next stage is requested during the first two k-steps, so that its latency
-          // (about a microsecond when the lines come from beyond L2) hides under the other two.
-          if (KB == 64 ? (ks < 2 && (j & 1)) : (j == 1))
-            issue_one(nst, kn, KB == 64 ? ks * INST + i * (TN / 2) + (j >> 1) : ks * INST + i);
+          if (j == 0) af[nxt][i] = *reinterpret_cast<const bf16x8*>(from + a_row + i * 32 * ROWB + c);
+          if (j == 1 && i < TN) bfr[nxt][i] = *reinterpret_cast<const bf16x8*>(from + b_row + i * 32 * ROWB + c);
+          if (j & 1) {
+            if (last) issue_half(st, k2, 0, i * (TN / 2) + (j >> 1));
+            if (ks == 0) issue_half(nst, k1, 1, i * (TN / 2) + (j >> 1));
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
