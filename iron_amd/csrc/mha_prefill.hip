@@ -19,6 +19,7 @@ namespace iron {
 
 constexpr int BQ = 128;   // query rows per block
 constexpr int BKV = 64;   // key rows per tile
+constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks split each block's tiles over two halves
 
 // K and V tiles go straight from global memory into LDS (global_load_lds, no register staging), as
 // stored: [64 keys][D], STAGES tiles deep.  16-byte chunks of a row are XOR-swizzled so unpadded
@@ -29,8 +30,13 @@ constexpr int BKV = 64;   // key rows per tile
 // At least two waves a SIMD caps the register budget at 256, which makes the compiler keep MFMA
 // accumulators in ordinary VGPRs: the softmax reads S and rescales O in place instead of copying
 // every value out of (and back into) accumulation registers.
-template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mha_prefill_kernel(
+//
+// SPLIT = 2: eight waves; waves 4..7 serve the same four groups of 32 queries as waves 0..3 but take
+// the odd key tiles (their own loads, their own stage buffers), and the two halves' (max, sum, O)
+// are merged through LDS at the end.  A query block's chain of tiles is half as long, which is what
+// bounds a short sequence: its blocks are few and the one that sees every key finishes last.
+template <int D, int SPLIT>
+__global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(2))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -44,9 +50,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
   constexpr int STAGE = 2 * TILE;
   constexpr int INST = TILE / 1024 / 4;  // 1 KB loads of K (and of V) a wave issues per tile
   constexpr int RPI = 1024 / ROWB;       // rows one load covers
-  __shared__ __align__(1024) char smem[STAGES * STAGE];
+  extern __shared__ __align__(1024) char smem_all[];   // SPLIT * STAGES * STAGE bytes
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int half = (tid >> 6) >> 2, wave = (tid >> 6) & 3;   // which tiles, and which 32 queries
+  char* smem = smem_all + half * (STAGES * STAGE);            // this half's stage buffers
   const int col = lane & 31, g = lane >> 5;
   // Blocks are dispatched in id order, so the id runs over the query blocks from the last (under a
   // causal mask the heaviest: it sees the most keys) to the first, all heads of one query block
@@ -73,7 +81,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
   bf16_t* Oh = O + (size_t)head * q_head_stride;
   // Rows of this block past the bound: zeros.  A block wholly past it does only that.
   if (q0 >= q_tokens || offset < 0) {
-    for (int i = tid; i < BQ * CPR; i += 256) {
+    for (int i = tid; i < BQ * CPR; i += 256 * SPLIT) {
       const int r = q0 + i / CPR, c = (i % CPR) * 8;
       if (r < seq) *reinterpret_cast<uint4*>(Oh + (size_t)r * q_row_stride + c) = make_uint4(0, 0, 0, 0);
     }
@@ -107,6 +115,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
   int kv_lo = 0;
   if (window >= 0) kv_lo = max(0, offset + q0 - window) / BKV * BKV;
   const int ntiles = (kv_hi - kv_lo + BKV - 1) / BKV;
+  // This half's tiles are half, half + SPLIT, ...; both halves make the same number of steps (a
+  // block's waves share its barriers), the last of which may be past this half's last tile: it
+  // then loads the last tile again and computes nothing.
+  const int steps = (ntiles + SPLIT - 1) / SPLIT;
 
   if (ntiles > 0) {
     const bf16_t* Kh = K + (size_t)kvh * kv_head_stride;
@@ -144,7 +156,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     // Always STAGES-1 tiles in flight before the loop and one more each iteration (past the end
     // the last tile again, into a buffer nobody reads), so the wait counts below are exact.
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(min(s, ntiles - 1), s);
+    for (int s = 0; s < STAGES - 1; ++s) issue(min(s * SPLIT + half, ntiles - 1), s);
 
     // Fragment addressing.  K (A operand of S^T): lane reads key t*32 + col, chunk 2s + g.
     const int k_frag = col * ROWB, k_swz = (col >> 1) & 7;
@@ -161,11 +173,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     }
     const unsigned lds_base = (unsigned)(size_t)IRON_LDS_PTR(smem);
 
-    for (int tile = 0; tile < ntiles; ++tile) {
+    for (int step = 0; step < steps; ++step) {
+      const int tile = step * SPLIT + half;
       const int kv0 = kv_lo + tile * BKV;
       wait_vmcnt<(STAGES - 2) * 2 * INST>();   // this wave's share of the tile has landed
-      block_barrier();                          // everyone's has; everyone is done with tile - 1
-      const int buf = tile % STAGES;
+      block_barrier();                          // everyone's has; everyone is done with the step before
+      const int buf = step % STAGES;
+      if constexpr (SPLIT > 1) {
+        if (tile >= ntiles) {   // past this half's last tile: keep the loads (and the wait counts) going
+          issue(ntiles - 1, (step + STAGES - 1) % STAGES);
+          continue;
+        }
+      }
       {
         const char* kt = smem + buf * STAGE;
         const unsigned vt = lds_base + buf * STAGE + TILE;
@@ -192,7 +211,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
         }
         // The prefetch goes out while the score MFMAs run (its buffer, tile - 1's, is free since
         // the barrier above).
-        issue(min(tile + STAGES - 1, ntiles - 1), (tile + STAGES - 1) % STAGES);
+        issue(min(tile + (STAGES - 1) * SPLIT, ntiles - 1), (step + STAGES - 1) % STAGES);
         // Only tiles that touch a bound or the mask's edge pay for masking.  Element e of half t
         // is key kv0 + 32 t + 8 (e/4) + 4 g + e%4, query `col`.
         bool edge = kv0 + BKV > kv_tokens;
@@ -273,6 +292,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     wait_vmcnt<0>();   // the idle fetches of the last iterations land before the block's LDS is released
   }
 
+  if constexpr (SPLIT == 2) {
+    // The odd tiles' half hands its (max, sum, O) over through LDS, a value a lane a row (no bank
+    // conflicts); the even tiles' half folds it in by the usual rule and stores.
+    constexpr int FIELDS = 2 + 16 * DT;
+    static_assert(4 * FIELDS * 64 * 4 <= SPLIT * STAGES * STAGE, "the hand-over fits the stage buffers");
+    float* hand = reinterpret_cast<float*>(smem_all) + wave * FIELDS * 64 + lane;
+    block_barrier();   // every wave is out of the tile loop: the stage buffers are free
+    if (half == 1) {
+      hand[0] = m_run;
+      hand[64] = l_run;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) hand[(2 + 16 * t + e) * 64] = oacc[t][e];
+    }
+    __syncthreads();
+    if (half == 1) return;
+    const float m_other = hand[0], l_other = hand[64];
+    const float m_new = fmaxf(m_run, m_other);
+    const float mc = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
+    const float a_mine = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc));      // exp2(-inf) = 0: a half
+    const float a_other = __builtin_amdgcn_exp2f(fmaf(m_other, scale_log2, -mc));   // that saw no key
+    l_run = l_run * a_mine + l_other * a_other;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[t][e] = oacc[t][e] * a_mine + hand[(2 + 16 * t + e) * 64] * a_other;
+  }
+
   // Normalize and store: lane holds query `col`, columns 32 dt + 8 q + 4 g + 0..3.
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = (q_live && l_tot > 0.f) ? 1.0f / l_tot : 0.f;
@@ -288,6 +336,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
       }
   }
+}
+
+struct PrefillArgs {
+  const uint16_t *Q, *K, *V;
+  uint16_t* O;
+  int heads, group, seq, seq_len, kv_len;
+  float scale_log2;
+  int causal, window;
+  long q_row, q_head, kv_row, kv_head;
+  const int *valid, *kv_valid;
+};
+
+// The stage buffers are dynamic LDS (more than the 64 KB a kernel may declare statically).
+template <int D, int SPLIT>
+static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
+  constexpr int STAGES = D == 64 ? 3 : 2;
+  constexpr size_t lds = (size_t)SPLIT * STAGES * 2 * BKV * D * 2;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("mha_prefill: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  hipLaunchKernelGGL((mha_prefill_kernel<D, SPLIT>), dim3(blocks), dim3(256 * SPLIT), lds, (hipStream_t)stream, a.Q,
+                     a.K, a.V, a.O, a.heads, a.group, a.seq, a.seq_len, a.kv_len, a.scale_log2, a.causal, a.window,
+                     a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid);
+  return 0;
 }
 
 }  // namespace iron
@@ -315,15 +391,15 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   const long kv_row = kv_interleaved ? (long)kv_heads * d : d;
   const long kv_head = kv_interleaved ? d : (long)kv_len * d;
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid(((seq + BQ - 1) / BQ) * heads), block(256);
-  hipStream_t s = (hipStream_t)stream;
-  if (d == 64)
-    hipLaunchKernelGGL((mha_prefill_kernel<64>), grid, block, 0, s, Q, K, V, O, heads, heads / kv_heads, seq,
-                       seq_len, kv_len, scale_log2, causal, window, q_row, q_head, kv_row, kv_head,
-                       valid, kv_valid);
-  else
-    hipLaunchKernelGGL((mha_prefill_kernel<128>), grid, block, 0, s, Q, K, V, O, heads, heads / kv_heads,
-                       seq, seq_len, kv_len, scale_log2, causal, window, q_row, q_head, kv_row,
-                       kv_head, valid, kv_valid);
+  const int blocks = ((seq + BQ - 1) / BQ) * heads;
+  // Few blocks (a short sequence): the longest block's chain of tiles bounds the launch, so its
+  // tiles are split over two halves of eight waves.  Many blocks fill the chip better four waves each.
+  const bool split = blocks <= kSplitMaxBlocks;
+  PrefillArgs a{Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window,
+                q_row, q_head, kv_row, kv_head, valid, kv_valid};
+  int rc;
+  if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
+  else rc = split ? launch_prefill<128, 2>(a, blocks, stream) : launch_prefill<128, 1>(a, blocks, stream);
+  if (rc != 0) return rc;
   IRON_LAUNCH_CHECK();
 }
