@@ -306,12 +306,10 @@ struct QkvTail {
 };
 
 template <bool B_KN, bool QKV, int T>
-__global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
-                                                      const bf16_t* __restrict__ B_,
-                                                      bf16_t* __restrict__ C_, int M, int N_, int K,
-                                                      const int* __restrict__ valid, int tiles_m,
-                                                      int tiles_n, int patched, int run_above,
-                                                      int run_upto, QkvTail qkv) {
+__device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
+                                             bf16_t* __restrict__ C_, int M, int N_, int K,
+                                             const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                             int patched, int run_above, int run_upto, const QkvTail& qkv) {
   static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
   static_assert(T == 2 || (T == 1 && !B_KN && !QKV), "64x64 tiles: B (N,K), plain output");
   // T = 32x32 MFMA tiles a wave owns along each of m and n: 128x128 block tiles (T = 2), or 64x64
@@ -547,6 +545,16 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
     }
 }
 
+template <bool B_KN, bool QKV, int T>
+__global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
+                                                      const bf16_t* __restrict__ B,
+                                                      bf16_t* __restrict__ C, int M, int N, int K,
+                                                      const int* __restrict__ valid, int tiles_m,
+                                                      int tiles_n, int patched, int run_above,
+                                                      int run_upto, QkvTail qkv) {
+  gemm_nt_body<B_KN, QKV, T>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+}
+
 template <bool B_KN, bool QKV = false, int T = 2>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                           const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}, int run_above = -1,
@@ -565,6 +573,240 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV, T>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
                      valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+  IRON_LAUNCH_CHECK();
+}
+
+// The fused projections at 128 x 192 tiles: three 64-wide heads of the concatenated q | k | v head
+// list a tile, so a 2048-row chunk of a 32 + 8 + 8-head layer is 16 x 16 = 256 tiles -- one a CU in
+// one round, where 128 x 128 tiles make 384 (a round and a half, run as two).  Four waves stacked
+// along m: a wave owns 32 rows x 192 columns (6 accumulator tiles), so every head's two halves sit
+// in one wave and RoPE stays in registers.  Three stages of 40 KB; the loop is the 128 x 128
+// kernel's (direct-to-LDS loads, pinned interleave, the stage's barrier before its last k-step).
+constexpr int Q3_BM = 128, Q3_BN = 192, Q3_STAGES = 3;
+constexpr int Q3_A_BYTES = Q3_BM * BK * 2, Q3_STAGE_BYTES = (Q3_BM + Q3_BN) * BK * 2;
+
+__device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
+                                            bf16_t* __restrict__ Cq, int M, int heads, int kv_heads, int K,
+                                            const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                            int patched, int run_above, int run_upto, const QkvTail& qkv) {
+  constexpr int A_INST = Q3_BM / 8 / 4, B_INST = Q3_BN / 8 / 4, LOADS = A_INST + B_INST;   // 4 + 6 a wave
+  extern __shared__ __align__(16) char smem_q3[];
+  const int Mv = bound_or(valid, M);
+  if (Mv <= run_above || Mv > run_upto) return;
+
+  int tm, tn;
+  const int bid = blockIdx.x;
+  if (patched) {
+    const int xcd = bid & 7, loc = bid >> 3;
+    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
+    const int patches_n = tiles_n >> 2;
+    tm = (patch / patches_n) * 8 + (within & 7);
+    tn = (patch % patches_n) * 4 + (within >> 3);
+  } else {
+    constexpr int BAND = 8;
+    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
+    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
+    tm = first + in_band % height;
+    tn = in_band / height;
+  }
+  const int m0 = tm * Q3_BM;
+  if (m0 >= Mv) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane >> 3, pch = lane & 7;
+  // Head g of the concatenated list: its weight rows and where its 64 columns go.
+  auto head_weight = [&](int g) {
+    if (g < heads) return Bq + (size_t)g * 64 * K;
+    if (g < heads + kv_heads) return qkv.Bk + (size_t)(g - heads) * 64 * K;
+    return qkv.Bv + (size_t)(g - heads - kv_heads) * 64 * K;
+  };
+  const bf16_t* a_src[A_INST];
+  const bf16_t* b_src[B_INST];
+#pragma unroll
+  for (int i = 0; i < A_INST; ++i) {
+    const int r = (wave * A_INST + i) * 8 + lrow;
+    a_src[i] = A + (size_t)min(m0 + r, M - 1) * K + (pch ^ ((r >> 1) & 7)) * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < B_INST; ++i) {
+    const int r = (wave * B_INST + i) * 8 + lrow;   // row of the 192-row tile: head r / 64, its row r % 64
+    b_src[i] = head_weight(tn * 3 + r / 64) + (size_t)(r % 64) * K + (pch ^ ((r >> 1) & 7)) * 8;
+  }
+  auto issue_one = [&](char* st, int kt, int idx) {
+    const int k0 = kt * BK;
+    if (idx < A_INST)
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_src[idx] + k0),
+                                       IRON_LDS_PTR(st + (wave * A_INST + idx) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(b_src[idx - A_INST] + k0),
+                                       IRON_LDS_PTR(st + Q3_A_BYTES + (wave * B_INST + idx - A_INST) * 1024), 16, 0, 0);
+  };
+
+  f32x16 acc[6];
+#pragma unroll
+  for (int j = 0; j < 6; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int s = 0; s < Q3_STAGES - 1; ++s)
+#pragma unroll
+    for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_q3 + s * Q3_STAGE_BYTES, min(s, nk - 1), idx);
+
+  const int fr = lane & 31, kh = lane >> 5;
+  const int swz = (fr >> 1) & 7;   // tile rows are multiples of 32 apart: one swizzle for all
+  const int a_off = (wave * 32 + fr) * 128, b_off = Q3_A_BYTES + fr * 128;
+  auto frag = [&](const char* st, int off, int ks) {
+    return *reinterpret_cast<const bf16x8*>(st + off + (((ks * 2 + kh) ^ swz) << 4));
+  };
+
+  wait_vmcnt<LOADS>();   // stage 0 has landed once only stage 1's loads are out
+  block_barrier();
+  bf16x8 af[2], bfr[2][6];
+  af[0] = frag(smem_q3, a_off, 0);
+#pragma unroll
+  for (int j = 0; j < 6; ++j) bfr[0][j] = frag(smem_q3, b_off + j * 32 * 128, 0);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int kn = min(kt + Q3_STAGES - 1, nk - 1);
+    char* nst = smem_q3 + ((kt + Q3_STAGES - 1) % Q3_STAGES) * Q3_STAGE_BYTES;
+    const char* st = smem_q3 + (kt % Q3_STAGES) * Q3_STAGE_BYTES;
+    const char* st1 = smem_q3 + ((kt + 1) % Q3_STAGES) * Q3_STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      const bool last = ks == BK / 16 - 1;
+      if (last) {
+        // Of the loads in flight the oldest LOADS are stage kt+1's; the 9 issued so far for stage
+        // kt+2 may stay out.  After the barrier nobody reads stage kt any more.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_vmcnt<9>();
+        block_barrier();
+      }
+      const char* from = last ? st1 : st;
+      const int nks = last ? 0 : ks + 1;
+#pragma unroll
+      for (int j = 0; j < 6; ++j) {
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur], acc[j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j == 0) af[nxt] = frag(from, a_off, nks);
+        bfr[nxt][j] = frag(from, b_off + j * 32 * 128, nks);
+        // Ten loads a stage: three under each of the first three k-steps, the tenth under the last.
+        if (!last && j < 3) issue_one(nst, kn, ks * 3 + j);
+        if (last && j == 0) issue_one(nst, kn, 9);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  wait_vmcnt<0>();   // the idle fetches of the last iterations land before the block's LDS is released
+
+  // acc[2h][e] and acc[2h+1][e] are columns c and c + 32 of head h of the tile, c = 8 (e/4) + 4 kh + e%4,
+  // of row fr of the wave's 32: the pair RoPE turns by the angle row's (cos, sin) number c.
+  const int m = m0 + wave * 32 + fr;
+  const bf16_t* ang = qkv.angles + (size_t)min(m, M - 1) * 64 + 8 * kh;
+#pragma unroll
+  for (int h = 0; h < 3; ++h) {
+    const int g = tn * 3 + h;
+    bf16_t* C;
+    int N, col;
+    if (g < heads) { C = Cq; N = heads * 64; col = g * 64; }
+    else if (g < heads + kv_heads) { C = qkv.Ck; N = kv_heads * 64; col = (g - heads) * 64; }
+    else { C = qkv.Cv; N = kv_heads * 64; col = (g - heads - kv_heads) * 64; }
+    if (g < heads + kv_heads) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float cs[8];
+        unpack8(*reinterpret_cast<const uint4*>(ang + 16 * q), cs);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x1 = round_bf16(acc[2 * h][4 * q + e]), x2 = round_bf16(acc[2 * h + 1][4 * q + e]);
+          const float c = cs[2 * e], sn = cs[2 * e + 1];
+          acc[2 * h][4 * q + e] = x1 * c - x2 * sn;
+          acc[2 * h + 1][4 * q + e] = x2 * c + x1 * sn;
+        }
+      }
+    }
+    if (m < Mv) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          bf16_t* p = C + (size_t)m * N + col + 32 * half + 8 * q + 4 * kh;
+          const f32x16& a = acc[2 * h + half];
+          *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(a[4 * q], a[4 * q + 1]), pack_bf16(a[4 * q + 2], a[4 * q + 3]));
+        }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void qkv192_kernel(const bf16_t* __restrict__ A,
+                                                     const bf16_t* __restrict__ Bq, bf16_t* __restrict__ Cq,
+                                                     int M, int heads, int kv_heads, int K,
+                                                     const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                                     int patched, int run_above, int run_upto, QkvTail qkv) {
+  qkv192_body(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+}
+
+// Both tilings in one launch: the row bound is read on the device, and which tiling makes fewer
+// rounds over the chip depends on it, so the blocks choose -- the 192-wide tiles when the bound is
+// past `above` (if wide_top, else when it is not), the 128-wide ones otherwise.  The grid is the
+// larger of the two; a block past its tiling's tiles leaves at once.
+struct Tiling {
+  int tiles_m, tiles_n, patched;
+};
+__global__ __launch_bounds__(256) void qkv_either_kernel(const bf16_t* __restrict__ A,
+                                                         const bf16_t* __restrict__ Bq, bf16_t* __restrict__ Cq,
+                                                         int M, int heads, int kv_heads, int K,
+                                                         const int* __restrict__ valid, Tiling narrow, Tiling wide,
+                                                         int above, int wide_top, QkvTail qkv) {
+  const bool past = bound_or(valid, M) > above;
+  if (past == (wide_top != 0)) {
+    if ((int)blockIdx.x < wide.tiles_m * wide.tiles_n)
+      qkv192_body(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, -1, INT_MAX, qkv);
+  } else {
+    if ((int)blockIdx.x < narrow.tiles_m * narrow.tiles_n)
+      gemm_nt_body<false, true, 2>(A, Bq, Cq, M, heads * 64, K, valid, narrow.tiles_m, narrow.tiles_n, narrow.patched,
+                                   -1, INT_MAX, qkv);
+  }
+}
+
+static int patched_order(int tiles_m, int tiles_n) {
+  return (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
+}
+
+static int launch_qkv_either(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, int heads, int kv_heads, int K,
+                             const int* valid, hipStream_t s, QkvTail qkv, int above, bool wide_top) {
+  const int tiles_m = (M + 127) / 128;
+  const Tiling narrow{tiles_m, (heads + 2 * kv_heads) / 2, patched_order(tiles_m, (heads + 2 * kv_heads) / 2)};
+  const Tiling wide{tiles_m, (heads + 2 * kv_heads) / 3, patched_order(tiles_m, (heads + 2 * kv_heads) / 3)};
+  const size_t lds_narrow = (size_t)NT_STAGES * 256 * BK * 2, lds_wide = (size_t)Q3_STAGES * Q3_STAGE_BYTES;
+  const size_t lds = lds_narrow > lds_wide ? lds_narrow : lds_wide;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv_either_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  const int blocks = tiles_m * (narrow.tiles_n > wide.tiles_n ? narrow.tiles_n : wide.tiles_n);
+  hipLaunchKernelGGL(qkv_either_kernel, dim3(blocks), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid, narrow,
+                     wide, above, wide_top ? 1 : 0, qkv);
+  IRON_LAUNCH_CHECK();
+}
+
+static int launch_qkv192(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, int heads, int kv_heads, int K,
+                         const int* valid, hipStream_t s, QkvTail qkv, int run_above, int run_upto) {
+  const int tiles_m = (M + Q3_BM - 1) / Q3_BM, tiles_n = (heads + 2 * kv_heads) / 3;
+  const size_t lds = (size_t)Q3_STAGES * Q3_STAGE_BYTES;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv192_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  hipLaunchKernelGGL(qkv192_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid,
+                     tiles_m, tiles_n, patched_order(tiles_m, tiles_n), run_above, run_upto, qkv);
   IRON_LAUNCH_CHECK();
 }
 
@@ -868,5 +1110,25 @@ extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, cons
                  (uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)v_out) & 15) == 0,
                "prefill_qkv: operands must be 16-byte aligned");
   QkvTail tail{Wk, Wv, k_out, v_out, angles, kv_heads * d};
-  return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, (hipStream_t)stream, tail);
+  hipStream_t s = (hipStream_t)stream;
+  // 192-wide tiles (three heads) when they make fewer rounds over the chip than 128-wide ones: in
+  // units of a 128 x 128 tile's work a launch costs rounds x tile width.  The row bound is read on
+  // the device, so with one the blocks of one launch choose the tiling by it.
+  const int total = heads + 2 * kv_heads, cus = 256;
+  auto cost = [&](int live_rows, int tile_n, int n_tiles) {
+    const int tiles = ((live_rows + 127) / 128) * n_tiles;
+    return (double)((tiles + cus - 1) / cus) * tile_n;
+  };
+  auto wide_wins = [&](int live_rows) { return cost(live_rows, 192, total / 3) < cost(live_rows, 128, total / 2); };
+  if (total % 3 != 0) return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, s, tail);
+  // The bound above which the winner at `rows` wins, if the two ever change places below `rows`.
+  int above = -1;
+  if (valid != nullptr)
+    for (int live = 128; live <= rows; live += 128)
+      if (wide_wins(live) != wide_wins(rows)) above = live;
+  if (above < 0) {
+    if (wide_wins(rows)) return launch_qkv192(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, -1, INT_MAX);
+    return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, s, tail);
+  }
+  return launch_qkv_either(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, above, wide_wins(rows));
 }

@@ -155,7 +155,12 @@ def test_gemm_weight_layout_fast_paths(cuda, M, Kdim, N, rows):
     assert np.all(got[lim:] == 5.0)
 
 
-@pytest.mark.parametrize("rows,bound,H,G", [(2048, None, 32, 8), (256, 150, 16, 4), (128, None, 2, 2)])
+@pytest.mark.parametrize("rows,bound,H,G", [(2048, None, 32, 8), (256, 150, 16, 4), (128, None, 2, 2),
+                                            # bounds on either side of where the 192-wide tiles take over
+                                            (2048, 1280, 32, 8), (2048, 1281, 32, 8), (2048, 1999, 32, 8),
+                                            (2048, 2048, 32, 8), (2048, 70, 32, 8),
+                                            # heads that do not come in threes keep the 128-wide tiles
+                                            (2048, None, 32, 4), (1024, None, 8, 2), (4096, 3000, 16, 4)])
 def test_prefill_qkv_equals_three_projections_then_rope(cuda, rows, bound, H, G):
     """The fused launch against the oracle's separate steps: project and round, rotate and round."""
     rng = np.random.default_rng(91)
