@@ -857,12 +857,10 @@ constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stage
 constexpr int BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
 
 template <int WAVES, int KB>
-__global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
-                                                         const bf16_t* __restrict__ B,
-                                                         bf16_t* __restrict__ C, int M, int N, int K,
-                                                         const int* __restrict__ valid, int tiles_m,
-                                                         int tiles_n, int patched, int run_above,
-                                                         int run_upto) {
+__device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+                                                bf16_t* __restrict__ C, int M, int N, int K,
+                                                const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                                int patched, int run_above, int run_upto) {
   static_assert(KB == 64, "k per stage: 64 (32 with four stages of half-line rows measured 13 % slower)");
   constexpr int ROWB = KB * 2;               // bytes of a tile row in LDS
   constexpr int CPR = KB / 8;                // its 16-byte chunks
@@ -1027,6 +1025,72 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
   }
 }
 
+template <int WAVES, int KB>
+__global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
+                                                         const bf16_t* __restrict__ B,
+                                                         bf16_t* __restrict__ C, int M, int N, int K,
+                                                         const int* __restrict__ valid, int tiles_m,
+                                                         int tiles_n, int patched, int run_above,
+                                                         int run_upto) {
+  gemm_nt256_body<WAVES, KB>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto);
+}
+
+// A row bound read on the device decides which tile size fills the chip best (512 valid rows of
+// 2048 leave 64 of 256 large tiles), so under one the blocks of ONE launch choose: 256 x 256 tiles
+// past `few256` rows (BIG: the shape takes them), 128 x 128 past `few128`, 64 x 64 below.  Each
+// tiling's grid covers only the rows it can be chosen for; the launch's grid is the largest of
+// them and a block past its tiling's tiles leaves at once.  LDS is the largest tiling's, so a CU
+// holds one block whatever the choice.
+template <bool BIG>
+__global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restrict__ A,
+                                                          const bf16_t* __restrict__ B, bf16_t* __restrict__ C,
+                                                          int M, int N, int K, const int* __restrict__ valid,
+                                                          Tiling t256, Tiling t128, Tiling t64, int few256,
+                                                          int few128) {
+  static_assert(BIG_WAVES == 4, "the blocks of this launch are four waves");
+  const int Mv = bound_or(valid, M), bid = blockIdx.x;
+  if (BIG && Mv > few256) {
+    if (bid < t256.tiles_m * t256.tiles_n)
+      gemm_nt256_body<BIG_WAVES, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched, -1, INT_MAX);
+  } else if (Mv > few128) {
+    if (bid < t128.tiles_m * t128.tiles_n)
+      gemm_nt_body<false, false, 2>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX,
+                                    QkvTail{});
+  } else {
+    if (bid < t64.tiles_m * t64.tiles_n)
+      gemm_nt_body<false, false, 1>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX,
+                                    QkvTail{});
+  }
+}
+
+template <bool BIG>
+static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K, const int* valid,
+                              hipStream_t s, int few256, int few128) {
+  // Rows a tiling can be chosen for: the large one all of them, the others up to the next one's bound.
+  const int rows128 = BIG ? (few256 < M ? few256 : M) : M, rows64 = few128 < M ? few128 : M;
+  const int n128 = (N + 127) / 128, n64 = (N + 63) / 64;
+  const Tiling t256{BIG ? M / BIG_BM : 0, BIG ? N / BIG_BN : 0, BIG ? patched_order(M / BIG_BM, N / BIG_BN) : 0};
+  const Tiling t128{(rows128 + 127) / 128, n128, patched_order((rows128 + 127) / 128, n128)};
+  const Tiling t64{(rows64 + 63) / 64, n64, patched_order((rows64 + 63) / 64, n64)};
+  constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
+  constexpr size_t lds256 = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
+  constexpr size_t lds128 = (size_t)NT_STAGES * 256 * BK * 2;
+  constexpr size_t lds = BIG ? (lds256 > lds128 ? lds256 : lds128) : lds128;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_either_kernel<BIG>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  int blocks = t128.tiles_m * t128.tiles_n;
+  if (t256.tiles_m * t256.tiles_n > blocks) blocks = t256.tiles_m * t256.tiles_n;
+  if (t64.tiles_m * t64.tiles_n > blocks) blocks = t64.tiles_m * t64.tiles_n;
+  hipLaunchKernelGGL((gemm_either_kernel<BIG>), dim3(blocks), dim3(256), lds, s, A, B, C, M, N, K, valid, t256, t128, t64,
+                     few256, few128);
+  IRON_LAUNCH_CHECK();
+}
+
 static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                              const int* valid, hipStream_t s, int run_above = -1, int run_upto = INT_MAX) {
   const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
@@ -1065,18 +1129,20 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
     if (b_col_maj && M % BIG_BM == 0 && N % BIG_BN == 0 && (long)(M / BIG_BM) * (N / BIG_BN) >= 192 &&
         K <= (1 << 24)) {
       // Under a row bound read on the device the large tiles may cover too few rows to fill the
-      // chip (512 valid rows of 2048 leave 64 of 256 tiles).  Both kernels are launched, each
-      // running only for its range of the bound, decided where the bound is known: on the device.
-      const int tiles_n256 = N / BIG_BN;
-      const int few = tiles_n256 >= 128 ? 0 : BIG_BM * (128 / tiles_n256);   // rows up to which 128x128 tiles win
-      if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt256(A, B, C, M, N, K, valid, s);
-      const int rc = launch_gemm_nt256(A, B, C, M, N, K, valid, s, few, INT_MAX);
-      if (rc != 0) return rc;
-      return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, QkvTail{}, -1, few);
+      // chip (512 valid rows of 2048 leave 64 of 256 tiles): the blocks of one launch then choose
+      // the tile size where the bound is known, on the device.
+      const int tiles_n256 = N / BIG_BN, tiles_n128 = N / 128;
+      const int few256 = tiles_n256 >= 128 ? 0 : BIG_BM * (128 / tiles_n256);   // rows up to which 128x128 tiles win
+      const int few128 = tiles_n128 >= 128 ? 0 : 128 * (127 / tiles_n128);      // ... and 64x64 ones
+      if (valid == nullptr || few256 == 0 || few256 >= M) return launch_gemm_nt256(A, B, C, M, N, K, valid, s);
+      return launch_gemm_either<true>(A, B, C, M, N, K, valid, s, few256, few128);
     }
     if (b_col_maj) {
       // 128x128 tiles that would occupy under half the CUs give way to 64x64 ones: always, where
-      // the shape says so; under a row bound, by a second launch for the low range of the bound.
+      // the shape says so; under a row bound, by a second launch for the low range of the bound
+      // (two launches, not one whose blocks choose: on their own the 64x64 tiles' 64 KB of LDS let
+      // a CU hold two blocks, worth more than the empty launch costs -- 35 against 40 us at
+      // 512 rows of 2048 x 2048 x 8192).
       const int tiles_n128 = (N + 127) / 128;
       const long tiles128 = (long)((M + 127) / 128) * tiles_n128;
       if (tiles128 < 128) return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s);
