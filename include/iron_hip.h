@@ -48,6 +48,14 @@ int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16_t* y, int 
                          int batches, int repeat, const int* valid, int rows_per_wave,
                          int k_split, void* stream);
 
+/* C = bf16(residual_scale * bf16(A B^T) + R) for the rows under *valid (or M): a projection over many
+ * rows with its residual (a scale of 1: the plain sum; another: AXPY's) in the product's epilogue.
+ * A (M,K), B (N,K), R and C (M,N); K % 64 == 0, M, N >= 64.  C may be R.
+ * Replaces GEMM followed by ElementwiseAdd / AXPY (iron/lm/blocks.py:386-391,723-733), rounding
+ * where they round. */
+int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
+                            int N, int K, float residual_scale, const int* valid, void* stream);
+
 /* One-row fusions of a decoder layer (no single counterpart in the reference: each replaces a run
  * of its steps, iron/lm/blocks.py:627-648,697-699,723-733, and rounds where those steps round).
  *   y = E(W @ N(x)):  N = RMSNorm(x, eps) * norm_w when norm_w is not NULL (else x itself);

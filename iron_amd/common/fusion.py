@@ -15,6 +15,7 @@ and, in a prompt chunk's version (several rows, 64-wide heads),
 
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
   SiLU, ElementwiseMul (the gated feed-forward)          => iron_silu_mul_bf16
+  GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
 
 A run is fused only if every intermediate it hides is read by nothing else.
 """
@@ -198,6 +199,29 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 kw = dict(rows=M, hidden=gq.op.K, heads=gq.op.N // d, kv_heads=gk.op.N // d, d=d,
                           valid=word(gq.values.get("valid")))
                 got = Fused("prefill_qkv", i, 5, lambda a=args, kw=kw: kernels.prefill_qkv(**a, **kw))
+        elif (_name(s) == "GEMM" and i + 1 < len(steps) and _name(steps[i + 1]) in ("ElementwiseAdd", "AXPY")
+              and s.op.b_col_maj and not s.op.c_col_maj and "valid_k" not in s.values
+              and s.op.M >= 64 and s.op.N >= 64 and s.op.K % 64 == 0):
+            # a projection over many rows and its residual: the sum rides the product's epilogue
+            ad = steps[i + 1]
+            c = s.outputs["C"]
+            a, b = ad.inputs["a"], ad.inputs["b"]
+            if _name(ad) == "AXPY":   # scalar_factor * a + b: the product is the one scaled
+                other, scale = (b if _same_view(a, c) else None), float(ad.op.scalar_factor)
+            else:
+                other, scale = (a if _same_view(b, c) else (b if _same_view(a, c) else None)), 1.0
+            gv, av = s.values.get("valid"), ad.values.get("valid")
+            # the sum's bound counts elements, the product's rows
+            bounds_agree = (gv is None and av is None) or (
+                gv is not None and av is not None and gv.value == av.value and gv.linear and av.linear
+                and av.scale == gv.scale * s.op.N and av.bias == gv.bias * s.op.N)
+            flat = all(h.index is None and h.ids is None
+                       for h in (*s.inputs.values(), c, a, b, ad.outputs["y"]))
+            if (other is not None and flat and once(c) and bounds_agree and other.elements == c.elements
+                    and ad.outputs["y"].elements == c.elements and set(ad.values) <= {"valid"}):
+                args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), R=tensor(other), C=tensor(ad.outputs["y"]))
+                kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, residual_scale=scale, valid=word(gv))
+                got = Fused("gemm_add", i, 2, lambda a=args, kw=kw: kernels.gemm_residual(**a, **kw))
         elif _name(s) == "SiLU" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseMul":
             # a gated feed-forward's activation and gate over many rows: one pass instead of two
             m = steps[i + 1]

@@ -303,6 +303,10 @@ struct QkvTail {
   bf16_t* Cv;
   const bf16_t* angles;
   int kv_n;
+  // Not of the fused projections: a plain product's epilogue, C = bf16(residual_scale * bf16(A B) + residual)
+  // (one fused multiply-add; residual (M, N) like C), when residual is not NULL.
+  const bf16_t* residual;
+  float residual_scale;
 };
 
 template <bool B_KN, bool QKV, int T>
@@ -394,6 +398,25 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
     for (int j = 0; j < T; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // A residual's pieces this lane will add in the epilogue are requested now, so that their
+  // latency passes under the whole product instead of at its end (N a multiple of 4: 8-byte pieces).
+  uint2 res[T][T][4];
+  const bool res_ahead = !QKV && qkv.residual != nullptr && (N & 3) == 0;
+  if constexpr (!QKV) {
+    if (res_ahead) {
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int m = min(m0 + wm * 32 * T + i * 32 + (lane & 31), M - 1);
+            const int n = min(n0 + wn * 32 * T + j * 32 + 8 * q + (lane >> 5) * 4, N - 4);
+            res[i][j][q] = *reinterpret_cast<const uint2*>(qkv.residual + (size_t)m * N + n);
+          }
+    }
+  }
 
   const int nk = K / BK;
   // Always three stages in flight before the loop (short K repeats its last stage), so the
@@ -535,6 +558,22 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
         const int n = nb + 8 * q + hi;
         if (m >= Mv || n >= N) continue;
         bf16_t* p = C + (size_t)m * N + n;
+        if constexpr (!QKV) {
+          if (qkv.residual != nullptr) {   // the product rounded as it would be stored, then scale * it + residual
+            const bf16_t* r = qkv.residual + (size_t)m * N + n;
+            float rf[4] = {0.f, 0.f, 0.f, 0.f};
+            if (vec && n + 4 <= N) {
+              const uint2 rv = res_ahead ? res[i][j][q] : *reinterpret_cast<const uint2*>(r);
+              rf[0] = __uint_as_float(rv.x << 16); rf[1] = __uint_as_float(rv.x & 0xffff0000u);
+              rf[2] = __uint_as_float(rv.y << 16); rf[3] = __uint_as_float(rv.y & 0xffff0000u);
+            } else {
+              for (int e = 0; e < 4 && n + e < N; ++e) rf[e] = bf16_to_f32(r[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              acc[i][j][4 * q + e] = fmaf(qkv.residual_scale, round_bf16(acc[i][j][4 * q + e]), rf[e]);
+          }
+        }
         if (vec && n + 4 <= N) {
           *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
                                                     pack_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
@@ -1160,6 +1199,28 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   if (tiles128 >= 128 || (M >= 128 && N >= 128))
     return launch_gemm<128, 128, 2, 2>(A, B, C, M, N, K, b_col_maj, c_col_maj, valid, valid_k, s);
   return launch_gemm<64, 64, 2, 2>(A, B, C, M, N, K, b_col_maj, c_col_maj, valid, valid_k, s);
+}
+
+extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
+                                       int N, int K, float residual_scale, const int* valid, void* stream) {
+  IRON_REQUIRE(A && B && R && C, "gemm_residual: null operand");
+  IRON_REQUIRE(M >= 64 && N >= 64 && K > 0 && K % BK == 0,
+               "gemm_residual: M (%d) and N (%d) at least 64, K (%d) a positive multiple of %d", M, N, K, BK);
+  IRON_REQUIRE((((uintptr_t)A | (uintptr_t)B | (uintptr_t)R | (uintptr_t)C) & 15) == 0,
+               "gemm_residual: operands must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  QkvTail tail{};
+  tail.residual = R;
+  tail.residual_scale = residual_scale;
+  // The tile sizes of iron_gemm_bf16's (N,K) path below the 256-wide ones.
+  const int tiles_n128 = (N + 127) / 128;
+  const long tiles128 = (long)((M + 127) / 128) * tiles_n128;
+  if (tiles128 < 128) return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, tail);
+  const int few = tiles_n128 >= 128 ? 0 : 128 * (127 / tiles_n128);
+  if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, tail);
+  const int rc = launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, tail, few, INT_MAX);
+  if (rc != 0) return rc;
+  return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, tail, -1, few);
 }
 
 extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,

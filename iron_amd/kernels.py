@@ -69,6 +69,16 @@ def gemv(W, x, y, *, M, K, batches=1, repeat=1, valid=None, rows_per_wave=0, k_s
     )
 
 
+def gemm_residual(A, B, R, C, *, M, N, K, residual_scale=1.0, valid=None):
+    """``C = residual_scale * (A @ B.T) + R`` over many rows, B stored ``(N, K)``."""
+    _numel(_dev(A, "A"), M * K, "A")
+    _numel(_dev(B, "B"), N * K, "B")
+    _numel(_dev(R, "R"), M * N, "R")
+    _numel(_dev(C, "C"), M * N, "C")
+    check(lib().iron_gemm_residual_bf16(ptr(A), ptr(B), ptr(R), ptr(C), M, N, K, float(residual_scale),
+                                        ptr(_word(valid, "valid")), current_stream()), "iron_gemm_residual_bf16")
+
+
 def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, residual_scale=1.0, epilogue=0):
     """One-row fusion: ``[RMSNorm ->] GEMV [-> + residual | gate/up -> SiLU -> Mul]``."""
     _numel(_dev(W, "W"), M * K, "W")

@@ -183,6 +183,33 @@ def test_prefill_qkv_equals_three_projections_then_rope(cuda, rows, bound, H, G)
         assert np.all(got[lim:] == 7.0)
 
 
+@pytest.mark.parametrize("M,Kdim,N,rows,scale", [(2048, 512, 2048, None, 1.0), (2048, 256, 2048, 512, 1.0),
+                                                 (2048, 256, 2048, 1500, 0.22), (256, 128, 512, 100, 1.0),
+                                                 (128, 64, 64, None, -0.5), (4096, 192, 1024, 3000, 1.0)])
+def test_gemm_residual_epilogue(cuda, M, Kdim, N, rows, scale):
+    """A projection over many rows with its residual in the epilogue: the product rounded as the
+    separate step would store it, then one fused multiply-add with the residual (the sum, or AXPY)."""
+    rng = np.random.default_rng(M + N)
+    A, B, R = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.05), bf(rng, M, N)
+    lim = M if rows is None else rows
+    want = ops.axpy(scale, ops.gemm(A, B, b_col_maj=True), R)
+    if scale == 1.0:
+        assert np.array_equal(want, ops.add(ops.gemm(A, B, b_col_maj=True), R))
+    if rows is not None:
+        A[rows:] = np.nan
+    C = out_like((M, N), cuda, fill=7.0)
+    K.gemm_residual(dev(A, cuda), dev(B, cuda), dev(R, cuda), C, M=M, N=N, K=Kdim, residual_scale=scale,
+                    valid=None if rows is None else word(rows, cuda))
+    got = from_torch(C)
+    close(got[:lim], want[:lim], rtol=1e-2, atol=1e-2)
+    assert np.all(got[lim:] == 7.0)
+    # in place: the residual stream is its own output
+    Rd = dev(R, cuda)
+    K.gemm_residual(dev(np.nan_to_num(A), cuda), dev(B, cuda), Rd, Rd, M=M, N=N, K=Kdim, residual_scale=scale,
+                    valid=None if rows is None else word(rows, cuda))
+    close(from_torch(Rd)[:lim], want[:lim], rtol=1e-2, atol=1e-2)
+
+
 @pytest.mark.parametrize("b_col_maj", [False, True])
 def test_gemm_bounded_rows_and_k_do_not_read_the_poison(cuda, b_col_maj):
     """NaN past the bounds must not reach the output (test_gemm_bounded_k.py)."""
