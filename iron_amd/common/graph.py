@@ -124,12 +124,14 @@ class Affine:
     __rmul__ = __mul__
 
     def __floordiv__(self, c):
-        if not isinstance(c, (int, np.integer)) or c <= 0 or c & (c - 1):
-            raise TypeError(f"{self.name} // {c}: only a power of two divides a per-call value")
+        if not isinstance(c, (int, np.integer)) or c <= 0:
+            raise TypeError(f"{self.name} // {c}: a per-call value is divided by a positive integer")
         if self.clamped:
             raise TypeError(f"{self.name}: // after a clamp is not a per-call expression")
-        if self.linear and self.scale % c == 0 and self.bias % c == 0:  # the floor folds
+        if self.linear and self.scale % c == 0 and self.bias % c == 0:  # the floor folds (12 heads' rows // 12)
             return dataclasses.replace(self, scale=self.scale // int(c), bias=self.bias // int(c))
+        if c & (c - 1):
+            raise TypeError(f"{self.name} // {c}: only a power of two divides a per-call value it does not divide evenly")
         return dataclasses.replace(self, down=self.down + int(c).bit_length() - 1)
 
     def clamp(self, lo=None, hi=None):

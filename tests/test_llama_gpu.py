@@ -11,8 +11,9 @@ import numpy as np
 import pytest
 
 import oracle
-from iron_amd.applications.llama import LLAMA_3_2_1B, Llama
+from iron_amd.applications.llama import LLAMA_3_2_1B, Llama, shapes
 from iron_amd.lm.causal import OnHost
+from oracle import ops
 from tests.llama_support import BIASED, BIASED_GOLDEN, SCALED, Golden, assert_close, kl, weights
 
 pytestmark = pytest.mark.gpu
@@ -133,6 +134,46 @@ def test_refusals_before_any_dispatch(toy):
         toy(token=3, position=0, nonsense=1)
     with pytest.raises(ValueError, match="takes"):
         toy(np.zeros(7, np.int32), token=0, position=0)
+
+
+@pytest.mark.parametrize("shape", [
+    # 128-wide heads (Llama 3 8B's proportions): the prompt chunk's projections stay separate steps
+    dict(hidden_size=1024, num_attention_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=2816),
+    # heads that do not come in threes or pairs of tiles, an odd multiple of 64 in the feed-forward, untied head
+    dict(hidden_size=768, num_attention_heads=12, num_key_value_heads=4, head_dim=64, intermediate_size=1984,
+         tie_word_embeddings=False),
+    # one KV head (multi-query), a sliding window shorter than the prompt
+    dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=1, head_dim=64, intermediate_size=1024,
+         sliding_window=48),
+], ids=["d128", "twelve_heads_untied", "multi_query_window"])
+def test_other_decoder_shapes_match_the_host_reference(cuda, shape):
+    """Shapes off the benchmark's: every fused path either takes the shape or leaves the steps as
+    recorded; either way the GPU's logits are the host reference's, prompt (in two chunks) and decode."""
+    config = dataclasses.replace(SCALED, vocab_size=1000, num_hidden_layers=2, max_seq_len=256, prefill_chunk=64,
+                                 rope_scaling=None, **shape)
+    names = dict(shapes(config))
+    if not config.tie_word_embeddings:
+        names["lm_head.weight"] = (config.vocab_size, config.hidden_size)
+    w = ops.filled(names, seed=3)
+    gpu, cpu = Llama(config, w), HostLlama(config, w)
+    gpu.load_versions()
+    cpu.load_versions()
+    try:
+        tokens = np.random.default_rng(5).integers(0, config.vocab_size, 90)
+        want, got = cpu.logits(tokens), gpu.logits(tokens)
+        assert_close(got, want)
+        for step in range(3):
+            tokens = np.append(tokens, want.argmax())
+            want, got = cpu.logits(tokens), gpu.logits(tokens)
+            assert_close(got, want, f"decode step {step}")
+        # The device-carried run draws what host-started steps draw; its first token is the host
+        # reference's best within the logits' tolerance (drawn weights leave near-ties).
+        drawn = gpu.generate(tokens[:20], 8)
+        assert drawn == list(gpu.session.draw(tokens[:20], 8, each=True))
+        first = cpu.logits(tokens[:20])
+        assert first[drawn[0]] >= first.max() - 0.05 * np.abs(first).max()
+    finally:
+        gpu.release()
 
 
 def test_two_layers_at_llama_1b_width_match_the_host_reference(cuda):
