@@ -223,8 +223,10 @@ int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_
                      int record_len, const int* at, int* token_copy, void* stream);
 
 /* Evaluate n per-call word expressions in order, on the device, in one thread:
- *   words[e.dst] = clamp(((words[e.src] * e.mul + e.add) >> e.shift), e.lo, e.hi)
- * exprs is n records of 7 int32 {dst, src, mul, add, shift, lo, hi} in device memory.
+ *   words[e.dst] = (clamp(((words[e.src] * e.mul + e.add) >> e.shift), e.lo, e.hi) & e.mask) + e.post
+ * exprs is n records of 9 int32 {dst, src, mul, add, shift, lo, hi, mask, post} in device memory
+ * (mask -1 keeps every bit; 2^k - 1 is the remainder a ring of 2^k rows indexes by, post the
+ * rows its mirror lies further on).
  * The device-side carry/Emit of a decode loop (position += 1, kv_valid = position + 1):
  * iron/common/graph/carried.py:189-276, iron/operators/emit.py. */
 int iron_eval_words(int* words, int n_words, const int* exprs, int n, void* stream);

@@ -51,7 +51,7 @@ class Carried(Generic[T]):
 
 @dataclasses.dataclass(frozen=True)
 class Affine:
-    """``clamp(((value * scale + bias) >> down), lo, hi)`` of one per-call value."""
+    """``(clamp(((value * scale + bias) >> down), lo, hi) & mask) + post`` of one per-call value."""
 
     value: str
     scale: int = 1
@@ -59,10 +59,18 @@ class Affine:
     down: int = 0
     lo: int | None = None
     hi: int | None = None
+    mask: int = -1  # 2^k - 1: the remainder by 2^k, a ring's row
+    post: int = 0   # added after the floor, clamp or remainder
 
     @property
     def linear(self) -> bool:
-        return self.down == 0 and self.lo is None and self.hi is None
+        return self.down == 0 and self.lo is None and self.hi is None and self.mask == -1 and self.post == 0
+
+    def record(self) -> list[int]:
+        """``{mul, add, shift, lo, hi, mask, post}`` of the device's expression table."""
+        big = 2**31 - 1
+        return [self.scale, self.bias, self.down, -big - 1 if self.lo is None else self.lo,
+                big if self.hi is None else self.hi, self.mask, self.post]
 
     @property
     def clamped(self) -> bool:
@@ -79,6 +87,10 @@ class Affine:
             n += f"_d{self.down}"
         if self.clamped:
             n += f"_c{'' if self.lo is None else self.lo}_{'' if self.hi is None else self.hi}"
+        if self.mask != -1:
+            n += f"_r{self.mask + 1}"
+        if self.post:
+            n += f"_{'p' if self.post > 0 else 'm'}{abs(self.post)}"
         return n
 
     def evaluate(self, values: Mapping[str, int]) -> int:
@@ -87,7 +99,15 @@ class Affine:
             v = max(v, self.lo)
         if self.hi is not None:
             v = min(v, self.hi)
-        return v
+        return (v & self.mask) + self.post
+
+    def __mod__(self, c):
+        """The remainder by a power of two of a value that is never negative (a ring's row)."""
+        if not isinstance(c, (int, np.integer)) or c <= 0 or c & (c - 1):
+            raise TypeError(f"{self.name} % {c}: a per-call value's remainder is by a power of two")
+        if self.post:
+            raise TypeError(f"{self.name} % {c}: a remainder after a later sum is not a per-call expression")
+        return dataclasses.replace(self, mask=self.mask & (int(c) - 1))
 
     def _need_linear(self, what):
         if not self.linear:
@@ -100,13 +120,16 @@ class Affine:
             return dataclasses.replace(self, scale=self.scale + c.scale, bias=self.bias + c.bias)
         if not isinstance(c, (int, np.integer)):
             return NotImplemented
-        self._need_linear("+")
+        if not self.linear:  # past a floor, clamp or remainder a number is added last
+            return dataclasses.replace(self, post=self.post + int(c))
         return dataclasses.replace(self, bias=self.bias + int(c))
 
     __radd__ = __add__
 
     def __sub__(self, c):
         if isinstance(c, Affine):
+            if not self.linear and dataclasses.replace(c, post=0) == dataclasses.replace(self, post=0):
+                return Affine(self.value, scale=0, bias=self.post - c.post)  # a fixed distance
             return self + (c * -1)
         return self + (-int(c))
 
@@ -126,8 +149,8 @@ class Affine:
     def __floordiv__(self, c):
         if not isinstance(c, (int, np.integer)) or c <= 0:
             raise TypeError(f"{self.name} // {c}: a per-call value is divided by a positive integer")
-        if self.clamped:
-            raise TypeError(f"{self.name}: // after a clamp is not a per-call expression")
+        if self.clamped or self.mask != -1 or self.post:
+            raise TypeError(f"{self.name}: // after a clamp or a remainder is not a per-call expression")
         if self.linear and self.scale % c == 0 and self.bias % c == 0:  # the floor folds (12 heads' rows // 12)
             return dataclasses.replace(self, scale=self.scale // int(c), bias=self.bias // int(c))
         if c & (c - 1):
@@ -135,6 +158,8 @@ class Affine:
         return dataclasses.replace(self, down=self.down + int(c).bit_length() - 1)
 
     def clamp(self, lo=None, hi=None):
+        if self.mask != -1 or self.post:
+            raise TypeError(f"{self.name}: a clamp after a remainder is not a per-call expression")
         return dataclasses.replace(
             self,
             lo=lo if self.lo is None else (self.lo if lo is None else max(lo, self.lo)),
@@ -145,9 +170,9 @@ class Affine:
         raise TypeError(f"{self.name} is known per call, not while recording")
 
     def _refuse(self, *_):
-        raise TypeError(f"{self.name}: only + - * // 2^k and clamp build per-call expressions")
+        raise TypeError(f"{self.name}: only + - * // 2^k, % 2^k and clamp build per-call expressions")
 
-    __mod__ = __lt__ = __le__ = __gt__ = __ge__ = __truediv__ = _refuse
+    __lt__ = __le__ = __gt__ = __ge__ = __truediv__ = _refuse
 
 
 def clamp(x, lo=None, hi=None):
@@ -374,8 +399,6 @@ class Handle:
         if isinstance(key, Affine):
             if self.index is not None or self.ids is not None:
                 raise TypeError("a per-call view is indexed once")
-            if not (key.linear or key.clamped or key.down):
-                raise TypeError("index: not a per-call expression")
             return dataclasses.replace(self, shape=self.shape[1:], index=key, index_stride=row,
                                        index_rows=self.shape[0], valid={})
         if isinstance(key, (int, np.integer)):
@@ -425,6 +448,9 @@ class Handle:
         from ..operators.elementwise_add import ElementwiseAdd, RowwiseAdd
         from ..operators.elementwise_mul import ElementwiseMul, RowwiseMul
 
+        if isinstance(other, (int, float, np.integer, np.floating)) and not isinstance(other, bool):
+            # A number is a constant row in bf16 (iron/common/graph/handle.py:652-661).
+            other = _constant_row(float(other), self.shape[-1] if self.shape else 1)
         if isinstance(other, Resident):
             other = other._handle()
         if not isinstance(other, Handle):
@@ -446,6 +472,25 @@ class Handle:
 
     def __mul__(self, other):
         return self._binary(other, "*")
+
+    __radd__ = __add__
+    __rmul__ = __mul__
+
+    def __truediv__(self, other):
+        if not isinstance(other, (int, float, np.integer, np.floating)) or isinstance(other, bool):
+            raise TypeError(f"{self!r} is divided by a number, not {other!r}")
+        return self * (1 / other)
+
+
+_CONSTANT_ROWS: dict[tuple[float, int], "Weight"] = {}
+
+
+def _constant_row(value: float, cols: int) -> "Weight":
+    """One row of ``cols`` copies of ``value`` in bf16, the same tensor wherever it is asked for."""
+    key = (value, cols)
+    if key not in _CONSTANT_ROWS:
+        _CONSTANT_ROWS[key] = weight(np.full(cols, value, dtype=np.float32))
+    return _CONSTANT_ROWS[key]
 
 
 # ------------------------------------------------------------------ recorder
@@ -1034,6 +1079,7 @@ def _host_tensor(array, dtype):
 # ------------------------------------------------------------ compiled graph
 
 WORD_SLOTS = 64  # int32 words of the per-call scratchpad
+EXPR_WORDS = 9  # int32 words of one record of the device's expression table
 
 
 class DeviceOutput:
@@ -1092,7 +1138,7 @@ class CompiledGraph:
             raise ValueError(f"{graph.name}: more than {WORD_SLOTS} per-call words")
         # The words and the expression table outlive a call (a replay starts from the last
         # one's values; the table is written once), so they are residents of this version.
-        self._words_resident = State((WORD_SLOTS * 8,), np.int32)
+        self._words_resident = State((WORD_SLOTS * (1 + EXPR_WORDS),), np.int32)
         arena.place_resident(self._words_resident)
         arena.reserve_transients(pool.size)
         self._loaded_generation = None
@@ -1134,7 +1180,7 @@ class CompiledGraph:
             return self
         base = self.arena.resident_offsets[id(self._words_resident)]
         self.words = self.arena.view(base, (WORD_SLOTS,), np.int32)
-        self.expr_table = self.arena.view(base + WORD_SLOTS * 4, (WORD_SLOTS * 7,), np.int32)
+        self.expr_table = self.arena.view(base + WORD_SLOTS * 4, (WORD_SLOTS * EXPR_WORDS,), np.int32)
         self.host_words = torch.zeros(WORD_SLOTS, dtype=torch.int32).pin_memory()
         # Device-side expression table: derived words, then the carried values.
         rows = []
@@ -1143,19 +1189,17 @@ class CompiledGraph:
             src = self.slots.get(expr.value)
             if expr.value == "__const__":
                 src, expr = 0, dataclasses.replace(expr, scale=0)
-            rows.append([slot, src, expr.scale, expr.bias, expr.down,
-                         -big - 1 if expr.lo is None else expr.lo, big if expr.hi is None else expr.hi])
+            rows.append([slot, src, *expr.record()])
         self.n_derived = len(rows)
         carried = self.recording.carry or {}
         self.carry_copies = []  # (value slot, handle) for values carried from a device buffer
         for k, v in carried.items():
             if isinstance(v, Affine):
-                rows.append([self.slots[k], self.slots[v.value], v.scale, v.bias, v.down,
-                             -big - 1 if v.lo is None else v.lo, big if v.hi is None else v.hi])
+                rows.append([self.slots[k], self.slots[v.value], *v.record()])
             elif isinstance(v, Handle):
                 self.carry_copies.append((self.slots[k], v))
             else:
-                rows.append([self.slots[k], 0, 0, int(v), 0, -big - 1, big])
+                rows.append([self.slots[k], 0, 0, int(v), 0, -big - 1, big, -1, 0])
         self.n_exprs = len(rows)
         # A replay ends by carrying its values and re-deriving the words the next replay reads, in
         # one launch: the carried rows are followed by a second copy of the derived ones.
@@ -1238,9 +1282,9 @@ class CompiledGraph:
             kernels.copy_rows(self._tensor(h).view(-1)[:1], self.words[slot : slot + 1], rows=1, row_elems=1,
                               src_rows=1, dst_rows=1)
         if self.n_tail:
-            kernels.eval_words(self.words, self.expr_table[7 * self.n_derived :], self.n_tail)
+            kernels.eval_words(self.words, self.expr_table[EXPR_WORDS * self.n_derived :], self.n_tail)
         elif self.n_exprs > self.n_derived:
-            kernels.eval_words(self.words, self.expr_table[7 * self.n_derived :], self.n_exprs - self.n_derived)
+            kernels.eval_words(self.words, self.expr_table[EXPR_WORDS * self.n_derived :], self.n_exprs - self.n_derived)
             self._derive()
 
     def _capture(self) -> None:

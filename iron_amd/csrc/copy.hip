@@ -107,12 +107,12 @@ __global__ void eval_words_kernel(int* __restrict__ words, int n_words,
                                   const int* __restrict__ exprs, int n) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   for (int e = 0; e < n; ++e) {
-    const int* x = exprs + 7 * e;
+    const int* x = exprs + 9 * e;
     const int dst = x[0], src = x[1];
     if (dst < 0 || dst >= n_words || src < 0 || src >= n_words) continue;
     long v = ((long)words[src] * x[2] + x[3]) >> x[4];
     v = v < x[5] ? x[5] : (v > x[6] ? x[6] : v);
-    words[dst] = (int)v;
+    words[dst] = ((int)v & x[7]) + x[8];
   }
 }
 

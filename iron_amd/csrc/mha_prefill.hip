@@ -36,7 +36,7 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 // are merged through LDS at the end.  A query block's chain of tiles is half as long, which is what
 // bounds a short sequence: its blocks are few and the one that sees every key finishes last.
 template <int D, int SPLIT>
-__global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(2))) void mha_prefill_kernel(
+__global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -378,7 +378,7 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   IRON_REQUIRE(Q && K && V && O, "mha_prefill: null operand");
   IRON_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "mha_prefill: heads (%d) must be a positive multiple of kv_heads (%d)", heads, kv_heads);
-  IRON_REQUIRE(d == 64 || d == 128, "mha_prefill: d (%d) must be 64 or 128", d);
+  IRON_REQUIRE(d == 64 || d == 128 || d == 256, "mha_prefill: d (%d) must be 64, 128 or 256", d);
   IRON_REQUIRE(seq > 0 && seq_len > 0 && seq_len <= seq,
                "mha_prefill: seq_len (%d) must be in [1, seq (%d)]", seq_len, seq);
   IRON_REQUIRE(kv_len >= seq, "mha_prefill: kv_len (%d) must be at least seq (%d): the queries are its last rows",
@@ -399,7 +399,8 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
                 q_row, q_head, kv_row, kv_head, valid, kv_valid};
   int rc;
   if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
-  else rc = split ? launch_prefill<128, 2>(a, blocks, stream) : launch_prefill<128, 1>(a, blocks, stream);
+  else if (d == 128) rc = split ? launch_prefill<128, 2>(a, blocks, stream) : launch_prefill<128, 1>(a, blocks, stream);
+  else rc = launch_prefill<256, 1>(a, blocks, stream);
   if (rc != 0) return rc;
   IRON_LAUNCH_CHECK();
 }

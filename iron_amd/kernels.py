@@ -376,7 +376,7 @@ def sample(logits, draws, token, *, n=None, row=None, k_max=64, workspace=None, 
 def eval_words(words, exprs, n=None):
     _dev(words, "words", torch.int32)
     _dev(exprs, "exprs", torch.int32)
-    n = exprs.numel() // 7 if n is None else n
+    n = exprs.numel() // 9 if n is None else n  # nine words a record
     check(lib().iron_eval_words(ptr(words), words.numel(), ptr(exprs), n, current_stream()), "iron_eval_words")
 
 

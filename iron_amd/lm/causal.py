@@ -162,8 +162,13 @@ class CausalLM(iron.Graph):
 
     @property
     def recurrent(self) -> list:
-        """States that restart only at some positions (ring caches): none in this build."""
-        return []
+        """The states that restart only at some positions: the layers' ring caches."""
+        rings = {id(l.cache): l.cache for l in self.layers if getattr(l.cache, "ring", None) is not None}
+        return list(rings.values())
+
+    def layer(self, call, i: int, w, x):
+        """Layer ``i``, ``w``, on ``x``: a model whose layers take more than the call says what."""
+        return w(x, call)
 
     def head(self, x):
         """The final norm, then the output head (the embedding, if tied)."""
@@ -189,8 +194,8 @@ class CausalLM(iron.Graph):
         for rope in (layer.rope for layer in self.layers):
             if rope is not None and id(rope) not in call.ropes:
                 call.ropes[id(rope)] = rope.rows(call)
-        for layer in self.layers:
-            x = layer(x, call)
+        for i, layer in enumerate(self.layers):
+            x = self.layer(call, i, layer, x)
         if call.prompt:
             x = Copy.step(x[call.rows - 1]).reshape(1, c.hidden_size)  # the last row's logits alone
         return self.draw(self.head(x), call)

@@ -96,8 +96,6 @@ class MHA(Operator):
     def validate(self) -> None:
         if self.d not in (64, 128, 256):
             raise ValueError(f"MHA: d ({self.d}) must be 64, 128 or 256")
-        if self.seq_len != 1 and self.d == 256:
-            raise ValueError("MHA: many queries take d of 64 or 128")
         if self.window is not None and self.window <= 0:
             raise ValueError(f"MHA: window ({self.window}) must be positive or None")
         if not 0 <= self.scale < np.inf:

@@ -400,6 +400,24 @@ def test_mha_prefill_d128_and_ragged_seq(cuda):
     close(got, want)
 
 
+def test_mha_prefill_d256_ragged_windowed_and_bounded(cuda):
+    """256-wide heads (a global layer's of a toy Gemma 4): a ragged causal sequence, a window, and a
+    prompt chunk bounded by device words at the end of a longer cache, unscaled as Gemma attends."""
+    rng = np.random.default_rng(21)
+    H, G, d, S = 4, 1, 256, 200
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    for window in (None, 37):
+        got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=S, window=window)
+        close(got, want)
+    C, L, rows, kv = 64, 512, 40, 300
+    Q, Kc, Vc = bf(rng, C, H, d) * 0.25, bf(rng, L, G, d) * 0.25, bf(rng, L, G, d)
+    Q[rows:], Kc[kv:], Vc[kv:] = np.nan, np.nan, np.nan
+    got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=C, seq_len=C, kv_len=L, valid=rows, kv_valid=kv,
+                            scale=1.0)
+    assert np.all(got[rows:] == 0)
+    close(got[:rows], want[:rows])
+
+
 @pytest.mark.parametrize("L", [1024, 4096, 16384])
 def test_mha_decode_llama_shape(cuda, L):
     rng = np.random.default_rng(15)
@@ -663,8 +681,11 @@ def test_sample_special_values_and_row_bounds(cuda):
 
 def test_eval_words_advances_a_decode_step(cuda):
     words = torch.tensor([11, 40, 0, 0, 0, 0, 0, 0], dtype=torch.int32, device=cuda)
-    # position += 1; kv_valid = position + 1; rope_row = min(position, 5); half = position >> 1
-    exprs = torch.tensor([[1, 1, 1, 1, 0, -(2**31), 2**31 - 1], [2, 1, 1, 1, 0, -(2**31), 2**31 - 1],
-                          [3, 1, 1, 0, 0, 0, 5], [4, 1, 1, 0, 1, -(2**31), 2**31 - 1]], dtype=torch.int32, device=cuda)
+    # position += 1; kv_valid = position + 1; rope_row = min(position, 5); half = position >> 1;
+    # ring_row = max(position - 3, 0) % 16; its mirror's = ring_row + 16
+    exprs = torch.tensor([[1, 1, 1, 1, 0, -(2**31), 2**31 - 1, -1, 0], [2, 1, 1, 1, 0, -(2**31), 2**31 - 1, -1, 0],
+                          [3, 1, 1, 0, 0, 0, 5, -1, 0], [4, 1, 1, 0, 1, -(2**31), 2**31 - 1, -1, 0],
+                          [5, 1, 1, -3, 0, 0, 2**31 - 1, 15, 0], [6, 1, 1, -3, 0, 0, 2**31 - 1, 15, 16]],
+                         dtype=torch.int32, device=cuda)
     K.eval_words(words, exprs)
-    assert words.cpu().tolist() == [11, 41, 42, 5, 20, 0, 0, 0]
+    assert words.cpu().tolist() == [11, 41, 42, 5, 20, 6, 22, 0]
