@@ -88,6 +88,15 @@ int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t*
                           const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
                           uint16_t* k_out, uint16_t* v_out, int rows, int hidden, int heads,
                           int kv_heads, int d, const int* valid, void* stream);
+/* The same with k and v written straight into the chunk's rows of the layer's KV caches, rows
+ * *start on of keys and values (cache_rows, kv_heads*d): replaces the two Copy steps that follow as
+ * well (iron/lm/blocks.py:472-486).  The first row is held where the rows under the bound end inside
+ * the cache; without a bound rows <= cache_rows. */
+int iron_prefill_qkv_cache_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
+                                const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
+                                uint16_t* keys, uint16_t* values, int rows, int hidden, int heads,
+                                int kv_heads, int d, int cache_rows, const int* start,
+                                const int* valid, void* stream);
 
 /* y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) per row; w NULL = unweighted (one rounding).
  * x,y (rows, cols); w (cols).  cols % 8 == 0.  valid: rows computed.

@@ -199,6 +199,28 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 kw = dict(rows=M, hidden=gq.op.K, heads=gq.op.N // d, kv_heads=gk.op.N // d, d=d,
                           valid=word(gq.values.get("valid")))
                 got = Fused("prefill_qkv", i, 5, lambda a=args, kw=kw: kernels.prefill_qkv(**a, **kw))
+                # ... and the two copies of k and v into the chunk's rows of the layer's caches
+                ck, cv = (steps[i + 5], steps[i + 6]) if i + 6 < len(steps) else (None, None)
+                if ck is not None and _name(ck) == "Copy" and _name(cv) == "Copy":
+                    kd, vd = ck.outputs["dst"], cv.outputs["dst"]
+                    gvalid = gq.values.get("valid")
+                    cached = (
+                        _same_view(ck.inputs["src"], rk.outputs["y"]) and _same_view(cv.inputs["src"], v)
+                        and once(rk.outputs["y"]) and once(v)
+                        and all(h.index is not None and h.ids is None and h.offset == 0
+                                and h.index_stride == gk.op.N and h.elements == M * gk.op.N for h in (kd, vd))
+                        and kd.index == vd.index and kd.index_rows == vd.index_rows
+                        and kd.valid.get(0) == gvalid and vd.valid.get(0) == gvalid
+                        and ck.inputs["src"].valid.get(0) == gvalid and cv.inputs["src"].valid.get(0) == gvalid
+                        and (gvalid is not None or M <= kd.index_rows)
+                    )
+                    if cached:
+                        args = {k_: t for k_, t in args.items() if k_ not in ("k_out", "v_out")}
+                        args |= dict(keys=tensor(kd)[: kd.index_rows * kd.index_stride],
+                                     values=tensor(vd)[: vd.index_rows * vd.index_stride])
+                        kw = dict(kw, cache_rows=kd.index_rows, start=word(kd.index))
+                        got = Fused("prefill_qkv_cache", i, 7,
+                                    lambda a=args, kw=kw: kernels.prefill_qkv_cache(**a, **kw))
         elif (_name(s) == "GEMM" and i + 1 < len(steps) and _name(steps[i + 1]) in ("ElementwiseAdd", "AXPY")
               and s.op.b_col_maj and not s.op.c_col_maj and "valid_k" not in s.values
               and s.op.M >= 64 and s.op.N >= 64 and s.op.K % 64 == 0):

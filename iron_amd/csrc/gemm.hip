@@ -307,7 +307,21 @@ struct QkvTail {
   // (one fused multiply-add; residual (M, N) like C), when residual is not NULL.
   const bf16_t* residual;
   float residual_scale;
+  // Of the fused projections again: Ck and Cv are KV caches of kv_rows rows (a row kv_n wide, as the
+  // projections write one), and the chunk's rows go to rows *kv_row0 on, when kv_row0 is not NULL.
+  const int* kv_row0;
+  int kv_rows;
 };
+
+// The k and v outputs moved to the chunk's rows of their caches.  The first row is held where the
+// rows under the bound still end inside the cache, whatever the word holds.
+__device__ __forceinline__ void to_cache_rows(QkvTail& t, const int* __restrict__ valid, int M) {
+  if (t.kv_row0 == nullptr) return;
+  const int rows = bound_or(valid, M);
+  const int first = max(0, min(*t.kv_row0, t.kv_rows - rows));
+  t.Ck += (size_t)first * t.kv_n;
+  t.Cv += (size_t)first * t.kv_n;
+}
 
 template <bool B_KN, bool QKV, int T>
 __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
@@ -591,6 +605,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       const int* __restrict__ valid, int tiles_m,
                                                       int tiles_n, int patched, int run_above,
                                                       int run_upto, QkvTail qkv) {
+  if constexpr (QKV) to_cache_rows(qkv, valid, M);
   gemm_nt_body<B_KN, QKV, T>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
 }
 
@@ -783,6 +798,7 @@ __global__ __launch_bounds__(256) void qkv192_kernel(const bf16_t* __restrict__ 
                                                      int M, int heads, int kv_heads, int K,
                                                      const int* __restrict__ valid, int tiles_m, int tiles_n,
                                                      int patched, int run_above, int run_upto, QkvTail qkv) {
+  to_cache_rows(qkv, valid, M);
   qkv192_body(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
 }
 
@@ -799,6 +815,7 @@ __global__ __launch_bounds__(256) void qkv_either_kernel(const bf16_t* __restric
                                                          const int* __restrict__ valid, Tiling narrow, Tiling wide,
                                                          int above, int wide_top, QkvTail qkv) {
   const bool past = bound_or(valid, M) > above;
+  to_cache_rows(qkv, valid, M);
   if (past == (wide_top != 0)) {
     if ((int)blockIdx.x < wide.tiles_m * wide.tiles_n)
       qkv192_body(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, -1, INT_MAX, qkv);
@@ -1223,10 +1240,10 @@ extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, con
   return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, tail, -1, few);
 }
 
-extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
-                                     const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
-                                     uint16_t* k_out, uint16_t* v_out, int rows, int hidden, int heads,
-                                     int kv_heads, int d, const int* valid, void* stream) {
+static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,
+                       const uint16_t* angles, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out, int rows,
+                       int hidden, int heads, int kv_heads, int d, const int* valid, const int* kv_row0,
+                       int kv_rows, void* stream) {
   IRON_REQUIRE(x && Wq && Wk && Wv && angles && q_out && k_out && v_out, "prefill_qkv: null operand");
   IRON_REQUIRE(d == 64, "prefill_qkv: d (%d) must be 64 (a wave's 64 output columns are one head)", d);
   IRON_REQUIRE(rows >= 64 && heads > 0 && kv_heads > 0 && heads % 2 == 0 && kv_heads % 2 == 0,
@@ -1237,6 +1254,8 @@ extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, cons
                  (uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)v_out) & 15) == 0,
                "prefill_qkv: operands must be 16-byte aligned");
   QkvTail tail{Wk, Wv, k_out, v_out, angles, kv_heads * d};
+  tail.kv_row0 = kv_row0;
+  tail.kv_rows = kv_rows;
   hipStream_t s = (hipStream_t)stream;
   // 192-wide tiles (three heads) when they make fewer rounds over the chip than 128-wide ones: in
   // units of a 128 x 128 tile's work a launch costs rounds x tile width.  The row bound is read on
@@ -1258,4 +1277,25 @@ extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, cons
     return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, s, tail);
   }
   return launch_qkv_either(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, above, wide_wins(rows));
+}
+
+extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
+                                     const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
+                                     uint16_t* k_out, uint16_t* v_out, int rows, int hidden, int heads,
+                                     int kv_heads, int d, const int* valid, void* stream) {
+  return prefill_qkv(x, Wq, Wk, Wv, angles, q_out, k_out, v_out, rows, hidden, heads, kv_heads, d, valid, nullptr, 0,
+                     stream);
+}
+
+extern "C" int iron_prefill_qkv_cache_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
+                                           const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
+                                           uint16_t* keys, uint16_t* values, int rows, int hidden, int heads,
+                                           int kv_heads, int d, int cache_rows, const int* start,
+                                           const int* valid, void* stream) {
+  IRON_REQUIRE(start != nullptr, "prefill_qkv_cache: null start");
+  IRON_REQUIRE(cache_rows > 0, "prefill_qkv_cache: cache_rows (%d) must be positive", cache_rows);
+  IRON_REQUIRE(valid != nullptr || rows <= cache_rows,
+               "prefill_qkv_cache: without a bound the chunk's %d rows must fit the cache's %d", rows, cache_rows);
+  return prefill_qkv(x, Wq, Wk, Wv, angles, q_out, keys, values, rows, hidden, heads, kv_heads, d, valid, start,
+                     cache_rows, stream);
 }

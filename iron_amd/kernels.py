@@ -135,6 +135,25 @@ def prefill_qkv(x, Wq, Wk, Wv, angles, q_out, k_out, v_out, *, rows, hidden, hea
     )
 
 
+def prefill_qkv_cache(x, Wq, Wk, Wv, angles, q_out, keys, values, *, rows, hidden, heads, kv_heads, d, cache_rows,
+                      start, valid=None):
+    """``prefill_qkv`` with k and v written into rows ``start`` on of the layer's KV caches."""
+    _numel(_dev(x, "x"), rows * hidden, "x")
+    _numel(_dev(Wq, "Wq"), heads * d * hidden, "Wq")
+    _numel(_dev(Wk, "Wk"), kv_heads * d * hidden, "Wk")
+    _numel(_dev(Wv, "Wv"), kv_heads * d * hidden, "Wv")
+    _numel(_dev(angles, "angles"), rows * d, "angles")
+    _numel(_dev(q_out, "q_out"), rows * heads * d, "q_out")
+    _numel(_dev(keys, "keys"), cache_rows * kv_heads * d, "keys")
+    _numel(_dev(values, "values"), cache_rows * kv_heads * d, "values")
+    check(
+        lib().iron_prefill_qkv_cache_bf16(ptr(x), ptr(Wq), ptr(Wk), ptr(Wv), ptr(angles), ptr(q_out), ptr(keys),
+                                          ptr(values), rows, hidden, heads, kv_heads, d, cache_rows,
+                                          ptr(_word(start, "start")), ptr(_word(valid, "valid")), current_stream()),
+        "iron_prefill_qkv_cache_bf16",
+    )
+
+
 def rmsnorm(x, w, y, *, rows, cols, eps, valid=None):
     _numel(_dev(x, "x"), rows * cols, "x")
     _numel(_dev(y, "y"), rows * cols, "y")

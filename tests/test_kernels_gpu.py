@@ -183,6 +183,38 @@ def test_prefill_qkv_equals_three_projections_then_rope(cuda, rows, bound, H, G)
         assert np.all(got[lim:] == 7.0)
 
 
+@pytest.mark.parametrize("rows,bound,start,L,H,G", [(256, 150, 300, 1024, 16, 4), (2048, 512, 0, 2048, 32, 8),
+                                                    (2048, 1500, 548, 2048, 32, 8), (128, None, 128, 256, 2, 2),
+                                                    (256, 64, 960, 1024, 6, 2)])
+def test_prefill_qkv_writes_k_and_v_into_the_cache_rows(cuda, rows, bound, start, L, H, G):
+    """k and v land in rows start .. start + bound of the caches, bit for bit what the launch with
+    outputs of its own writes; every other cache row is left as it was."""
+    rng = np.random.default_rng(92)
+    E, D = 512, 64
+    x = bf(rng, rows, E)
+    Wq, Wk, Wv = bf(rng, H * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05)
+    table = round_bf16(ops.rope_angles(D, rows, 500000.0))
+    lim = rows if bound is None else bound
+    if bound is not None:
+        x[bound:] = np.nan
+    valid = None if bound is None else word(bound, cuda)
+    args = [dev(a, cuda) for a in (x, Wq, Wk, Wv, table)]
+    outs = [out_like((rows, n), cuda, fill=7.0) for n in (H * D, G * D, G * D)]
+    K.prefill_qkv(*args, *outs, rows=rows, hidden=E, heads=H, kv_heads=G, d=D, valid=valid)
+    q = out_like((rows, H * D), cuda, fill=7.0)
+    keys, values = (out_like((L, G * D), cuda, fill=3.0) for _ in range(2))
+    K.prefill_qkv_cache(*args, q, keys, values, rows=rows, hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
+                        start=word(start, cuda), valid=valid)
+    assert torch.equal(q, outs[0])
+    for cache, own in ((keys, outs[1]), (values, outs[2])):
+        assert torch.equal(cache[start : start + lim], own[:lim])
+        assert bool((cache[:start] == 3.0).all()) and bool((cache[start + lim :] == 3.0).all())
+    # A first row whose rows would end past the cache is held inside it.
+    K.prefill_qkv_cache(*args, q, keys, values, rows=rows, hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
+                        start=word(L, cuda), valid=valid)
+    assert torch.equal(keys[L - lim :], outs[1][:lim])
+
+
 @pytest.mark.parametrize("M,Kdim,N,rows,scale", [(2048, 512, 2048, None, 1.0), (2048, 256, 2048, 512, 1.0),
                                                  (2048, 256, 2048, 1500, 0.22), (256, 128, 512, 100, 1.0),
                                                  (128, 64, 64, None, -0.5), (4096, 192, 1024, 3000, 1.0)])

@@ -202,12 +202,12 @@ def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
     assert plain.decode_step.launches_per_call == steps
     # per layer 18 steps become 5 launches (qkv, attention, o+add, gate/up, down+add); the head 2 -> 1.
     assert fused.decode_step.launches_per_call == 2 + 5 * SCALED.num_hidden_layers + 2
-    # the prompt chunk: per layer the three projections and two rotations become one launch, the
-    # feed-forward's SiLU and Mul another, each residual sum rides its projection's epilogue, and
-    # the last row's final norm and head are one
+    # the prompt chunk: per layer the three projections, two rotations and two cache writes become
+    # one launch, the feed-forward's SiLU and Mul another, each residual sum rides its projection's
+    # epilogue, and the last row's final norm and head are one
     psteps = len(fused.prompt_chunk.recording.steps)
     assert plain.prompt_chunk.launches_per_call == psteps
-    assert fused.prompt_chunk.launches_per_call == psteps - 7 * SCALED.num_hidden_layers - 1
+    assert fused.prompt_chunk.launches_per_call == psteps - 9 * SCALED.num_hidden_layers - 1
     prompt = np.random.default_rng(7).integers(0, SCALED.vocab_size, 8)
     a, b = fused.logits(prompt), plain.logits(prompt)
     assert np.abs(a - b).max() <= 0.02 * np.abs(b).max()
