@@ -3,7 +3,7 @@
 
 ``python bench.py [--gpus 1] [--steps K] [--warmup W]`` prints ONE JSON line.
 
-Workload (BASELINE.json configs): the bf16 GEMM (M=N=K=2048), the decode GEMV
+Workload: the reference's benchmark configurations -- the bf16 GEMM (M=N=K=2048), the decode GEMV
 sweep and the Llama-3.2-1B-shape decode step.  A "step" is one pass over the
 workload's timed unit.  Inputs are synthetic (seeded numpy draws, bf16) and
 resident in HBM before the timed region.  Kernels are timed with HIP events on
@@ -406,7 +406,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is a one-GPU hot path; --gpus must be 1 "
-              "(sharding is described in DESIGN.md, not built)", file=sys.stderr)
+              "(how the path would shard is described, not built)", file=sys.stderr)
         return 2
 
     import torch
