@@ -12,6 +12,7 @@ import pytest
 
 import oracle
 from iron_amd.applications.llama import LLAMA_3_2_1B, Llama, shapes
+from iron_amd.lm.blocks import KVCache
 from iron_amd.lm.causal import OnHost
 from oracle import ops
 from tests.llama_support import BIASED, BIASED_GOLDEN, SCALED, Golden, assert_close, kl, weights
@@ -145,12 +146,17 @@ def test_refusals_before_any_dispatch(toy):
     # one KV head (multi-query), a sliding window shorter than the prompt
     dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=1, head_dim=64, intermediate_size=1024,
          sliding_window=48),
-], ids=["d128", "twelve_heads_untied", "multi_query_window"])
+    # a window short enough against the context that the layers keep rings (128 rows, wrapped by the 200-token prompt)
+    dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=2, head_dim=64, intermediate_size=1024,
+         sliding_window=20, max_seq_len=1024),
+], ids=["d128", "twelve_heads_untied", "multi_query_window", "ring"])
 def test_other_decoder_shapes_match_the_host_reference(cuda, shape):
     """Shapes off the benchmark's: every fused path either takes the shape or leaves the steps as
     recorded; either way the GPU's logits are the host reference's, prompt (in two chunks) and decode."""
-    config = dataclasses.replace(SCALED, vocab_size=1000, num_hidden_layers=2, max_seq_len=256, prefill_chunk=64,
-                                 rope_scaling=None, **shape)
+    config = dataclasses.replace(SCALED, **(dict(vocab_size=1000, num_hidden_layers=2, max_seq_len=256,
+                                                 prefill_chunk=64, rope_scaling=None) | shape))
+    ring = config.max_seq_len > 256
+    assert KVCache(config, config.window).ring == (128 if ring else None)
     names = dict(shapes(config))
     if not config.tie_word_embeddings:
         names["lm_head.weight"] = (config.vocab_size, config.hidden_size)
@@ -159,7 +165,7 @@ def test_other_decoder_shapes_match_the_host_reference(cuda, shape):
     gpu.load_versions()
     cpu.load_versions()
     try:
-        tokens = np.random.default_rng(5).integers(0, config.vocab_size, 90)
+        tokens = np.random.default_rng(5).integers(0, config.vocab_size, 200 if ring else 90)
         want, got = cpu.logits(tokens), gpu.logits(tokens)
         assert_close(got, want)
         for step in range(3):

@@ -1,0 +1,134 @@
+"""The decoder's memory modules, device-free: windows, rings, restarts and per-layer RoPE tables
+(iron/tests/lm/test_modules.py:216-300), on the toy Llama through the host stand-in."""
+
+import dataclasses
+
+import numpy as np
+import pytest
+
+import oracle
+from iron_amd.applications.llama import Llama
+from iron_amd.lm.blocks import Attention, KVCache, Rope
+from iron_amd.lm.causal import OnHost
+from tests.llama_support import SCALED, weights
+
+oracle.install()
+
+
+class HostLlama(OnHost, Llama):
+    pass
+
+
+def small(cls=Llama, **changes):
+    config = dataclasses.replace(SCALED, **changes)
+    return cls(config, weights(config))
+
+
+def names(recording):
+    return [type(s.op).__name__ for s in recording.steps]
+
+
+def test_attention_refuses_a_norm_of_other_than_q_k_and_v():
+    with pytest.raises(ValueError, match="'qo' names other than q, k and v"):
+        Attention(SCALED, 0, norms="qo")
+
+
+def test_a_cache_attends_within_its_window():
+    """Each layer's cache attends within the config's ``sliding_window``, the query's own position
+    not counted; one built with no window attends to every position before the query."""
+    model = small(sliding_window=65)
+    model.layers[1].cache = KVCache(model.config)
+    t = model.record(**model.shapes()[1])
+    assert [s.op.window for s in t.steps if type(s.op).__name__ == "MHA"] == [64, None]
+
+
+def test_a_ring_restarts_at_the_chunk_while_it_holds_the_window_before():
+    """A ring of 128 positions, a window of 7 and a chunk of 64: positions from 70 on changed after
+    70 or 185 ran restart at 64, whose window from 57 the ring still holds, and after 186 at the first."""
+    cache = KVCache(dataclasses.replace(SCALED, prefill_chunk=64, max_seq_len=512), 7)
+    assert cache.ring == 128 and cache.keys.shape[0] == 256 and cache.staged[0].shape[0] == 128
+    assert [cache.restart(70, ran) for ran in (70, 185, 186)] == [64, 64, 0]
+
+
+def test_a_window_keeps_every_position_where_a_ring_takes_as_many_rows():
+    """A ring and its staging take three rings' rows: at a context of three rings or fewer the cache
+    keeps every position, at any chunk, a short context's whole one among them."""
+    for L, C in ((384, 64), (200, 200)):
+        cache = KVCache(dataclasses.replace(SCALED, prefill_chunk=C, max_seq_len=L), 7)
+        assert cache.ring is None and cache.keys.shape[0] == L
+    with pytest.raises(ValueError, match="no power of two"):
+        KVCache(dataclasses.replace(SCALED, prefill_chunk=48, max_seq_len=4096), 7)
+
+
+def test_a_ring_s_rows_are_per_call_words_of_the_position():
+    """A decode step over a ring writes the new row and its mirror and copies the window out; every
+    row is a word derived from ``position`` on the device (remainders by the ring, clamps)."""
+    model = small(sliding_window=8, max_seq_len=4096, prefill_chunk=64)
+    assert model.layers[0].cache.ring == 128 and len(model.recurrent) == 2
+    t = model.record()
+    values = {"token": 5, "position": 300}
+    full = t.check_values(values)
+    found = {e.name: e.evaluate(full) for s in t.steps for h in (*s.inputs.values(), *s.outputs.values())
+             for e in (h.index, h.valid.get(0)) if e is not None and e.value == "position"}
+    assert found["position_r128"] == 300 % 128 and found["position_r128_p128"] == 300 % 128 + 128
+    assert found["position_m7_c0__r128"] == (300 - 7) % 128 and found["position_p1_c_8"] == 8
+    assert names(t).count("MHA") == 2 and names(t).count("Copy") >= 2 + 2 * 6
+
+
+def test_a_ring_s_chunk_attends_from_its_valid_rows_alone():
+    """A chunk's queries over a ring are its whole chunk, the rows past ``rows`` masked; the output is
+    bounded to ``rows`` again, so ``o_proj`` runs on them alone."""
+    model = small(sliding_window=8, max_seq_len=4096)
+    assert model.layers[0].cache.ring == 512
+    t = model.record(**model.shapes()[1])
+    mha = names(t).index("MHA")
+    assert not t.steps[mha].inputs["Q"].valid and "valid" not in t.steps[mha].values
+    o_proj = next(s for s in t.steps[mha + 1 :] if type(s.op).__name__ == "GEMM")
+    assert o_proj.values["valid"].name == "rows"
+
+
+def test_a_turn_over_a_ring_is_the_run_from_scratch_bit_for_bit():
+    """A turn of 150 tokens after 550 ran, over a ring of 512 positions and chunks of 256, reruns its
+    chunk from 512; its logits are those of the whole run from scratch."""
+    model = small(HostLlama, sliding_window=65, max_seq_len=4096)
+    model.load_versions()
+    assert model.layers[0].cache.ring == 512
+    rng = np.random.default_rng(1)
+    whole, other = rng.integers(0, model.config.vocab_size, (2, 700))
+    model.logits(whole[:550])
+    assert model.session.resume(550) == 512
+    turn = model.logits(whole)
+    model.logits(other)
+    scratch = model.logits(whole)
+    np.testing.assert_array_equal(turn, scratch)
+
+
+def test_a_ring_gives_the_logits_of_the_whole_cache():
+    """The same weights and window with the whole cache kept (a context of three rings or fewer)
+    and with a ring: the same logits after a prompt of several chunks and after decode steps."""
+    kept = small(HostLlama, sliding_window=20, prefill_chunk=64, max_seq_len=256)
+    ring = small(HostLlama, sliding_window=20, prefill_chunk=64, max_seq_len=1024)
+    assert kept.layers[0].cache.ring is None and ring.layers[0].cache.ring == 128
+    kept.load_versions()
+    ring.load_versions()
+    tokens = np.random.default_rng(2).integers(0, SCALED.vocab_size, 250)
+    for n in (40, 200, 201, 202, 250):
+        # The same keys in another buffer of another length: the sums' order differs, not the keys.
+        a, b = ring.logits(tokens[:n]), kept.logits(tokens[:n])
+        assert np.abs(a - b).max() <= 0.02 * np.abs(b).max() and a.argmax() == b.argmax(), n
+
+
+def test_each_layer_reads_the_rows_of_its_own_rope():
+    """A layer holding another ``Rope`` turns q and k by its table's rows, copied once a call however
+    many layers hold it; one holding none turns nothing."""
+    model = small(num_hidden_layers=3, rope_scaling=None)
+    other = Rope(dataclasses.replace(model.config, rope_theta=1e4))
+    model.layers[1].rope = model.layers[2].rope = other
+    t = model.record(**model.shapes()[1])
+    tables = {id(h.buffer.source) for s in t.steps for h in s.inputs.values() if h.buffer.kind == "resident"}
+    assert {id(model.rotary_emb.table), id(other.table)} <= tables
+    assert names(t).count("RoPE") == 6
+    model.layers[0].rope = None
+    t = model.record(**model.shapes()[1])
+    tables = {id(h.buffer.source) for s in t.steps for h in s.inputs.values() if h.buffer.kind == "resident"}
+    assert id(model.rotary_emb.table) not in tables and names(t).count("RoPE") == 4
