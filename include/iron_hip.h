@@ -174,7 +174,8 @@ int iron_softmax_bf16(const void* x, int x_is_f32, const float* addend, uint16_t
  * q_tokens = *valid (or seq_len), kv_tokens = *kv_valid (or kv_len - seq + q_tokens).
  * causal masks key > position; window >= 0 also masks key < position - window (and, when not
  * causal, key > position + window); window < 0 = none.  Rows >= q_tokens of O are zeros.
- * d in {64, 128}; heads % kv_heads == 0.
+ * d in {64, 128, 256} (MFMA tiles) or 512 (a block a query row and head scans its keys; seq at
+ * most 65535); heads % kv_heads == 0.
  * Replaces kernels.linalg.mha + partial_softmax + matmul_PV:
  * iron/operators/mha.py:191,574-667,1073-1116. */
 int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
@@ -185,6 +186,7 @@ int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* 
 /* Attention, one query (decode; the reference's "packed" MHA, seq_len == 1).
  * Q,O: (heads, d).  K,V as above.  kv_tokens = *kv_valid (or kv_len); the query sits at
  * kv_tokens - 1.  workspace: iron_mha_decode_workspace_bytes(heads, d) bytes of device memory.
+ * d in {64, 128, 256} with 1, 2, 3, 4, 5, 6 or 8 query heads a KV head, or d = 512 with any.
  * Replaces the packed single-query MHA: iron/operators/mha.py:476-477,1073-1116. */
 int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
                          int heads, int kv_heads, int d, int kv_len, float scale, int window,

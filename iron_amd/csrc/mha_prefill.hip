@@ -366,6 +366,12 @@ static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
   return 0;
 }
 
+// Row-wise attention for 512-wide heads (mha_decode.hip).
+int launch_prefill_rows512(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, int heads, int group,
+                           int seq, int seq_len, int kv_len, float scale_log2, int causal, int window,
+                           long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
+                           const int* valid, const int* kv_valid, void* stream);
+
 }  // namespace iron
 
 using namespace iron;
@@ -378,7 +384,7 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   IRON_REQUIRE(Q && K && V && O, "mha_prefill: null operand");
   IRON_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "mha_prefill: heads (%d) must be a positive multiple of kv_heads (%d)", heads, kv_heads);
-  IRON_REQUIRE(d == 64 || d == 128 || d == 256, "mha_prefill: d (%d) must be 64, 128 or 256", d);
+  IRON_REQUIRE(d == 64 || d == 128 || d == 256 || d == 512, "mha_prefill: d (%d) must be 64, 128, 256 or 512", d);
   IRON_REQUIRE(seq > 0 && seq_len > 0 && seq_len <= seq,
                "mha_prefill: seq_len (%d) must be in [1, seq (%d)]", seq_len, seq);
   IRON_REQUIRE(kv_len >= seq, "mha_prefill: kv_len (%d) must be at least seq (%d): the queries are its last rows",
@@ -391,6 +397,13 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   const long kv_row = kv_interleaved ? (long)kv_heads * d : d;
   const long kv_head = kv_interleaved ? d : (long)kv_len * d;
   const float scale_log2 = scale * 1.4426950408889634f;
+  if (d == 512) {
+    IRON_REQUIRE(seq <= 65535, "mha_prefill: at d = 512 seq (%d) is a grid dimension, at most 65535", seq);
+    const int rc512 = launch_prefill_rows512(Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal,
+                                             window, q_row, q_head, kv_row, kv_head, valid, kv_valid, stream);
+    if (rc512 != 0) return rc512;
+    IRON_LAUNCH_CHECK();
+  }
   const int blocks = ((seq + BQ - 1) / BQ) * heads;
   // Few blocks (a short sequence): the longest block's chain of tiles bounds the launch, so its
   // tiles are split over two halves of eight waves.  Many blocks fill the chip better four waves each.

@@ -94,8 +94,8 @@ class MHA(Operator):
         return self.kv_len - self.seq_pad + self.q_tokens
 
     def validate(self) -> None:
-        if self.d not in (64, 128, 256):
-            raise ValueError(f"MHA: d ({self.d}) must be 64, 128 or 256")
+        if self.d not in (64, 128, 256, 512):
+            raise ValueError(f"MHA: d ({self.d}) must be 64, 128, 256 or 512")
         if self.window is not None and self.window <= 0:
             raise ValueError(f"MHA: window ({self.window}) must be positive or None")
         if not 0 <= self.scale < np.inf:

@@ -41,11 +41,11 @@ def golden():
     return Golden(GOLDEN)
 
 
-def weights():
+def weights(config=TOY):
     """The drawn tensors, q's and k's norms each scaled by ``head_dim ** -0.25``: attention is
     unscaled, so a trained model's norms carry the ``head_dim ** -0.5`` that unit norms leave out
     (tests/applications/gemma4/reference/test.py:110-122)."""
-    w = ops.filled(shapes(TOY), seed=0)
+    w = ops.filled(shapes(config), seed=0)
     for name, weight in w.items():
         if name.endswith(("q_norm.weight", "k_norm.weight")):
             w[name] = round_bf16(weight.astype(np.float32) * np.float32(weight.size**-0.25))
@@ -172,8 +172,11 @@ def test_the_compiled_graph_matches_hugging_face_on_the_gpu(cuda, golden, w):
 
 
 @pytest.mark.gpu
-def test_the_gpu_matches_the_host_step_by_step_past_a_ring(cuda, w):
-    gpu, cpu = Gemma4(TOY, w), host(TOY, w)
+@pytest.mark.parametrize("global_head_dim", [256, 512])   # 512: Gemma 4 E2B's own global heads
+def test_the_gpu_matches_the_host_step_by_step_past_a_ring(cuda, global_head_dim):
+    config = dataclasses.replace(TOY, global_head_dim=global_head_dim)
+    w = weights(config)
+    gpu, cpu = Gemma4(config, w), host(config, w)
     gpu.load_versions()
     try:
         tokens = np.random.default_rng(11).integers(0, TOY.vocab_size, 300)

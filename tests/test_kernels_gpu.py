@@ -450,6 +450,34 @@ def test_mha_prefill_d256_ragged_windowed_and_bounded(cuda):
     close(got[:rows], want[:rows])
 
 
+def test_mha_512_wide_heads_prefill_and_decode(cuda):
+    """512-wide heads (a global layer's of Gemma 4): the row-wise prompt kernel under every mask and
+    a bound, and the one-query kernel on either side of 2048 keys."""
+    rng = np.random.default_rng(22)
+    H, G, d, S, L = 4, 1, 512, 70, 200
+    Q, Kc, Vc = bf(rng, S, H, d) * 0.25, bf(rng, L, G, d) * 0.25, bf(rng, L, G, d)
+    for causal, window in ((True, None), (True, 37), (False, 20), (False, None)):
+        got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=L, causal=causal,
+                                window=window, scale=1.0)
+        close(got, want)
+    Qp, Kp, Vp = Q.copy(), Kc.copy(), Vc.copy()
+    Qp[40:], Kp[150:], Vp[150:] = np.nan, np.nan, np.nan
+    got, want = run_prefill(cuda, Qp, Kp, Vp, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=L, valid=40, kv_valid=150, scale=1.0)
+    assert np.all(got[40:] == 0)
+    close(got[:40], want[:40])
+    for L, kv_valid, window in ((300, 257, None), (4096, 3000, None), (4096, 3000, 99)):
+        H, G = 8, 2
+        Q, Kc, Vc = bf(rng, 1, H, d) * 0.25, bf(rng, L, G, d) * 0.25, bf(rng, L, G, d)
+        Kc[kv_valid:], Vc[kv_valid:] = np.nan, np.nan
+        O = out_like((1, H, d), cuda, fill=float("nan"))
+        K.mha_decode(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, kv_len=L, scale=1.0,
+                     window=window, kv_interleaved=True, kv_valid=word(kv_valid, cuda),
+                     workspace=K.mha_decode_workspace(H, d, cuda))
+        want = ops.mha(Q, Kc, Vc, num_heads=H, num_KV_heads=G, seq_len=1, kv_len=L, d=d, scale=1.0, window=window,
+                       heads_interleaved=True, kv_interleaved=True, kv_valid=kv_valid)
+        close(O, want)
+
+
 @pytest.mark.parametrize("L", [1024, 4096, 16384])
 def test_mha_decode_llama_shape(cuda, L):
     rng = np.random.default_rng(15)
