@@ -636,14 +636,21 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
 // along m: a wave owns 32 rows x 192 columns (6 accumulator tiles), so every head's two halves sit
 // in one wave and RoPE stays in registers.  Three stages of 40 KB; the loop is the 128 x 128
 // kernel's (direct-to-LDS loads, pinned interleave, the stage's barrier before its last k-step).
+// HPT = heads a tile: 3 as above, or 1 -- 128 x 64 tiles, for a row bound so short that wider
+// tiles leave most CUs idle (512 rows of that layer: 192 tiles of one head against 64 of three).
 constexpr int Q3_BM = 128, Q3_BN = 192, Q3_STAGES = 3;
 constexpr int Q3_A_BYTES = Q3_BM * BK * 2, Q3_STAGE_BYTES = (Q3_BM + Q3_BN) * BK * 2;
+constexpr int Q1_STAGE_BYTES = (Q3_BM + 64) * BK * 2;
 
-__device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
-                                            bf16_t* __restrict__ Cq, int M, int heads, int kv_heads, int K,
-                                            const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                            int patched, int run_above, int run_upto, const QkvTail& qkv) {
-  constexpr int A_INST = Q3_BM / 8 / 4, B_INST = Q3_BN / 8 / 4, LOADS = A_INST + B_INST;   // 4 + 6 a wave
+template <int HPT>
+__device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
+                                               bf16_t* __restrict__ Cq, int M, int heads, int kv_heads, int K,
+                                               const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                               int patched, int run_above, int run_upto, const QkvTail& qkv) {
+  constexpr int Q3_BN = 64 * HPT, Q3_STAGE_BYTES = (Q3_BM + Q3_BN) * BK * 2, NACC = 2 * HPT;
+  constexpr int A_INST = Q3_BM / 8 / 4, B_INST = Q3_BN / 8 / 4, LOADS = A_INST + B_INST;   // 4 + 6 (or 2) a wave
+  constexpr int PER = LOADS / 3, REST = LOADS - 3 * PER;   // loads issued under each of a stage's first three k-steps, and its last
+  static_assert(PER <= NACC && REST <= NACC, "a load rides an MFMA");
   extern __shared__ __align__(16) char smem_q3[];
   const int Mv = bound_or(valid, M);
   if (Mv <= run_above || Mv > run_upto) return;
@@ -683,8 +690,8 @@ __device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const 
   }
 #pragma unroll
   for (int i = 0; i < B_INST; ++i) {
-    const int r = (wave * B_INST + i) * 8 + lrow;   // row of the 192-row tile: head r / 64, its row r % 64
-    b_src[i] = head_weight(tn * 3 + r / 64) + (size_t)(r % 64) * K + (pch ^ ((r >> 1) & 7)) * 8;
+    const int r = (wave * B_INST + i) * 8 + lrow;   // row of the tile's weight rows: head r / 64, its row r % 64
+    b_src[i] = head_weight(tn * HPT + r / 64) + (size_t)(r % 64) * K + (pch ^ ((r >> 1) & 7)) * 8;
   }
   auto issue_one = [&](char* st, int kt, int idx) {
     const int k0 = kt * BK;
@@ -696,9 +703,9 @@ __device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const 
                                        IRON_LDS_PTR(st + Q3_A_BYTES + (wave * B_INST + idx - A_INST) * 1024), 16, 0, 0);
   };
 
-  f32x16 acc[6];
+  f32x16 acc[NACC];
 #pragma unroll
-  for (int j = 0; j < 6; ++j)
+  for (int j = 0; j < NACC; ++j)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
 
@@ -717,10 +724,10 @@ __device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const 
 
   wait_vmcnt<LOADS>();   // stage 0 has landed once only stage 1's loads are out
   block_barrier();
-  bf16x8 af[2], bfr[2][6];
+  bf16x8 af[2], bfr[2][NACC];
   af[0] = frag(smem_q3, a_off, 0);
 #pragma unroll
-  for (int j = 0; j < 6; ++j) bfr[0][j] = frag(smem_q3, b_off + j * 32 * 128, 0);
+  for (int j = 0; j < NACC; ++j) bfr[0][j] = frag(smem_q3, b_off + j * 32 * 128, 0);
   for (int kt = 0; kt < nk; ++kt) {
     const int kn = min(kt + Q3_STAGES - 1, nk - 1);
     char* nst = smem_q3 + ((kt + Q3_STAGES - 1) % Q3_STAGES) * Q3_STAGE_BYTES;
@@ -731,23 +738,23 @@ __device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const 
       const int cur = ks & 1, nxt = cur ^ 1;
       const bool last = ks == BK / 16 - 1;
       if (last) {
-        // Of the loads in flight the oldest LOADS are stage kt+1's; the 9 issued so far for stage
+        // Of the loads in flight the oldest LOADS are stage kt+1's; the 3 PER issued so far for stage
         // kt+2 may stay out.  After the barrier nobody reads stage kt any more.
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        wait_vmcnt<9>();
+        wait_vmcnt<3 * PER>();
         block_barrier();
       }
       const char* from = last ? st1 : st;
       const int nks = last ? 0 : ks + 1;
 #pragma unroll
-      for (int j = 0; j < 6; ++j) {
+      for (int j = 0; j < NACC; ++j) {
         acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur], acc[j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (j == 0) af[nxt] = frag(from, a_off, nks);
         bfr[nxt][j] = frag(from, b_off + j * 32 * 128, nks);
-        // Ten loads a stage: three under each of the first three k-steps, the tenth under the last.
-        if (!last && j < 3) issue_one(nst, kn, ks * 3 + j);
-        if (last && j == 0) issue_one(nst, kn, 9);
+        // A stage's loads (ten, or six): PER under each of the first three k-steps, the rest under the last.
+        if (!last && j < PER) issue_one(nst, kn, ks * PER + j);
+        if (last && j < REST) issue_one(nst, kn, 3 * PER + j);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -759,8 +766,8 @@ __device__ __forceinline__ void qkv192_body(const bf16_t* __restrict__ A, const 
   const int m = m0 + wave * 32 + fr;
   const bf16_t* ang = qkv.angles + (size_t)min(m, M - 1) * 64 + 8 * kh;
 #pragma unroll
-  for (int h = 0; h < 3; ++h) {
-    const int g = tn * 3 + h;
+  for (int h = 0; h < HPT; ++h) {
+    const int g = tn * HPT + h;
     bf16_t* C;
     int N, col;
     if (g < heads) { C = Cq; N = heads * 64; col = g * 64; }
@@ -799,7 +806,15 @@ __global__ __launch_bounds__(256) void qkv192_kernel(const bf16_t* __restrict__ 
                                                      const int* __restrict__ valid, int tiles_m, int tiles_n,
                                                      int patched, int run_above, int run_upto, QkvTail qkv) {
   to_cache_rows(qkv, valid, M);
-  qkv192_body(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+  qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+}
+
+__global__ __launch_bounds__(256) void qkv64_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
+                                                    bf16_t* __restrict__ Cq, int M, int heads, int kv_heads, int K,
+                                                    const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                                    int patched, QkvTail qkv) {
+  to_cache_rows(qkv, valid, M);
+  qkv_heads_body<1>(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, -1, INT_MAX, qkv);
 }
 
 // Both tilings in one launch: the row bound is read on the device, and which tiling makes fewer
@@ -813,12 +828,17 @@ __global__ __launch_bounds__(256) void qkv_either_kernel(const bf16_t* __restric
                                                          const bf16_t* __restrict__ Bq, bf16_t* __restrict__ Cq,
                                                          int M, int heads, int kv_heads, int K,
                                                          const int* __restrict__ valid, Tiling narrow, Tiling wide,
-                                                         int above, int wide_top, QkvTail qkv) {
-  const bool past = bound_or(valid, M) > above;
+                                                         Tiling thin, int above, int wide_top, int thin_upto,
+                                                         QkvTail qkv) {
+  const int Mv = bound_or(valid, M);
+  const bool past = Mv > above;
   to_cache_rows(qkv, valid, M);
-  if (past == (wide_top != 0)) {
+  if (Mv <= thin_upto) {   // so few rows that one-head tiles still fit one round over the chip
+    if ((int)blockIdx.x < thin.tiles_m * thin.tiles_n)
+      qkv_heads_body<1>(A, Bq, Cq, M, heads, kv_heads, K, valid, thin.tiles_m, thin.tiles_n, thin.patched, -1, INT_MAX, qkv);
+  } else if (wide.tiles_n > 0 && past == (wide_top != 0)) {
     if ((int)blockIdx.x < wide.tiles_m * wide.tiles_n)
-      qkv192_body(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, -1, INT_MAX, qkv);
+      qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, -1, INT_MAX, qkv);
   } else {
     if ((int)blockIdx.x < narrow.tiles_m * narrow.tiles_n)
       gemm_nt_body<false, true, 2>(A, Bq, Cq, M, heads * 64, K, valid, narrow.tiles_m, narrow.tiles_n, narrow.patched,
@@ -830,11 +850,16 @@ static int patched_order(int tiles_m, int tiles_n) {
   return (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
 }
 
+// wide_ok: the head count comes in threes (else the 192-wide tiling is never chosen).  thin_upto: the
+// row bound up to which the one-head tiles run (0: never).
 static int launch_qkv_either(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, int heads, int kv_heads, int K,
-                             const int* valid, hipStream_t s, QkvTail qkv, int above, bool wide_top) {
-  const int tiles_m = (M + 127) / 128;
-  const Tiling narrow{tiles_m, (heads + 2 * kv_heads) / 2, patched_order(tiles_m, (heads + 2 * kv_heads) / 2)};
-  const Tiling wide{tiles_m, (heads + 2 * kv_heads) / 3, patched_order(tiles_m, (heads + 2 * kv_heads) / 3)};
+                             const int* valid, hipStream_t s, QkvTail qkv, int above, bool wide_top, bool wide_ok,
+                             int thin_upto) {
+  const int tiles_m = (M + 127) / 128, total = heads + 2 * kv_heads;
+  const Tiling narrow{tiles_m, total / 2, patched_order(tiles_m, total / 2)};
+  const Tiling wide{wide_ok ? tiles_m : 0, wide_ok ? total / 3 : 0, wide_ok ? patched_order(tiles_m, total / 3) : 0};
+  const int thin_m = (thin_upto + 127) / 128;
+  const Tiling thin{thin_m, total, patched_order(thin_m, total)};
   const size_t lds_narrow = (size_t)NT_STAGES * 256 * BK * 2, lds_wide = (size_t)Q3_STAGES * Q3_STAGE_BYTES;
   const size_t lds = lds_narrow > lds_wide ? lds_narrow : lds_wide;
   static bool once = false;
@@ -844,9 +869,26 @@ static int launch_qkv_either(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int 
     if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
-  const int blocks = tiles_m * (narrow.tiles_n > wide.tiles_n ? narrow.tiles_n : wide.tiles_n);
+  int blocks = tiles_m * (narrow.tiles_n > wide.tiles_n ? narrow.tiles_n : wide.tiles_n);
+  if (thin.tiles_m * thin.tiles_n > blocks) blocks = thin.tiles_m * thin.tiles_n;
   hipLaunchKernelGGL(qkv_either_kernel, dim3(blocks), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid, narrow,
-                     wide, above, wide_top ? 1 : 0, qkv);
+                     wide, thin, above, wide_top ? 1 : 0, thin_upto, qkv);
+  IRON_LAUNCH_CHECK();
+}
+
+static int launch_qkv64(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, int heads, int kv_heads, int K,
+                        const int* valid, hipStream_t s, QkvTail qkv) {
+  const int tiles_m = (M + Q3_BM - 1) / Q3_BM, tiles_n = heads + 2 * kv_heads;
+  const size_t lds = (size_t)Q3_STAGES * Q1_STAGE_BYTES;
+  static bool once = false;
+  if (!once) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv64_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
+    once = true;
+  }
+  hipLaunchKernelGGL(qkv64_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid,
+                     tiles_m, tiles_n, patched_order(tiles_m, tiles_n), qkv);
   IRON_LAUNCH_CHECK();
 }
 
@@ -1265,18 +1307,32 @@ static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk
     const int tiles = ((live_rows + 127) / 128) * n_tiles;
     return (double)((tiles + cus - 1) / cus) * tile_n;
   };
-  auto wide_wins = [&](int live_rows) { return cost(live_rows, 192, total / 3) < cost(live_rows, 128, total / 2); };
-  if (total % 3 != 0) return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, s, tail);
+  const bool wide_ok = total % 3 == 0;
+  auto wide_wins = [&](int live_rows) {
+    return wide_ok && cost(live_rows, 192, total / 3) < cost(live_rows, 128, total / 2);
+  };
+  // One-head tiles while they fit one round over the chip and beat both of the others' cost.
+  auto thin_wins = [&](int live_rows) {
+    const double c = cost(live_rows, 64, total);
+    return ((live_rows + 127) / 128) * total <= cus && c < cost(live_rows, 128, total / 2) &&
+           (!wide_ok || c < cost(live_rows, 192, total / 3));
+  };
+  int thin_upto = 0;
+  for (int live = 128; live <= ((rows + 127) / 128) * 128; live += 128)
+    if (thin_wins(live)) thin_upto = live;
+  if (thin_upto >= rows) return launch_qkv64(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail);
   // The bound above which the winner at `rows` wins, if the two ever change places below `rows`.
   int above = -1;
   if (valid != nullptr)
     for (int live = 128; live <= rows; live += 128)
       if (wide_wins(live) != wide_wins(rows)) above = live;
-  if (above < 0) {
+  if (valid == nullptr) thin_upto = 0;
+  if (above < 0 && thin_upto == 0) {
     if (wide_wins(rows)) return launch_qkv192(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, -1, INT_MAX);
     return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, s, tail);
   }
-  return launch_qkv_either(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, above, wide_wins(rows));
+  return launch_qkv_either(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, above, wide_wins(rows), wide_ok,
+                           thin_upto);
 }
 
 extern "C" int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
