@@ -132,3 +132,42 @@ def test_each_layer_reads_the_rows_of_its_own_rope():
     t = model.record(**model.shapes()[1])
     tables = {id(h.buffer.source) for s in t.steps for h in s.inputs.values() if h.buffer.kind == "resident"}
     assert id(model.rotary_emb.table) not in tables and names(t).count("RoPE") == 4
+
+
+def test_per_call_expressions_fold_floor_clamp_remainder_and_a_trailing_sum():
+    """What a ring's rows are made of: ``clamp(position - W, 0) % R + R`` is one expression of one
+    value, evaluated alike on the host and by the device's table (its nine-word record)."""
+    from iron_amd.common.graph import Affine, clamp
+
+    p = Affine("position")
+    row = clamp(p - 7, lo=0) % 128
+    assert [row.evaluate({"position": v}) for v in (0, 7, 8, 135, 300)] == [0, 0, 1, 0, 37]
+    mirror = row + 128
+    assert mirror.evaluate({"position": 300}) == 165 and (mirror - row).evaluate({"position": 5}) == 128
+    assert mirror.record() == [1, -7, 0, 0, 2**31 - 1, 127, 128]
+    assert (p * 12 // 12) == p and (p * 12 + 24) // 12 == p + 2      # an even division folds
+    assert ((p + 1) // 4).evaluate({"position": 10}) == 2            # a power of two floors
+    with pytest.raises(TypeError, match="power of two"):
+        (p + 1) // 3
+    with pytest.raises(TypeError, match="power of two"):
+        p % 12
+    with pytest.raises(TypeError):
+        clamp(row, hi=5)          # a clamp after a remainder is not one expression
+    with pytest.raises(TypeError):
+        row * 2
+    assert row.name == "position_m7_c0__r128" and mirror.name == "position_m7_c0__r128_p128"
+
+
+def test_a_number_meets_a_handle_as_a_constant_row():
+    """``x * 0.5`` records one rowwise multiply by a bf16 row of that number, the same tensor
+    wherever the number and width recur (iron/common/graph/handle.py:652-661)."""
+    from iron_amd.common import graph as iron
+
+    class Halve(iron.Graph):
+        def body(self, x):
+            return (x * 0.5 + x / 2) * 0.5
+
+    t = Halve().record(x=((4, 64), iron.bfloat16))
+    assert names(t) == ["RowwiseMul", "RowwiseMul", "ElementwiseAdd", "RowwiseMul"]
+    rows = [s.inputs["row"].buffer.source for s in t.steps if type(s.op).__name__ == "RowwiseMul"]
+    assert rows[0] is rows[1] is rows[2] and np.all(np.asarray(rows[0].array) == 0.5)
