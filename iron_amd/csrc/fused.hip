@@ -106,6 +106,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
   __shared__ float part[4][MATS][RPW];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int row0 = blockIdx.x * RPW;
+  // The residual a thread will add at the end is requested first, so that its trip to memory
+  // passes under the weights' instead of after the block's last barrier.
+  float res_ahead = 0.f;
+  if (EPI == EPI_ADD && threadIdx.x < RPW) res_ahead = bf16_to_f32(res[min(row0 + (int)threadIdx.x, M - 1)]);
   Activation<CH, NORM> act;
   act.issue(x, nw, K);
   uint4 w[MATS][RPW][CH];
@@ -129,7 +133,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
     const int r = threadIdx.x, row = row0 + r;
     if (row < M) {
       float v = round_bf16(part[0][0][r] + part[1][0][r] + part[2][0][r] + part[3][0][r]);  // the GEMV's own rounding
-      if (EPI == EPI_ADD) v = fmaf(res_scale, v, bf16_to_f32(res[row]));   // scale 1: the plain sum
+      if (EPI == EPI_ADD) v = fmaf(res_scale, v, res_ahead);   // scale 1: the plain sum
       if (EPI == EPI_SILU_MUL) {
         const float u = round_bf16(part[0][MATS - 1][r] + part[1][MATS - 1][r] + part[2][MATS - 1][r] +
                                    part[3][MATS - 1][r]);
@@ -162,6 +166,10 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   else if (pair < q_pairs + k_pairs) { kind = 1; Wm = Wk; const int p = pair - q_pairs; const int h = p / HALF; j = p % HALF; r0 = h * D + j; r1 = r0 + HALF; }
   else { kind = 2; Wm = Wv; const int p = pair - q_pairs - k_pairs; r0 = 2 * p; r1 = r0 + 1; }
 
+  // What the block's last thread needs after the last barrier is requested first: the pair's
+  // angle and the position word ride under the weights' trip to memory.
+  const float c_ahead = bf16_to_f32(angles[2 * j]), s_ahead = bf16_to_f32(angles[2 * j + 1]);
+  const int pos_ahead = *position;
   Activation<CH, true> act;
   act.issue(x, nw, K);
   uint4 w0[CH], w1[CH];
@@ -176,7 +184,7 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   float y0 = round_bf16(part[0][0] + part[1][0] + part[2][0] + part[3][0]);  // the projections' own rounding
   float y1 = round_bf16(part[0][1] + part[1][1] + part[2][1] + part[3][1]);
   if (kind != 2) {
-    const float c = bf16_to_f32(angles[2 * j]), s = bf16_to_f32(angles[2 * j + 1]);
+    const float c = c_ahead, s = s_ahead;
     const float t0 = y0 * c - y1 * s, t1 = y1 * c + y0 * s;
     y0 = t0; y1 = t1;
   }
@@ -184,7 +192,7 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
     q_out[r0] = f32_to_bf16(y0);
     q_out[r1] = f32_to_bf16(y1);
   } else {
-    const int pos = *position;
+    const int pos = pos_ahead;
     if (pos >= 0 && pos < cache_rows) {
       bf16_t* dst = (kind == 1 ? keys : values) + (size_t)pos * kv_heads * D;
       dst[r0] = f32_to_bf16(y0);
