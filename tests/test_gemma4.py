@@ -167,6 +167,10 @@ def test_the_compiled_graph_matches_hugging_face_on_the_gpu(cuda, golden, w):
         chunks_against(model, golden, TOY)
         prompt, _, _ = case(golden)
         assert model.generate(prompt, 12) == list(model.session.draw(prompt, 12, each=True))
+        # Replays whose ring rows the device derives from the carried position, across the wrap
+        # (positions 100 .. 159 over rings of 128 rows), against steps whose words the host wrote.
+        long = np.random.default_rng(12).integers(0, TOY.vocab_size, 100)
+        assert model.generate(long, 60) == list(model.session.draw(long, 60, each=True))
     finally:
         model.release()
 
