@@ -388,10 +388,29 @@ def counter_probe(torch, K, dev, rng):
         K.gemv(pool[i % 2], x, y, M=N, K=Kdim)
     for _ in range(2):
         K.copy_rows(src, dst, rows=rows, row_elems=row_bytes // 4, src_rows=rows, dst_rows=rows)
+    # The MFMA kernels, for a run that reads the matrix pipe's counters: the headline GEMM (weights as
+    # stored, (N,K)), the 256 x 256-tile kernel at 8192^3, and prompt attention at S = 2048 and 8192.
+    def drawn(*shape, scale=0.02):
+        return (torch.randn(*shape, device=dev) * scale).to(torch.bfloat16)
+
+    for n_, launches in ((2048, 3), (8192, 2)):
+        A, B, C = drawn(n_, n_), drawn(n_, n_), torch.empty((n_, n_), dtype=torch.bfloat16, device=dev)
+        for _ in range(launches):
+            K.gemm(A, B, C, M=n_, N=n_, K=n_, b_col_maj=True)
+        del A, B, C
+    H, G, D = 32, 8, 64
+    for S in (2048, 8192):
+        Q, Kc, Vc = drawn(S, H, D, scale=1.0), drawn(S, G, D, scale=1.0), drawn(S, G, D, scale=1.0)
+        O = torch.empty_like(Q)
+        for _ in range(2):
+            K.mha_prefill(Q, Kc, Vc, O, heads=H, kv_heads=G, d=D, seq=S, seq_len=S, kv_len=S, scale=D**-0.5, causal=True,
+                          q_interleaved=True, kv_interleaved=True)
     torch.cuda.synchronize()
     print(json.dumps({"probe": "counter", "gemv": {"K": Kdim, "N": N, "launches": 4,
                                                      "algorithmic_bytes": 2 * (N * Kdim + Kdim + N)},
-                      "copy": {"launches": 2, "bytes_read": PROBE_COPY_BYTES, "bytes_written": PROBE_COPY_BYTES}}))
+                      "copy": {"launches": 2, "bytes_read": PROBE_COPY_BYTES, "bytes_written": PROBE_COPY_BYTES},
+                      "gemm": [{"n": 2048, "launches": 3}, {"n": 8192, "launches": 2}],
+                      "attention_prefill": [{"S": 2048, "launches": 2}, {"S": 8192, "launches": 2}]}))
 
 
 def main():
@@ -402,7 +421,7 @@ def main():
     ap.add_argument("--kernel-launches", type=int, default=400, help="timed launches per kernel micro-benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--counter-probe", action="store_true",
-                    help="launch only the LM-head GEMV and a plain copy of known size (for a rocprofv3 --pmc run) and exit")
+                    help="launch only the LM-head GEMV, a plain copy of known size and the MFMA kernels (for a rocprofv3 --pmc run) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is a one-GPU hot path; --gpus must be 1 "
