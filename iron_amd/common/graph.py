@@ -593,11 +593,14 @@ class Recorder:
             bound.setdefault(name, expr)
         for k, v in bound.items():
             op.use_value(k, v)
-        # Operand sizes must be the declared ones.
+        # Operand sizes must be the declared ones, and only an operand that says so may be a view
+        # whose rows a call names (the launch would read the buffer from its first row).
         for b in op.inputs:
             h = inputs[b.name]
             if h.elements != b.elements and not op.takes_view(b.name):
                 raise ValueError(f"{b.name} takes {b.shape}, got {h.shape}")
+            if (h.index is not None or h.ids is not None) and not op.takes_view(b.name):
+                raise TypeError(f"{b.name} is a per-call view: Copy.step() it into a tensor of its own first")
         outputs: dict[str, Handle] = {}
         declared_out = op.outputs
         for i, b in enumerate(declared_out):
