@@ -182,6 +182,14 @@ int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* 
                           int heads, int kv_heads, int d, int seq, int seq_len, int kv_len,
                           float scale, int causal, int window, int q_interleaved,
                           int kv_interleaved, const int* valid, const int* kv_valid, void* stream);
+/* The same over a window of a longer buffer of keys: K, V (kv_rows, kv_heads, d), of which the kv_len
+ * rows from *kv_first on are the keys (the first row is held where they end inside the buffer).  What
+ * a sliding-window layer's ring cache needs (iron/lm/blocks.py:504-529: the reference copies the
+ * window into a staging tensor first; here attention reads it where it lies). */
+int iron_mha_prefill_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
+                             int heads, int kv_heads, int d, int seq, int seq_len, int kv_len,
+                             float scale, int causal, int window, int q_interleaved, const int* valid,
+                             const int* kv_valid, const int* kv_first, int kv_rows, void* stream);
 
 /* Attention, one query (decode; the reference's "packed" MHA, seq_len == 1).
  * Q,O: (heads, d).  K,V as above.  kv_tokens = *kv_valid (or kv_len); the query sits at
@@ -192,6 +200,11 @@ int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int heads, int kv_heads, int d, int kv_len, float scale, int window,
                          int kv_interleaved, const int* kv_valid, void* workspace, void* stream);
 int64_t iron_mha_decode_workspace_bytes(int heads, int d);
+/* One query over a window of a longer buffer of keys, as iron_mha_prefill_at_bf16. */
+int iron_mha_decode_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
+                            int heads, int kv_heads, int d, int kv_len, float scale, int window,
+                            const int* kv_valid, const int* kv_first, int kv_rows, void* workspace,
+                            void* stream);
 
 /* out[i] = table[ids[i]] for i < *valid (or n_ids); rows of row_bytes bytes (multiple of 4).
  * ids outside [0, table_rows) are skipped (the row is left untouched).

@@ -46,6 +46,14 @@ SIGNATURES = {
         [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, _P, _P],
     ),
     "iron_mha_decode_workspace_bytes": (c_int64, [c_int, c_int]),
+    "iron_mha_prefill_at_bf16": (
+        c_int,
+        [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, _P, _P, c_int, _P],
+    ),
+    "iron_mha_decode_at_bf16": (
+        c_int,
+        [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P, _P, c_int, _P, _P],
+    ),
     "iron_gather_rows": (c_int, [_P, _P, _P, c_int, c_int, c_int64, _P, _P]),
     "iron_copy_rows": (c_int, [_P, _P, c_int, c_int64, c_int64, c_int64, c_int, c_int, _P, _P, _P, _P]),
     "iron_argmax_bf16": (c_int, [_P, c_int, _P, _P, c_int, _P, _P, _P]),

@@ -134,11 +134,16 @@ template <int D, int G>
 __global__ __launch_bounds__(256) void mha_decode_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     float* __restrict__ part, int kv_len, float scale_log2, int window, long row_stride,
-    long head_stride, const int* __restrict__ kv_valid) {
+    long head_stride, const int* __restrict__ kv_valid, const int* __restrict__ kv_first, int kv_rows) {
   constexpr int LPR = D / 8, RW = 64 / LPR;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPR, rg = lane / LPR;
   const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y;
+  if (kv_first) {   // the keys are a window of a longer buffer, rows *kv_first on (held inside it)
+    const long first_row = max(0, min(*kv_first, kv_rows - kv_len));
+    K += first_row * row_stride;
+    V += first_row * row_stride;
+  }
 
   const int kv_tokens = bound_or(kv_valid, kv_len);
   const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
@@ -234,11 +239,17 @@ template <int D>
 __global__ __launch_bounds__(1024) void mha_decode_single_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int kv_len, int kv_heads, int group, float scale_log2, int window,
-    long row_stride, long head_stride, const int* __restrict__ kv_valid) {
+    long row_stride, long head_stride, const int* __restrict__ kv_valid, const int* __restrict__ kv_first,
+    int kv_rows) {
   constexpr int LPR = D / 8, RW = 64 / LPR, WAVES = 16, U = 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPR, rg = lane / LPR;
   const int kvh = blockIdx.x % kv_heads, head = kvh * group + blockIdx.x / kv_heads;
+  if (kv_first) {   // the keys are a window of a longer buffer, rows *kv_first on (held inside it)
+    const long first_row = max(0, min(*kv_first, kv_rows - kv_len));
+    K += first_row * row_stride;
+    V += first_row * row_stride;
+  }
 
   const int kv_tokens = bound_or(kv_valid, kv_len);
   const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
@@ -284,11 +295,16 @@ __global__ __launch_bounds__(1024) void mha_prefill_rows_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int group, int seq, int seq_len, int kv_len, float scale_log2, int causal,
     int window, long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
-    const int* __restrict__ valid, const int* __restrict__ kv_valid) {
+    const int* __restrict__ valid, const int* __restrict__ kv_valid, const int* __restrict__ kv_first, int kv_rows) {
   constexpr int LPR = D / 8, RW = 64 / LPR, WAVES = 16, U = 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPR, rg = lane / LPR;
   const int head = blockIdx.x, row = blockIdx.y, kvh = head / group;
+  if (kv_first) {   // the keys are a window of a longer buffer, rows *kv_first on (held inside it)
+    const long first_row = max(0, min(*kv_first, kv_rows - kv_len));
+    K += first_row * kv_row_stride;
+    V += first_row * kv_row_stride;
+  }
 
   const int q_tokens = valid ? bound_or(valid, seq) : seq_len;
   const int kv_tokens = kv_valid ? bound_or(kv_valid, kv_len) : (kv_len - seq + q_tokens);
@@ -342,19 +358,20 @@ __global__ __launch_bounds__(1024) void mha_prefill_rows_kernel(
 int launch_prefill_rows512(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, int heads, int group,
                            int seq, int seq_len, int kv_len, float scale_log2, int causal, int window,
                            long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
-                           const int* valid, const int* kv_valid, void* stream) {
+                           const int* valid, const int* kv_valid, const int* kv_first, int kv_rows, void* stream) {
   hipLaunchKernelGGL(mha_prefill_rows_kernel<512>, dim3(heads, seq), dim3(1024), 0, (hipStream_t)stream, Q, K, V, O,
                      group, seq, seq_len, kv_len, scale_log2, causal, window, q_row_stride, q_head_stride,
-                     kv_row_stride, kv_head_stride, valid, kv_valid);
+                     kv_row_stride, kv_head_stride, valid, kv_valid, kv_first, kv_rows);
   return 0;
 }
 
 template <int D, int G>
 static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, float* part,
                           int kv_heads, int kv_len, float scale_log2, int window, long row_stride,
-                          long head_stride, const int* kv_valid, int nsplit, hipStream_t s) {
+                          long head_stride, const int* kv_valid, const int* kv_first, int kv_rows, int nsplit,
+                          hipStream_t s) {
   hipLaunchKernelGGL((mha_decode_kernel<D, G>), dim3(nsplit, kv_heads), dim3(256), 0, s, Q, K, V,
-                     part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid);
+                     part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
   hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D > kMaxSplits ? D : kMaxSplits), 0, s,
                      part, O, nsplit);
 }
@@ -367,11 +384,13 @@ extern "C" int64_t iron_mha_decode_workspace_bytes(int heads, int d) {
   return (int64_t)heads * kMaxSplits * (d + 2) * sizeof(float);
 }
 
-extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
-                                    uint16_t* O, int heads, int kv_heads, int d, int kv_len,
-                                    float scale, int window, int kv_interleaved,
-                                    const int* kv_valid, void* workspace, void* stream) {
+static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O, int heads, int kv_heads,
+                      int d, int kv_len, float scale, int window, int kv_interleaved, const int* kv_valid,
+                      const int* kv_first, int kv_rows, void* workspace, void* stream) {
   IRON_REQUIRE(Q && K && V && O && workspace, "mha_decode: null operand");
+  IRON_REQUIRE(kv_first == nullptr || (kv_interleaved && kv_rows >= kv_len),
+               "mha_decode: a window of the keys takes them row by row (kv_interleaved) out of kv_rows (%d) >= kv_len (%d)",
+               kv_rows, kv_len);
   IRON_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "mha_decode: heads (%d) must be a positive multiple of kv_heads (%d)", heads, kv_heads);
   IRON_REQUIRE(kv_len > 0, "mha_decode: kv_len (%d) must be positive", kv_len);
@@ -395,22 +414,22 @@ extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const 
     const dim3 grid(heads), block(1024);
     if (d == 512)
       hipLaunchKernelGGL(mha_decode_single_kernel<512>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
-                         scale_log2, window, row_stride, head_stride, kv_valid);
+                         scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
     else if (d == 64)
       hipLaunchKernelGGL(mha_decode_single_kernel<64>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
-                         scale_log2, window, row_stride, head_stride, kv_valid);
+                         scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
     else if (d == 128)
       hipLaunchKernelGGL(mha_decode_single_kernel<128>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
-                         scale_log2, window, row_stride, head_stride, kv_valid);
+                         scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
     else
       hipLaunchKernelGGL(mha_decode_single_kernel<256>, grid, block, 0, s, Q, K, V, O, kv_len, kv_heads, G,
-                         scale_log2, window, row_stride, head_stride, kv_valid);
+                         scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
     IRON_LAUNCH_CHECK();
   }
 #define IRON_DEC(DD, GG)                                                                        \
   if (d == DD && G == GG) {                                                                     \
     launch_decode<DD, GG>(Q, K, V, O, part, kv_heads, kv_len, scale_log2, window, row_stride,   \
-                          head_stride, kv_valid, nsplit, s);                                    \
+                          head_stride, kv_valid, kv_first, kv_rows, nsplit, s);                 \
     IRON_LAUNCH_CHECK();                                                                        \
   }
 #define IRON_DEC_D(DD) \
@@ -420,4 +439,21 @@ extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const 
 #undef IRON_DEC
   IRON_REQUIRE(false, "mha_decode: no kernel for d=%d with %d query heads per KV head "
                "(d in {64,128,256} with a group in {1,2,3,4,5,6,8}, or d = 512)", d, G);
+}
+
+extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                    uint16_t* O, int heads, int kv_heads, int d, int kv_len,
+                                    float scale, int window, int kv_interleaved,
+                                    const int* kv_valid, void* workspace, void* stream) {
+  return mha_decode(Q, K, V, O, heads, kv_heads, d, kv_len, scale, window, kv_interleaved, kv_valid, nullptr, 0,
+                    workspace, stream);
+}
+
+extern "C" int iron_mha_decode_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                       uint16_t* O, int heads, int kv_heads, int d, int kv_len,
+                                       float scale, int window, const int* kv_valid, const int* kv_first,
+                                       int kv_rows, void* workspace, void* stream) {
+  IRON_REQUIRE(kv_first != nullptr, "mha_decode_at: null kv_first");
+  return mha_decode(Q, K, V, O, heads, kv_heads, d, kv_len, scale, window, 1, kv_valid, kv_first, kv_rows, workspace,
+                    stream);
 }

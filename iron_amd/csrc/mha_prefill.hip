@@ -40,7 +40,8 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
-    long kv_head_stride, const int* __restrict__ valid, const int* __restrict__ kv_valid) {
+    long kv_head_stride, const int* __restrict__ valid, const int* __restrict__ kv_valid,
+    const int* __restrict__ kv_first, int kv_rows) {
   constexpr int ROWB = D * 2;            // bytes of a tile row
   constexpr int KS = D / 16;             // k16 steps of S^T
   constexpr int DT = D / 32;             // 32-row tiles of O^T
@@ -121,8 +122,10 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   const int steps = (ntiles + SPLIT - 1) / SPLIT;
 
   if (ntiles > 0) {
-    const bf16_t* Kh = K + (size_t)kvh * kv_head_stride;
-    const bf16_t* Vh = V + (size_t)kvh * kv_head_stride;
+    // The keys may be a window of a longer buffer, rows *kv_first on (held inside the buffer).
+    const long first_row = kv_first ? max(0, min(*kv_first, kv_rows - kv_len)) : 0;
+    const bf16_t* Kh = K + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
+    const bf16_t* Vh = V + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
 
     // Loader: load i of a wave covers tile rows (wave*INST + i)*RPI .. ; lane -> (row, physical
     // chunk), and fetches the logical chunk that the row's swizzle maps there.  Rows past the
@@ -346,6 +349,8 @@ struct PrefillArgs {
   int causal, window;
   long q_row, q_head, kv_row, kv_head;
   const int *valid, *kv_valid;
+  const int* kv_first;
+  int kv_rows;
 };
 
 // The stage buffers are dynamic LDS (more than the 64 KB a kernel may declare statically).
@@ -362,7 +367,7 @@ static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
   }
   hipLaunchKernelGGL((mha_prefill_kernel<D, SPLIT>), dim3(blocks), dim3(256 * SPLIT), lds, (hipStream_t)stream, a.Q,
                      a.K, a.V, a.O, a.heads, a.group, a.seq, a.seq_len, a.kv_len, a.scale_log2, a.causal, a.window,
-                     a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid);
+                     a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid, a.kv_first, a.kv_rows);
   return 0;
 }
 
@@ -370,18 +375,20 @@ static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
 int launch_prefill_rows512(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, int heads, int group,
                            int seq, int seq_len, int kv_len, float scale_log2, int causal, int window,
                            long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
-                           const int* valid, const int* kv_valid, void* stream);
+                           const int* valid, const int* kv_valid, const int* kv_first, int kv_rows, void* stream);
 
 }  // namespace iron
 
 using namespace iron;
 
-extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
-                                     uint16_t* O, int heads, int kv_heads, int d, int seq,
-                                     int seq_len, int kv_len, float scale, int causal, int window,
-                                     int q_interleaved, int kv_interleaved, const int* valid,
-                                     const int* kv_valid, void* stream) {
+static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O, int heads, int kv_heads,
+                       int d, int seq, int seq_len, int kv_len, float scale, int causal, int window, int q_interleaved,
+                       int kv_interleaved, const int* valid, const int* kv_valid, const int* kv_first, int kv_rows,
+                       void* stream) {
   IRON_REQUIRE(Q && K && V && O, "mha_prefill: null operand");
+  IRON_REQUIRE(kv_first == nullptr || (kv_interleaved && kv_rows >= kv_len),
+               "mha_prefill: a window of the keys takes them row by row (kv_interleaved) out of kv_rows (%d) >= kv_len (%d)",
+               kv_rows, kv_len);
   IRON_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                "mha_prefill: heads (%d) must be a positive multiple of kv_heads (%d)", heads, kv_heads);
   IRON_REQUIRE(d == 64 || d == 128 || d == 256 || d == 512, "mha_prefill: d (%d) must be 64, 128, 256 or 512", d);
@@ -400,7 +407,8 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   if (d == 512) {
     IRON_REQUIRE(seq <= 65535, "mha_prefill: at d = 512 seq (%d) is a grid dimension, at most 65535", seq);
     const int rc512 = launch_prefill_rows512(Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal,
-                                             window, q_row, q_head, kv_row, kv_head, valid, kv_valid, stream);
+                                             window, q_row, q_head, kv_row, kv_head, valid, kv_valid, kv_first, kv_rows,
+                                             stream);
     if (rc512 != 0) return rc512;
     IRON_LAUNCH_CHECK();
   }
@@ -409,11 +417,30 @@ extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const
   // tiles are split over two halves of eight waves.  Many blocks fill the chip better four waves each.
   const bool split = blocks <= kSplitMaxBlocks;
   PrefillArgs a{Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window,
-                q_row, q_head, kv_row, kv_head, valid, kv_valid};
+                q_row, q_head, kv_row, kv_head, valid, kv_valid, kv_first, kv_rows};
   int rc;
   if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
   else if (d == 128) rc = split ? launch_prefill<128, 2>(a, blocks, stream) : launch_prefill<128, 1>(a, blocks, stream);
   else rc = launch_prefill<256, 1>(a, blocks, stream);
   if (rc != 0) return rc;
   IRON_LAUNCH_CHECK();
+}
+
+extern "C" int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                     uint16_t* O, int heads, int kv_heads, int d, int seq,
+                                     int seq_len, int kv_len, float scale, int causal, int window,
+                                     int q_interleaved, int kv_interleaved, const int* valid,
+                                     const int* kv_valid, void* stream) {
+  return mha_prefill(Q, K, V, O, heads, kv_heads, d, seq, seq_len, kv_len, scale, causal, window, q_interleaved,
+                     kv_interleaved, valid, kv_valid, nullptr, 0, stream);
+}
+
+extern "C" int iron_mha_prefill_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                        uint16_t* O, int heads, int kv_heads, int d, int seq,
+                                        int seq_len, int kv_len, float scale, int causal, int window,
+                                        int q_interleaved, const int* valid, const int* kv_valid,
+                                        const int* kv_first, int kv_rows, void* stream) {
+  IRON_REQUIRE(kv_first != nullptr, "mha_prefill_at: null kv_first");
+  return mha_prefill(Q, K, V, O, heads, kv_heads, d, seq, seq_len, kv_len, scale, causal, window, q_interleaved, 1,
+                     valid, kv_valid, kv_first, kv_rows, stream);
 }

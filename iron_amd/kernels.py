@@ -263,12 +263,26 @@ def softmax(x, y, *, rows, cols, addend=None, soft_cap=None, length=None):
 
 def mha_prefill(
     Q, K, V, O, *, heads, kv_heads, d, seq, seq_len=None, kv_len, scale=None, causal=True,
-    window=None, q_interleaved=False, kv_interleaved=False, valid=None, kv_valid=None,
+    window=None, q_interleaved=False, kv_interleaved=False, valid=None, kv_valid=None, kv_first=None, kv_rows=None,
 ):
+    """``kv_first`` (a device word) and ``kv_rows``: K and V are buffers of ``kv_rows`` rows (at the
+    least; ``kv_interleaved``) of which the ``kv_len`` from row ``*kv_first`` on are the keys."""
     seq_len = seq if seq_len is None else seq_len
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     _numel(_dev(Q, "Q"), seq * heads * d, "Q")
     _numel(_dev(O, "O"), seq * heads * d, "O")
+    if kv_first is not None:
+        _window(K, V, kv_rows, kv_len, kv_heads, d, kv_interleaved)
+        check(
+            lib().iron_mha_prefill_at_bf16(
+                ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, seq, seq_len, kv_len, float(scale),
+                int(causal), -1 if window is None else int(window), int(q_interleaved),
+                ptr(_word(valid, "valid")), ptr(_word(kv_valid, "kv_valid")), ptr(_word(kv_first, "kv_first")),
+                int(kv_rows), current_stream(),
+            ),
+            "iron_mha_prefill_at_bf16",
+        )
+        return
     _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
     _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
     check(
@@ -282,6 +296,15 @@ def mha_prefill(
     )
 
 
+def _window(K, V, kv_rows, kv_len, kv_heads, d, kv_interleaved):
+    if not kv_interleaved or kv_rows is None or kv_rows < kv_len:
+        raise ValueError(f"a window of the keys takes them row by row (kv_interleaved) out of kv_rows ({kv_rows}) "
+                         f">= kv_len ({kv_len})")
+    for name, t in (("K", K), ("V", V)):
+        if _dev(t, name).numel() < kv_rows * kv_heads * d:
+            raise ValueError(f"{name}: expected {kv_rows * kv_heads * d} elements at the least, got {t.numel()}")
+
+
 def mha_decode_workspace(heads, d, device="cuda"):
     n = lib().iron_mha_decode_workspace_bytes(heads, d)
     return torch.empty(n // 4, dtype=torch.float32, device=device)
@@ -289,17 +312,29 @@ def mha_decode_workspace(heads, d, device="cuda"):
 
 def mha_decode(
     Q, K, V, O, *, heads, kv_heads, d, kv_len, scale=None, window=None, kv_interleaved=False,
-    kv_valid=None, workspace,
+    kv_valid=None, workspace, kv_first=None, kv_rows=None,
 ):
+    """``kv_first`` / ``kv_rows``: the keys are a window of a longer buffer, as ``mha_prefill``'s."""
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     _numel(_dev(Q, "Q"), heads * d, "Q")
     _numel(_dev(O, "O"), heads * d, "O")
-    _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
-    _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
     _dev(workspace, "workspace", torch.float32)
     need = lib().iron_mha_decode_workspace_bytes(heads, d)
     if workspace.numel() * 4 < need:
         raise ValueError(f"workspace: {workspace.numel() * 4} bytes, need {need}")
+    if kv_first is not None:
+        _window(K, V, kv_rows, kv_len, kv_heads, d, kv_interleaved)
+        check(
+            lib().iron_mha_decode_at_bf16(
+                ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, kv_len, float(scale),
+                -1 if window is None else int(window), ptr(_word(kv_valid, "kv_valid")),
+                ptr(_word(kv_first, "kv_first")), int(kv_rows), ptr(workspace), current_stream(),
+            ),
+            "iron_mha_decode_at_bf16",
+        )
+        return
+    _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
+    _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
     check(
         lib().iron_mha_decode_bf16(
             ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, kv_len, float(scale),

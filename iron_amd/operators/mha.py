@@ -145,6 +145,10 @@ class MHA(Operator):
             bound["kv_valid"] = k.valid[0]
         return bound
 
+    def takes_view(self, name: str) -> bool:
+        """K and V may be a window of a longer buffer whose first row a call names (a ring cache's)."""
+        return name in ("K", "V") and self.kv_interleaved
+
     def output_valid(self, name, inputs):
         q = inputs.get("Q")
         return {0: q.valid[0]} if name == "O" and q is not None and 0 in q.valid else {}
@@ -179,7 +183,7 @@ class MHA(Operator):
                         ws = own["ws"] = kernels.mha_decode_workspace(H, d, t["Q"].device)
                 kernels.mha_decode(t["Q"], t["K"], t["V"], t["O"], heads=H, kv_heads=G, d=d, kv_len=L,
                                    scale=scale, window=window, kv_interleaved=kvi,
-                                   kv_valid=words.get("kv_valid"), workspace=ws)
+                                   kv_valid=words.get("kv_valid"), workspace=ws, **_key_window(words, G * d))
 
             return Built("iron_mha_decode_bf16", launch)
         seq, seq_len, causal = self.seq_pad, self.seq_len, self.causal
@@ -189,6 +193,22 @@ class MHA(Operator):
             kernels.mha_prefill(t["Q"], t["K"], t["V"], t["O"], heads=H, kv_heads=G, d=d, seq=seq,
                                 seq_len=seq_len, kv_len=L, scale=scale, causal=causal, window=window,
                                 q_interleaved=qi, kv_interleaved=kvi, valid=words.get("valid"),
-                                kv_valid=words.get("kv_valid"))
+                                kv_valid=words.get("kv_valid"), **_key_window(words, G * d))
 
         return Built("iron_mha_prefill_bf16", launch)
+
+
+def _key_window(words, row: int) -> dict:
+    """The launch's ``kv_first`` / ``kv_rows`` where K and V are windows of a longer buffer: both from
+    the same first row, a row of the buffer ``row`` elements."""
+    views = words.get("__views__") or {}
+    k, v = views.get("K"), views.get("V")
+    if k is None and v is None:
+        return {}
+    if k is None or v is None or k["index"] is None or v["index"] is None or k["ids"] is not None or v["ids"] is not None:
+        if all(x is None or (x["index"] is None and x["ids"] is None) for x in (k, v)):
+            return {}   # bounded only
+        raise ValueError("MHA: K and V are windows of their buffers from the same row, or neither is")
+    if k["index"].data_ptr() != v["index"].data_ptr() or k["rows"] != v["rows"] or k["stride"] != row or v["stride"] != row:
+        raise ValueError("MHA: K's and V's windows start at the same row of buffers alike")
+    return dict(kv_first=k["index"], kv_rows=k["rows"])

@@ -450,6 +450,52 @@ def test_mha_prefill_d256_ragged_windowed_and_bounded(cuda):
     close(got[:rows], want[:rows])
 
 
+@pytest.mark.parametrize("d,H,G", [(64, 8, 2), (128, 4, 1), (256, 4, 1), (512, 4, 1)])
+def test_mha_over_a_window_of_a_longer_buffer(cuda, d, H, G):
+    """Keys that are a run of rows of a longer buffer, from a row a device word names (a ring cache's
+    window): the launch that is handed those rows as tensors of their own, bit for bit; the buffer's
+    other rows (NaN here) reach nothing, and a word past the end is held inside the buffer."""
+    rng = np.random.default_rng(23)
+    rows, L, S = 300, 96, 64
+    Kb, Vb = bf(rng, rows, G, d) * 0.25, bf(rng, rows, G, d)
+    Q = bf(rng, S, H, d) * 0.25
+    ws = K.mha_decode_workspace(H, d, cuda)
+    for first, kv_valid in ((0, 96), (37, 80), (204, 96), (1000, 70)):
+        held = max(0, min(first, rows - L))
+        Kw, Vw = Kb[held : held + L].copy(), Vb[held : held + L].copy()
+        Kp, Vp = np.full_like(Kb, np.nan), np.full_like(Vb, np.nan)
+        Kp[held : held + kv_valid], Vp[held : held + kv_valid] = Kb[held : held + kv_valid], Vb[held : held + kv_valid]
+        for window in (None, 20):
+            own = out_like((S, H, d), cuda)
+            K.mha_prefill(dev(Q, cuda), dev(Kw, cuda), dev(Vw, cuda), own, heads=H, kv_heads=G, d=d, seq=S, kv_len=L,
+                          scale=1.0, window=window, q_interleaved=True, kv_interleaved=True, kv_valid=word(kv_valid, cuda))
+            at = out_like((S, H, d), cuda, fill=float("nan"))
+            K.mha_prefill(dev(Q, cuda), dev(Kp, cuda), dev(Vp, cuda), at, heads=H, kv_heads=G, d=d, seq=S, kv_len=L,
+                          scale=1.0, window=window, q_interleaved=True, kv_interleaved=True, kv_valid=word(kv_valid, cuda),
+                          kv_first=word(first, cuda), kv_rows=rows)
+            assert torch.equal(own, at), (first, kv_valid, window)
+            own1, at1 = out_like((1, H, d), cuda), out_like((1, H, d), cuda, fill=float("nan"))
+            K.mha_decode(dev(Q[:1], cuda), dev(Kw, cuda), dev(Vw, cuda), own1, heads=H, kv_heads=G, d=d, kv_len=L, scale=1.0,
+                         window=window, kv_interleaved=True, kv_valid=word(kv_valid, cuda), workspace=ws)
+            K.mha_decode(dev(Q[:1], cuda), dev(Kp, cuda), dev(Vp, cuda), at1, heads=H, kv_heads=G, d=d, kv_len=L, scale=1.0,
+                         window=window, kv_interleaved=True, kv_valid=word(kv_valid, cuda), workspace=ws,
+                         kv_first=word(first, cuda), kv_rows=rows)
+            assert torch.equal(own1, at1), (first, kv_valid, window)
+    # ... and the long-cache kernel (splits and their merge) over a window.
+    if d == 64:
+        rows, L = 6000, 4096
+        Kb, Vb, q = bf(rng, rows, G, d), bf(rng, rows, G, d), bf(rng, 1, H, d)
+        own1, at1 = out_like((1, H, d), cuda), out_like((1, H, d), cuda)
+        K.mha_decode(q_t := dev(q, cuda), dev(Kb[1500:5596], cuda), dev(Vb[1500:5596], cuda), own1, heads=H, kv_heads=G, d=d,
+                     kv_len=L, kv_interleaved=True, kv_valid=word(3000, cuda), workspace=ws)
+        K.mha_decode(q_t, dev(Kb, cuda), dev(Vb, cuda), at1, heads=H, kv_heads=G, d=d, kv_len=L, kv_interleaved=True,
+                     kv_valid=word(3000, cuda), workspace=ws, kv_first=word(1500, cuda), kv_rows=rows)
+        assert torch.equal(own1, at1)
+    with pytest.raises(ValueError, match="row by row"):
+        K.mha_decode(dev(Q[:1], cuda), dev(Kb, cuda), dev(Vb, cuda), out_like((1, H, d), cuda), heads=H, kv_heads=G, d=d,
+                     kv_len=96, kv_interleaved=False, workspace=ws, kv_first=word(0, cuda), kv_rows=300)
+
+
 def test_mha_512_wide_heads_prefill_and_decode(cuda):
     """512-wide heads (a global layer's of Gemma 4): the row-wise prompt kernel under every mask and
     a bound, and the one-query kernel on either side of 2048 keys."""
