@@ -176,3 +176,42 @@ def test_a_number_meets_a_handle_as_a_constant_row():
     assert names(t) == ["RowwiseMul", "RowwiseMul", "ElementwiseAdd", "RowwiseMul"]
     rows = [s.inputs["row"].buffer.source for s in t.steps if type(s.op).__name__ == "RowwiseMul"]
     assert rows[0] is rows[1] is rows[2] and np.all(np.asarray(rows[0].array) == 0.5)
+
+
+def test_a_profile_in_the_reference_s_format_fills_the_open_tunables_of_recorded_steps(tmp_path):
+    """``profiles/<device>.json`` as the reference writes it: entries by operator name, the most
+    specific match wins, an unknown operator or field is refused; the tunables are AIE tile counts
+    that the steps carry (iron/common/declare/profile.py:26-158)."""
+    import iron_amd
+    from iron_amd.operators.gemv import GEMV
+
+    E, Q = SCALED.hidden_size, SCALED.num_attention_heads * SCALED.head_dim   # o_proj is (E, Q)
+    file = tmp_path / "npu2.json"
+    file.write_text('{"entries": [\n'
+                    '  {"operator": "GEMV", "tile_size_input": 4},\n'
+                    f'  {{"operator": "GEMV", "M": {E}, "K": {Q}, "tile_size_input": 2, "num_aie_columns": 8}},\n'
+                    '  {"operator": "RMSNorm", "weighted": true, "rows": 1, "num_aie_columns": 1}\n]}\n')
+    profile = iron_amd.Profile.load(file)
+    assert len(profile) == 3
+    assert profile.tunables_for(GEMV, dict(M=E, K=Q)) == {"tile_size_input": 2, "num_aie_columns": 8}
+    assert profile.tunables_for(GEMV, dict(M=64, K=E)) == {"tile_size_input": 4}
+    assert profile.make(GEMV, M=E, K=Q, tile_size_input=1).tile_size_input == 1   # what a call gives stays
+    model = small()
+    model.profile = profile
+    t = model.record()
+    square = [s.op for s in t.steps if type(s.op).__name__ == "GEMV" and (s.op.M, s.op.K) == (E, Q)]
+    assert square and all(op.tile_size_input == 2 and op.num_aie_columns == 8 for op in square)
+    assert all(s.op.num_aie_columns == 1 for s in t.steps if type(s.op).__name__ == "RMSNorm" and s.op.weighted)
+    again = tmp_path / "again.json"
+    profile.save(again)
+    assert iron_amd.Profile.load(again).tunables_for(GEMV, dict(M=E, K=Q)) == profile.tunables_for(GEMV, dict(M=E, K=Q))
+    file.write_text('{"entries": [{"operator": "Conv2D", "tile": 4}]}')
+    with pytest.raises(ValueError, match="no operator 'Conv2D'"):
+        iron_amd.Profile.load(file)
+    with pytest.raises(TypeError, match="declares no field"):
+        profile.add(GEMV, tile_rows=4)
+    both = iron_amd.Profile()
+    both.add(GEMV, M=E, tile_size_input=2)
+    both.add(GEMV, K=Q, tile_size_input=4)
+    with pytest.raises(ValueError, match="ambiguous"):
+        both.tunables_for(GEMV, dict(M=E, K=Q))
