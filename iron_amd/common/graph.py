@@ -1328,9 +1328,25 @@ class CompiledGraph:
         self.arena.view(off, resident.shape, resident.dtype).copy_(_host_tensor(np.asarray(array), resident.dtype))
 
     def read(self, resident: Resident) -> np.ndarray:
+        """A state or weight as the device left it: a host copy, which ``push`` sends back."""
         self.load()
         off = self.arena.resident_offsets[id(resident)]
-        return from_torch(self.arena.view(off, resident.shape, resident.dtype))
+        array = from_torch(self.arena.view(off, resident.shape, resident.dtype))
+        vars(self).setdefault("_read", {})[id(resident)] = array
+        return array
+
+    def push(self, resident: Resident) -> None:
+        """Send to the device what the host wrote into the array ``read(resident)`` last returned
+        (iron/common/graph/compiled.py:850-854: there the array is the buffer's own host memory)."""
+        array = vars(self).get("_read", {}).get(id(resident))
+        if array is None:
+            raise ValueError("push() sends what read() returned: read the tensor first")
+        self.write(resident, array)
+
+    def upload(self, release=None, piece_bytes=None) -> None:
+        """Copy every weight the versions hold into the arena, once an arena (``load`` does it too;
+        the reference's keywords pace its host copies and mean nothing here)."""
+        self.arena.load()
 
     def __call__(self, *tensors, **values):
         """Run the version: inputs are host arrays (or device tensors), values per-call ints.

@@ -117,6 +117,26 @@ def test_sampled_tokens_are_the_host_s_token_for_token(toy):
     assert greedy == generate_on_host(toy, prompt, 24, Sampler(0.0)) and greedy != drawn
 
 
+def test_states_are_read_written_and_pushed(toy):
+    """``read`` a state as the device left it, ``push`` what the host wrote into that array,
+    ``write`` another (iron/common/graph/compiled.py:840-854); both versions see one arena."""
+    prompt = np.random.default_rng(21).integers(0, SCALED.vocab_size, 9)
+    toy.logits(prompt)
+    decode, chunk, keys = toy.decode_step, toy.prompt_chunk, toy.layers[1].cache.keys
+    saved = decode.read(keys).copy()
+    assert saved.shape == keys.shape and np.abs(saved[: len(prompt)]).max() > 0
+    held = decode.read(keys)
+    held[3] = 0.5
+    decode.push(keys)
+    assert np.array_equal(chunk.read(keys), held) and not np.array_equal(held, saved)
+    chunk.write(keys, saved)
+    assert np.array_equal(decode.read(keys), saved)
+    with pytest.raises(ValueError, match="read the tensor first"):
+        chunk.push(toy.layers[0].cache.values)
+    decode.upload()
+    toy.session.forget(0)
+
+
 def test_check_mode_judges_every_step_against_its_reference(cuda):
     model = Llama(SCALED, weights())
     model.load_versions(check=True)
