@@ -11,7 +11,7 @@ __version__ = "0.1.0"
 
 
 _LAZY = dict.fromkeys(
-    ["Carried", "CompiledGraph", "Graph", "Scratchpad", "carry", "clamp", "param", "state", "weight"],
+    ["Carried", "CarriedLoop", "CompiledGraph", "Graph", "Scratchpad", "carry", "clamp", "param", "state", "weight"],
     "iron_amd.common.graph",
 ) | dict.fromkeys(["Precision"], "iron_amd.common.declare") | dict.fromkeys(["Profile"], "iron_amd.common.profile")
 

@@ -9,6 +9,7 @@ The subset of the reference's graph layer the Llama decoder records
   per-call bound (``x[:n]``), a per-call row index (``x[p]``), a fixed-width window
   from a per-call start (``x[s:s+W]``), gather by ids (``table[ids]``), ``x[key] = v``
   (records a ``Copy``) and ``+`` / ``*`` (Elementwise steps).
+* ``CarriedLoop``: a version's carried values looped on the device (HIP-graph replays).
 * ``Affine``: per-call integer expressions of one value (``position + 1``,
   ``rows * 32``, clamp, ``>> k``), each a word of the device scratchpad.
 * ``CompiledGraph``: every version of a graph shares ONE device arena: residents
@@ -1458,3 +1459,57 @@ class CompiledGraph:
         self._graph = None
         self._launches = []
         self._loaded_generation = None
+
+
+class CarriedLoop:
+    """A graph's carried values looped on the device (iron/common/graph/carried.py:189-276).
+
+    ``first`` runs once from the host (a prompt chunk, or ``body`` itself); ``body`` -- a version
+    that takes no tensor, captured in a HIP graph -- then runs as replays, each starting from the
+    values the last run carried on the device, so the host only launches.  ``depth`` is the
+    reference's count of runs in flight; a stream orders the replays here and it changes nothing.
+
+    Raises:
+        ValueError: ``first`` and ``body`` are not versions of one graph (one arena), ``body`` takes
+            a tensor or carries nothing, or ``depth`` is under 1.
+    """
+
+    def __init__(self, first: CompiledGraph, body: CompiledGraph, depth: int = 2):
+        if first.arena is not body.arena:
+            raise ValueError("first and body are versions of one graph")
+        if body.recording.inputs:
+            raise ValueError(f"{body.recording.name}: the looped version takes no tensor, got "
+                             f"{[h.buffer.name for h in body.recording.inputs]}")
+        for version in (first, body):
+            if not version.recording.carry:
+                raise ValueError(f"{version.recording.name}: a version with carried values loops; this one carries none")
+        if depth < 1:
+            raise ValueError(f"depth is at least 1, got {depth}")
+        self.first, self.body, self.depth = first, body, depth
+        self._started = False
+
+    def run(self, steps: int, /, *tensors, **values):
+        """``start`` now, then ``steps``, each index yielded once launched."""
+        self.start(*tensors, **values)
+        return self.steps(steps)
+
+    def start(self, *tensors, **values) -> None:
+        """Run ``first`` on ``tensors`` and ``values``; what it carries is where ``body`` starts."""
+        self.body.load()
+        if not self.body.captured:
+            raise RuntimeError(f"{self.body.recording.name}: the looped version is captured in a HIP graph (capture=True)")
+        *_, carry = self.first(*tensors, **values)
+        self._carry, self._started = dict(carry), True
+
+    def steps(self, steps: int):
+        """Run ``steps`` steps of ``body``, yielding each index once its replay is launched; what the
+        steps wrote is read (``body.read``) after the last, which waits for them."""
+        if not self._started:
+            raise RuntimeError("start() runs the first version before the steps")
+        for k in range(steps):
+            if self._carry is not None:
+                self.body.start(**self._carry)   # the first step takes first's carried values from the host
+                self._carry = None
+            else:
+                self.body.replay(1)
+            yield k

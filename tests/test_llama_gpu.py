@@ -117,6 +117,31 @@ def test_sampled_tokens_are_the_host_s_token_for_token(toy):
     assert greedy == generate_on_host(toy, prompt, 24, Sampler(0.0)) and greedy != drawn
 
 
+def test_a_carried_loop_runs_the_decode_steps_on_the_device(toy):
+    """``CarriedLoop(first, body)``: the prompt chunk from the host, then the decode step replayed
+    from what each run carried (iron/common/graph/carried.py:189-276); the tokens are generate()'s."""
+    import iron_amd
+
+    prompt = np.random.default_rng(8).integers(0, SCALED.vocab_size, 40)
+    want = toy.generate(prompt, 24)
+    toy.session.forget(0)
+    ((ids,), values), = toy.session._chunks(prompt, 0)
+    loop = iron_amd.CarriedLoop(toy.prompt_chunk, toy.decode_step)
+    assert list(loop.run(23, ids, **values)) == list(range(23))
+    record = toy.decode_step.read(toy.drawn)
+    assert [int(t) for t in record[len(prompt) - 1 : len(prompt) + 23]] == want
+    # The decode step started from the host is a first version too.
+    again = iron_amd.CarriedLoop(toy.decode_step, toy.decode_step)
+    again.start(token=want[0], position=len(prompt))
+    assert len(list(again.steps(5))) == 5
+    assert [int(t) for t in toy.decode_step.read(toy.drawn)[len(prompt) : len(prompt) + 6]] == want[1:7]
+    with pytest.raises(ValueError, match="takes no tensor"):
+        iron_amd.CarriedLoop(toy.decode_step, toy.prompt_chunk)
+    with pytest.raises(RuntimeError, match="start"):
+        next(iron_amd.CarriedLoop(toy.prompt_chunk, toy.decode_step).steps(1))
+    toy.session.forget(0)
+
+
 def test_states_are_read_written_and_pushed(toy):
     """``read`` a state as the device left it, ``push`` what the host wrote into that array,
     ``write`` another (iron/common/graph/compiled.py:840-854); both versions see one arena."""
