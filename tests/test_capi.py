@@ -38,3 +38,14 @@ def test_argument_refusals_need_no_gpu():
     assert b"multiple of 8" in lib.iron_last_error()
     assert lib.iron_mha_prefill_bf16(one, one, one, one, 6, 4, 64, 8, 8, 8, 0.125, 1, -1, 0, 0, None, None, None) == 1
     assert b"multiple of kv_heads" in lib.iron_last_error()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """``bench.py --gpus N`` with N above 1 exits with a message: this build is the one-GPU path."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = Path(__file__).resolve().parent.parent / "bench.py"
+    done = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert done.returncode != 0 and "one-GPU" in done.stderr and done.stdout.strip() == ""
