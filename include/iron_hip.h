@@ -61,7 +61,8 @@ int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t
  *   y = E(W @ N(x)):  N = RMSNorm(x, eps) * norm_w when norm_w is not NULL (else x itself);
  *   epilogue 0: y = bf16(W N(x));  1: y = bf16(residual_scale * bf16(W N(x)) + residual), one fused
  *   multiply-add (a scale of 1 is the plain sum; another is AXPY's, iron/lm/blocks.py:386-391);
- *   2: y = bf16(bf16(silu(bf16(W N(x)))) * bf16(W2 N(x)))   (gate, up -> SiLU -> Mul).
+ *   2: y = bf16(bf16(silu(bf16(W N(x)))) * bf16(W2 N(x)))   (gate, up -> SiLU -> Mul);
+ *   3: the same with GELU by its tanh form for SiLU (Gemma's feed-forward).
  * W, W2 (M,K); x, norm_w (K); residual, y (M).  K % 8 == 0. */
 int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const uint16_t* x,
                          const uint16_t* norm_w, float eps, const uint16_t* residual,

@@ -148,7 +148,8 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                     got = Fused("decode_qkv", i, 8, lambda a=args, kw=kw: kernels.decode_qkv(**a, **kw))
             # the gated MLP's first half
             if (got is None and len(rest) >= 4 and gemv_row(rest[0], n) and gemv_row(rest[1], n) and once(n, 2)
-                    and _name(rest[2]) == "SiLU" and _name(rest[3]) == "ElementwiseMul"):
+                    and (_name(rest[2]) == "SiLU" or (_name(rest[2]) == "GELU" and rest[2].op.approximate == "tanh"))
+                    and _name(rest[3]) == "ElementwiseMul"):
                 gg, gu, si, mu = rest[:4]
                 g, u = gg.outputs["C"], gu.outputs["C"]
                 ok = (_same(si.inputs["x"], g) and once(g) and once(u) and once(si.outputs["y"])
@@ -159,8 +160,8 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                     args = dict(W=tensor(gg.inputs["A"]), W2=tensor(gu.inputs["A"]),
                                 x=tensor(s.inputs["x"]).reshape(-1), norm_w=tensor(s.inputs["weight"]).reshape(-1),
                                 y=tensor(mu.outputs["y"]).reshape(-1))
-                    kw = dict(M=gg.op.M, K=gg.op.K, eps=float(s.op.epsilon), epilogue=2)
-                    got = Fused("norm_gate_up_silu_mul", i, 5, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+                    kw = dict(M=gg.op.M, K=gg.op.K, eps=float(s.op.epsilon), epilogue=2 if _name(si) == "SiLU" else 3)
+                    got = Fused("norm_gate_up_silu_mul" if _name(si) == "SiLU" else "norm_gate_up_gelu_mul", i, 5, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
             # the head: norm, then one projection
             if got is None and rest and gemv_row(rest[0], n) and once(n, 1):
                 g0 = rest[0]

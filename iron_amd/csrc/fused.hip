@@ -12,6 +12,11 @@
 namespace iron {
 
 __device__ __forceinline__ float silu_ref(float v) { return v / (1.0f + __expf(-v)); }
+// GELU by its tanh form, as the catalog's unary kernel computes it.
+__device__ __forceinline__ float gelu_tanh_ref(float v) {
+  const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+  return 0.5f * v * (1.0f + tanhf(inner));
+}
 
 // All fused kernels share one shape: a block of 4 waves owns a few rows and its 256 threads
 // split K in 16-byte chunks (thread t takes chunks t, t+256, ...), so the weight loads of a row
@@ -90,7 +95,7 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[CH], const float (&xf)
   return acc;
 }
 
-enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2 };
+enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2, EPI_GELU_MUL = 3 };   // 2 and 3: gate, up -> activation -> Mul
 
 // y = E(W @ N(x)) for RPW rows a block; K <= CH * 2048.
 template <int RPW, int CH, bool NORM, int EPI>
@@ -101,7 +106,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
                                                          const bf16_t* __restrict__ res,
                                                          float res_scale, bf16_t* __restrict__ y,
                                                          int M, int K) {
-  constexpr int MATS = EPI == EPI_SILU_MUL ? 2 : 1;
+  constexpr int MATS = (EPI == EPI_SILU_MUL || EPI == EPI_GELU_MUL) ? 2 : 1;
   __shared__ float scratch4[4];
   __shared__ float part[4][MATS][RPW];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -134,10 +139,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
     if (row < M) {
       float v = round_bf16(part[0][0][r] + part[1][0][r] + part[2][0][r] + part[3][0][r]);  // the GEMV's own rounding
       if (EPI == EPI_ADD) v = fmaf(res_scale, v, res_ahead);   // scale 1: the plain sum
-      if (EPI == EPI_SILU_MUL) {
+      if (EPI == EPI_SILU_MUL || EPI == EPI_GELU_MUL) {
         const float u = round_bf16(part[0][MATS - 1][r] + part[1][MATS - 1][r] + part[2][MATS - 1][r] +
                                    part[3][MATS - 1][r]);
-        v = round_bf16(silu_ref(v)) * u;
+        v = round_bf16(EPI == EPI_SILU_MUL ? silu_ref(v) : gelu_tanh_ref(v)) * u;
       }
       y[row] = f32_to_bf16(v);
     }
@@ -211,9 +216,9 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
                                     void* stream) {
   IRON_REQUIRE(W && x && y, "gemv_fused: null operand");
   IRON_REQUIRE(M > 0 && K > 0 && K % 8 == 0, "gemv_fused: M (%d) positive, K (%d) a positive multiple of 8", M, K);
-  IRON_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemv_fused: epilogue (%d) is 0, 1 or 2", epilogue);
+  IRON_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemv_fused: epilogue (%d) is 0, 1, 2 or 3", epilogue);
   IRON_REQUIRE(epilogue != EPI_ADD || residual, "gemv_fused: epilogue 1 adds a residual; none given");
-  IRON_REQUIRE(epilogue != EPI_SILU_MUL || W2, "gemv_fused: epilogue 2 takes a second matrix; none given");
+  IRON_REQUIRE((epilogue != EPI_SILU_MUL && epilogue != EPI_GELU_MUL) || W2, "gemv_fused: epilogues 2 and 3 take a second matrix; none given");
   IRON_REQUIRE((((uintptr_t)W | (uintptr_t)W2 | (uintptr_t)x | (uintptr_t)norm_w) & 15) == 0,
                "gemv_fused: operands must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
@@ -221,7 +226,7 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   IRON_REQUIRE(K <= 8 * 2048, "gemv_fused: K (%d) exceeds %d", K, 8 * 2048);
   const int ch = K <= 2048 ? 1 : (K <= 4096 ? 2 : (K <= 8192 ? 4 : 8));
   // Rows a block takes: two where the matrix is tall and a row is short, else one.
-  const int rpw = (epilogue == EPI_SILU_MUL) ? (ch == 1 ? 2 : 1) : (ch == 1 && M > 2048 ? (M >= 65536 ? 4 : 2) : 1);
+  const int rpw = (epilogue == EPI_SILU_MUL || epilogue == EPI_GELU_MUL) ? (ch == 1 ? 2 : 1) : (ch == 1 && M > 2048 ? (M >= 65536 ? 4 : 2) : 1);
   const int blocks = (M + rpw - 1) / rpw;
 #define IRON_FUSED(R, C, NRM, E)                                                                   \
   if (rpw == R && ch == C && norm == NRM && epilogue == E) {                                       \
@@ -234,6 +239,8 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   IRON_FUSED_NE(1, 1) IRON_FUSED_NE(2, 1) IRON_FUSED_NE(4, 1) IRON_FUSED_NE(1, 2) IRON_FUSED_NE(1, 4) IRON_FUSED_NE(1, 8)
   IRON_FUSED(2, 1, false, 2) IRON_FUSED(2, 1, true, 2) IRON_FUSED(1, 2, false, 2) IRON_FUSED(1, 2, true, 2)
   IRON_FUSED(1, 4, false, 2) IRON_FUSED(1, 4, true, 2) IRON_FUSED(1, 8, false, 2) IRON_FUSED(1, 8, true, 2)
+  IRON_FUSED(2, 1, false, 3) IRON_FUSED(2, 1, true, 3) IRON_FUSED(1, 2, false, 3) IRON_FUSED(1, 2, true, 3)
+  IRON_FUSED(1, 4, false, 3) IRON_FUSED(1, 4, true, 3) IRON_FUSED(1, 8, false, 3) IRON_FUSED(1, 8, true, 3)
 #undef IRON_FUSED_NE
 #undef IRON_FUSED
   IRON_REQUIRE(false, "gemv_fused: no kernel for this combination");

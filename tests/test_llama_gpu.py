@@ -321,6 +321,9 @@ def test_fused_kernels_against_the_oracle_at_llama_1b_width(cuda):
     K.gemv_fused(dev(Wg), dev(x), m, M=F, K=E, W2=dev(Wu), norm_w=dev(g), eps=1e-5, epilogue=2)
     want_m = ops.mul(ops.silu(ops.gemv(Wg, n)), ops.gemv(Wu, n))
     close(m, want_m)
+    # ... gated by GELU (its tanh form) as Gemma's feed-forward is
+    K.gemv_fused(dev(Wg), dev(x), m, M=F, K=E, W2=dev(Wu), norm_w=dev(g), eps=1e-5, epilogue=3)
+    close(m, ops.mul(ops.gelu(ops.gemv(Wg, n)), ops.gemv(Wu, n)))
     y = torch.empty(E, dtype=torch.bfloat16, device=cuda)
     K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, residual=dev(x), epilogue=1)
     close(y, ops.add(x, ops.gemv(Wd, want_m)))
