@@ -105,6 +105,11 @@ int iron_prefill_qkv_cache_bf16(const uint16_t* x, const uint16_t* Wq, const uin
  * iron/common/elementwise.py:619-682. */
 int iron_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int rows, int cols,
                       float eps, const int* valid, void* stream);
+/* y = bf16(residual + the row above): a block's output normed again before its residual, the
+ * sandwich layer's RMSNorm and ElementwiseAdd in one pass (iron/lm/blocks.py:748-767), rounding
+ * where the two steps round.  residual (rows, cols); y may be residual. */
+int iron_rmsnorm_add_bf16(const uint16_t* x, const uint16_t* w, const uint16_t* residual, uint16_t* y,
+                          int rows, int cols, float eps, const int* valid, void* stream);
 
 /* Rotary embedding of x (rows, cols) by the packed table angles (angle_rows, cols), cos and
  * sin interleaved; row r uses angle row r / (rows / angle_rows).  two_halves: rotate the two

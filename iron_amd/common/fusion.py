@@ -16,6 +16,7 @@ and, in a prompt chunk's version (several rows, 64-wide heads),
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
   SiLU, ElementwiseMul (the gated feed-forward)          => iron_silu_mul_bf16
   GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
+  RMSNorm, ElementwiseAdd (a sandwich layer's residual)  => iron_rmsnorm_add_bf16
 
 A run is fused only if every intermediate it hides is read by nothing else.
 """
@@ -272,6 +273,26 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                             residual=tensor(other).reshape(-1), y=tensor(ad.outputs["y"]).reshape(-1))
                 kw = dict(M=s.op.M, K=s.op.K, epilogue=1, residual_scale=scale)
                 got = Fused("gemv_add", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+        if (got is None and _name(s) == "RMSNorm" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseAdd"
+                and set(s.values) <= {"valid"}):
+            # a block's output normed again before its residual (a sandwich layer): the sum rides the norm's pass
+            ad = steps[i + 1]
+            n = s.outputs["y"]
+            a, b = ad.inputs["a"], ad.inputs["b"]
+            other = a if _same_view(b, n) else (b if _same_view(a, n) else None)
+            nv, av = s.values.get("valid"), ad.values.get("valid")
+            cols = s.op.tile_size
+            bounds_agree = (nv is None and av is None) or (
+                nv is not None and av is not None and nv.value == av.value and nv.linear and av.linear
+                and av.scale == nv.scale * cols and av.bias == nv.bias * cols)
+            flat = all(h.index is None and h.ids is None
+                       for h in (*s.inputs.values(), n, a, b, ad.outputs["y"]))
+            if (other is not None and flat and once(n) and bounds_agree and other.elements == n.elements
+                    and ad.outputs["y"].elements == n.elements and set(ad.values) <= {"valid"}):
+                args = dict(x=tensor(s.inputs["x"]), w=tensor(s.inputs["weight"]) if s.op.weighted else None,
+                            y=tensor(ad.outputs["y"]), residual=tensor(other))
+                kw = dict(rows=s.op.rows, cols=cols, eps=float(s.op.epsilon), valid=word(nv))
+                got = Fused("norm_add", i, 2, lambda a=args, kw=kw: kernels.rmsnorm(**a, **kw))
         if got is not None:
             fused.append(got)
             i += got.count

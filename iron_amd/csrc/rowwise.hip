@@ -13,13 +13,16 @@ template <int CHUNKS>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__ x,
                                                       const bf16_t* __restrict__ w,
                                                       bf16_t* __restrict__ y, int rows, int cols,
-                                                      float eps, const int* __restrict__ valid) {
+                                                      float eps, const int* __restrict__ valid,
+                                                      const bf16_t* residual) {
   const int row = blockIdx.x;
   if (row >= bound_or(valid, rows)) return;
   const int nchunk = cols >> 3;
   const uint4* xr = reinterpret_cast<const uint4*>(x + (size_t)row * cols);
   uint4* yr = reinterpret_cast<uint4*>(y + (size_t)row * cols);
   const uint4* wr = reinterpret_cast<const uint4*>(w);
+  // A residual (which y may be) the normed row is added to, rounded as the separate sum rounds.
+  const uint4* rr = reinterpret_cast<const uint4*>(residual + (residual ? (size_t)row * cols : 0));
 
   uint4 held[CHUNKS];
   float ss = 0.f;
@@ -59,6 +62,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[j] = f[j] * inv;
+    }
+    if (residual != nullptr) {
+      float r[8];
+      unpack8(rr[c], r);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = r[j] + round_bf16(f[j]);
     }
     yr[c] = pack8(f);
   };
@@ -215,21 +224,34 @@ __global__ __launch_bounds__(256) void row_broadcast_kernel(const bf16_t* __rest
 
 using namespace iron;
 
-extern "C" int iron_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int rows,
-                                 int cols, float eps, const int* valid, void* stream) {
+static int rmsnorm(const uint16_t* x, const uint16_t* w, const uint16_t* residual, uint16_t* y, int rows, int cols,
+                   float eps, const int* valid, void* stream) {
   IRON_REQUIRE(x && y, "rmsnorm: null operand");
+  IRON_REQUIRE(((uintptr_t)residual & 15) == 0, "rmsnorm: operands must be 16-byte aligned");
   IRON_REQUIRE(rows > 0 && cols > 0, "rmsnorm: rows (%d) and cols (%d) must be positive", rows, cols);
   IRON_REQUIRE(cols % 8 == 0, "rmsnorm: cols (%d) must be a multiple of 8", cols);
   IRON_REQUIRE((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) == 0,
                "rmsnorm: operands must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   if (cols <= 2048)
-    hipLaunchKernelGGL((rmsnorm_kernel<1>), dim3(rows), dim3(256), 0, s, x, w, y, rows, cols, eps, valid);
+    hipLaunchKernelGGL((rmsnorm_kernel<1>), dim3(rows), dim3(256), 0, s, x, w, y, rows, cols, eps, valid, residual);
   else if (cols <= 4096)
-    hipLaunchKernelGGL((rmsnorm_kernel<2>), dim3(rows), dim3(256), 0, s, x, w, y, rows, cols, eps, valid);
+    hipLaunchKernelGGL((rmsnorm_kernel<2>), dim3(rows), dim3(256), 0, s, x, w, y, rows, cols, eps, valid, residual);
   else
-    hipLaunchKernelGGL((rmsnorm_kernel<4>), dim3(rows), dim3(256), 0, s, x, w, y, rows, cols, eps, valid);
+    hipLaunchKernelGGL((rmsnorm_kernel<4>), dim3(rows), dim3(256), 0, s, x, w, y, rows, cols, eps, valid, residual);
   IRON_LAUNCH_CHECK();
+}
+
+extern "C" int iron_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* y, int rows,
+                                 int cols, float eps, const int* valid, void* stream) {
+  return rmsnorm(x, w, nullptr, y, rows, cols, eps, valid, stream);
+}
+
+extern "C" int iron_rmsnorm_add_bf16(const uint16_t* x, const uint16_t* w, const uint16_t* residual,
+                                     uint16_t* y, int rows, int cols, float eps, const int* valid,
+                                     void* stream) {
+  IRON_REQUIRE(residual, "rmsnorm_add: null residual");
+  return rmsnorm(x, w, residual, y, rows, cols, eps, valid, stream);
 }
 
 extern "C" int iron_rope_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows,

@@ -154,11 +154,20 @@ def prefill_qkv_cache(x, Wq, Wk, Wv, angles, q_out, keys, values, *, rows, hidde
     )
 
 
-def rmsnorm(x, w, y, *, rows, cols, eps, valid=None):
+def rmsnorm(x, w, y, *, rows, cols, eps, valid=None, residual=None):
+    """``residual``: the normed rows are added to it (the sum rounded as the separate step rounds)."""
     _numel(_dev(x, "x"), rows * cols, "x")
     _numel(_dev(y, "y"), rows * cols, "y")
     if w is not None:
         _numel(_dev(w, "weight"), cols, "weight")
+    if residual is not None:
+        _numel(_dev(residual, "residual"), rows * cols, "residual")
+        check(
+            lib().iron_rmsnorm_add_bf16(ptr(x), ptr(w), ptr(residual), ptr(y), rows, cols, float(eps),
+                                        ptr(_word(valid, "valid")), current_stream()),
+            "iron_rmsnorm_add_bf16",
+        )
+        return
     check(
         lib().iron_rmsnorm_bf16(
             ptr(x), ptr(w), ptr(y), rows, cols, float(eps), ptr(_word(valid, "valid")),

@@ -295,6 +295,28 @@ def test_rmsnorm_bound(cuda):
     assert np.all(got[5:] == 3.0)
 
 
+@pytest.mark.parametrize("rows,cols,weighted,bound", [(1, 2048, True, None), (64, 512, True, 40), (7, 8192, False, None)])
+def test_rmsnorm_with_its_residual(cuda, rows, cols, weighted, bound):
+    """The normed rows added to a residual in the norm's own pass: bit for bit the norm launch
+    followed by the sum (each rounds where the other does), in place too; rows past a bound keep theirs."""
+    rng = np.random.default_rng(9)
+    x, r = bf(rng, rows, cols), bf(rng, rows, cols)
+    w = dev(round_bf16(rng.uniform(0.9, 1.1, cols)), cuda) if weighted else None
+    valid = None if bound is None else word(bound, cuda)
+    lim = rows if bound is None else bound
+    normed, summed = out_like((rows, cols), cuda), out_like((rows, cols), cuda, fill=3.0)
+    K.rmsnorm(dev(x, cuda), w, normed, rows=rows, cols=cols, eps=1e-6)
+    K.add(dev(r, cuda).reshape(-1), normed.reshape(-1), summed.reshape(-1), n=rows * cols,
+          valid=None if bound is None else word(bound * cols, cuda))
+    once = out_like((rows, cols), cuda, fill=3.0)
+    K.rmsnorm(dev(x, cuda), w, once, rows=rows, cols=cols, eps=1e-6, valid=valid, residual=dev(r, cuda))
+    assert torch.equal(once, summed)
+    close(from_torch(once)[:lim], ops.add(r, ops.rms_norm(x, None if w is None else from_torch(w), epsilon=1e-6))[:lim])
+    stream = dev(r, cuda)
+    K.rmsnorm(dev(x, cuda), w, stream, rows=rows, cols=cols, eps=1e-6, valid=valid, residual=stream)
+    assert torch.equal(stream[:lim], summed[:lim]) and np.array_equal(from_torch(stream)[lim:], r[lim:])
+
+
 def angle_table(rng, angle_rows, cols):
     theta = rng.uniform(-np.pi, np.pi, (angle_rows, cols // 2))
     table = np.empty((angle_rows, cols), np.float32)
