@@ -92,7 +92,7 @@ int iron_prefill_qkv_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t*
 /* The same with k and v written straight into the chunk's rows of the layer's KV caches, rows
  * *start on of keys and values (cache_rows, kv_heads*d): replaces the two Copy steps that follow as
  * well (iron/lm/blocks.py:472-486).  The first row is held where the rows under the bound end inside
- * the cache; without a bound rows <= cache_rows. */
+ * the cache; rows <= cache_rows. */
 int iron_prefill_qkv_cache_bf16(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk,
                                 const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out,
                                 uint16_t* keys, uint16_t* values, int rows, int hidden, int heads,

@@ -214,7 +214,7 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                         and kd.index == vd.index and kd.index_rows == vd.index_rows
                         and kd.valid.get(0) == gvalid and vd.valid.get(0) == gvalid
                         and ck.inputs["src"].valid.get(0) == gvalid and cv.inputs["src"].valid.get(0) == gvalid
-                        and (gvalid is not None or M <= kd.index_rows)
+                        and M <= kd.index_rows
                     )
                     if cached:
                         args = {k_: t for k_, t in args.items() if k_ not in ("k_out", "v_out")}

@@ -1350,8 +1350,8 @@ extern "C" int iron_prefill_qkv_cache_bf16(const uint16_t* x, const uint16_t* Wq
                                            const int* valid, void* stream) {
   IRON_REQUIRE(start != nullptr, "prefill_qkv_cache: null start");
   IRON_REQUIRE(cache_rows > 0, "prefill_qkv_cache: cache_rows (%d) must be positive", cache_rows);
-  IRON_REQUIRE(valid != nullptr || rows <= cache_rows,
-               "prefill_qkv_cache: without a bound the chunk's %d rows must fit the cache's %d", rows, cache_rows);
+  // Whatever the bound word holds it is at most `rows`: the rows under it then fit the cache from some row on.
+  IRON_REQUIRE(rows <= cache_rows, "prefill_qkv_cache: the chunk's %d rows must fit the cache's %d", rows, cache_rows);
   return prefill_qkv(x, Wq, Wk, Wv, angles, q_out, keys, values, rows, hidden, heads, kv_heads, d, valid, start,
                      cache_rows, stream);
 }
