@@ -189,3 +189,17 @@ def test_the_gpu_matches_the_host_step_by_step_past_a_ring(cuda, global_head_dim
             assert np.abs(got - want).max() <= 0.03 * np.abs(want).max(), n
     finally:
         gpu.release()
+
+
+@pytest.mark.gpu
+def test_check_mode_judges_every_step_of_gemma_against_its_reference(cuda, w):
+    """Every recorded step launched on its own and judged against its operator's reference by the
+    operator's own tolerance: the per-head norms, GELU, the capped logits and the constant rows too."""
+    model = Gemma4(TOY, w)
+    model.load_versions(check=True)
+    try:
+        prompt = np.random.default_rng(9).integers(0, TOY.vocab_size, 70)   # two chunks
+        model.logits(prompt)
+        model.logits(np.append(prompt, 5))
+    finally:
+        model.release()
