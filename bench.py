@@ -270,6 +270,30 @@ def llama_weights(torch, config, dev, seed=0):
     return out
 
 
+def prompt_probe(torch, dev, repeats=20):
+    """Only the decoder's 512-token prompt chunk, ``repeats`` times: what a kernel trace of the time
+    to the first token needs (the bench's own run buries its one chunk under the micro-benchmarks)."""
+    import dataclasses
+
+    from iron_amd.applications.llama import LLAMA_3_2_1B, Llama
+
+    config = dataclasses.replace(LLAMA_3_2_1B, max_seq_len=2048, prefill_chunk=2048)
+    model = Llama(config, llama_weights(torch, config, dev))
+    model.load_versions()
+    prompt = np.random.default_rng(512).integers(0, config.vocab_size, 512)
+    times = []
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for inputs, values in model.session._chunks(prompt, 0):
+            model(*inputs, **values)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    print(json.dumps({"probe": "prompt", "prefill_tokens": 512, "repeats": repeats,
+                      "launches_per_chunk": model.prompt_chunk.launches_per_call,
+                      "ttft_ms_median": round(1e3 * float(np.median(times)), 3)}))
+
+
 def bench_decoder(torch, dev, steps, warmup, with_cpu):
     """Llama-3.2-1B shape: a 512-token prompt prefill, then ``steps`` greedy decode steps as
     replays of the captured decode step (each starts from the token and position the last one
@@ -422,6 +446,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--counter-probe", action="store_true",
                     help="launch only the LM-head GEMV, a plain copy of known size and the MFMA kernels (for a rocprofv3 --pmc run) and exit")
+    ap.add_argument("--prompt-probe", action="store_true",
+                    help="run only the decoder's 512-token prompt chunk, 20 times (for a rocprofv3 --kernel-trace run) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is a one-GPU hot path; --gpus must be 1 "
@@ -451,6 +477,9 @@ def main():
 
     if args.counter_probe:
         counter_probe(torch, K, dev, rng)
+        return 0
+    if args.prompt_probe:
+        prompt_probe(torch, dev)
         return 0
 
     t_wall = time.perf_counter()
