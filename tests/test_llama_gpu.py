@@ -142,6 +142,24 @@ def test_a_carried_loop_runs_the_decode_steps_on_the_device(toy):
     toy.session.forget(0)
 
 
+def test_accuracy_and_determinism_as_the_reference_accepts_a_model(toy):
+    """The reference's acceptance of a model on its device (iron/lm/testing.py:136-289): the KL of
+    each next-token distribution against the float32 reference's, teacher-forced on the reference's
+    greedy tokens, under its bounds (mean 0.02, p90 0.04, max 0.2), and logits bitwise the same run
+    after run over two alternating prompts."""
+    from iron_amd.lm.generation import accuracy, determinism, kl_stats
+
+    host = HostLlama(SCALED, weights())
+    host.load_versions()
+    prompt = np.random.default_rng(31).integers(0, SCALED.vocab_size, 24)
+    results = accuracy(toy, host, prompt, 10)
+    stats = kl_stats(results)
+    assert stats["Mean"] < 0.02 and stats["P90"] < 0.04 and stats["Max"] < 0.2, stats
+    assert sum(same for _, same in results) >= 9   # a near-tie of drawn weights may flip one
+    other = np.random.default_rng(32).integers(0, SCALED.vocab_size, 17)
+    assert determinism(toy, [prompt, other], 6, rounds=3) == 0
+
+
 def test_states_are_read_written_and_pushed(toy):
     """``read`` a state as the device left it, ``push`` what the host wrote into that array,
     ``write`` another (iron/common/graph/compiled.py:840-854); both versions see one arena."""
