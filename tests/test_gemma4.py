@@ -187,6 +187,10 @@ def test_the_gpu_matches_the_host_step_by_step_past_a_ring(cuda, global_head_dim
         for n in (150, 151, 152, 300):
             got, want = gpu.logits(tokens[:n]), cpu.logits(tokens[:n])
             assert np.abs(got - want).max() <= 0.03 * np.abs(want).max(), n
+        # Logits bitwise the same run after run, over rings that wrap and alternating prompts.
+        from iron_amd.lm.generation import determinism
+
+        assert determinism(gpu, [tokens[:150], tokens[40:200]], 3, rounds=2) == 0
     finally:
         gpu.release()
 
