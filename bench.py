@@ -347,7 +347,8 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu):
            "bytes_per_token": int(per_token), "GBps": round(per_token * tok_s / 1e9, 1),
            "frac_hbm": round(per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
            "steps_recorded": len(decode.recording.steps),
-           "launches_per_step": decode.launches_per_call, "first_tokens": [int(t) for t in tokens[:4]]}
+           "launches_per_step": decode.launches_per_call,
+           "launches_per_prompt_chunk": model.prompt_chunk.launches_per_call, "first_tokens": [int(t) for t in tokens[:4]]}
     cpu = None
     if with_cpu:
         cpu = cpu_decoder_baseline(torch, config, weights)
