@@ -1,4 +1,4 @@
-"""Step fusion for a one-row (decode) version of a graph.
+"""Step fusion for the versions of a graph.
 
 The recorded steps stay what the reference records -- one operator per step, which is
 what ``Graph.reference`` and check mode run.  When a version is loaded for the GPU, runs
@@ -8,14 +8,19 @@ round:
 
   RMSNorm, GEMV q/k/v, RoPE q/k, Copy k/v -> cache      => iron_decode_qkv_bf16
   RMSNorm, GEMV gate, GEMV up, SiLU, ElementwiseMul      => iron_gemv_fused_bf16 (epilogue 2)
-  GEMV, ElementwiseAdd (the residual)                    => iron_gemv_fused_bf16 (epilogue 1)
+  ... with GELU (tanh) for SiLU                          => iron_gemv_fused_bf16 (epilogue 3)
+  GEMV, ElementwiseAdd / AXPY (the residual)             => iron_gemv_fused_bf16 (epilogue 1)
   RMSNorm, GEMV (the head)                               => iron_gemv_fused_bf16 (epilogue 0)
 
-and, in a prompt chunk's version (several rows, 64-wide heads),
+in a prompt chunk's version (several rows, 64-wide heads),
 
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
+  ... and Copy k/v -> the chunk's cache rows             => iron_prefill_qkv_cache_bf16
   SiLU, ElementwiseMul (the gated feed-forward)          => iron_silu_mul_bf16
   GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
+
+and in either,
+
   RMSNorm, ElementwiseAdd (a sandwich layer's residual)  => iron_rmsnorm_add_bf16
 
 A run is fused only if every intermediate it hides is read by nothing else.
