@@ -1312,15 +1312,41 @@ class CompiledGraph:
             stream.synchronize()
         torch.cuda.current_stream().wait_stream(stream)
         self._graph = graph
+        self._host_values = None   # the warm-up's values start no run of replays
 
     # -- calling -------------------------------------------------------------
     def _write_words(self, full: Mapping[str, int]) -> None:
+        import torch
+
+        # The words travel from one pinned buffer by an asynchronous copy: the last call's copy may
+        # still be queued behind earlier work, and must have read the buffer before it is refilled.
+        copied = vars(self).get("_words_copied")
+        if copied is not None:
+            copied.synchronize()
+        self._host_values = {k: int(v) for k, v in full.items() if k != "__const__"}
         self.host_words.zero_()
         for name, slot in self.slots.items():
             self.host_words[slot] = int(full[name])
         for expr, slot in self.exprs.items():
             self.host_words[slot] = expr.evaluate(full)
         self.words.copy_(self.host_words, non_blocking=True)
+        self._words_copied = torch.cuda.Event()
+        self._words_copied.record()
+
+    def _after(self, values: Mapping[str, int], steps: int) -> dict[str, int]:
+        """The per-call values ``steps`` runs after ``values``, as far as the host can follow them:
+        what the body carries by a formula (``position + 1``); a value the device computes (the drawn
+        token) keeps its last known number."""
+        carry = self.recording.carry or {}
+        values = dict(values)
+        for _ in range(steps):
+            at = {**values, "__const__": 0}
+            for k, v in carry.items():
+                if isinstance(v, Affine):
+                    values[k] = v.evaluate(at)
+                elif not isinstance(v, Handle):
+                    values[k] = int(v)
+        return values
 
     def write(self, resident: Resident, array) -> None:
         """Write a state or weight of the graph from a host array."""
@@ -1426,8 +1452,24 @@ class CompiledGraph:
         """Replay the captured step ``n`` more times, each starting from the values the last one carried."""
         if self._graph is None:
             raise RuntimeError(f"{self.recording.name}: this version is not captured in a HIP graph")
+        if n <= 0:
+            return
+        known = vars(self).get("_host_values")
+        if known is None:
+            raise RuntimeError(f"{self.recording.name}: start() or a call runs the first step of a replayed run")
+        # Every step's values are checked before any is launched, as a call's are: past a limit the
+        # device would drop its cache writes and go on from stale rows without a word.  The carried
+        # formulas move one way, so the first and the last replay bound the rest.
+        first = self._after(known, 1)
+        last = self._after(first, n - 1)
+        try:
+            self.recording.check_values(first)
+            self.recording.check_values(last)
+        except IndexError as e:
+            raise IndexError(f"{e}; {n} replay(s) from {known} leave the limits") from None
         for _ in range(n):
             self._graph.replay()
+        self._host_values = last
 
     def _run_checked(self, full) -> None:
         """Per-step eager launches, each judged against its operator's ``reference()``."""

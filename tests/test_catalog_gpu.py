@@ -33,6 +33,43 @@ def test_operator_case(cuda, cls, case, record_property):
     assert not errors, {k: e.detail for k, e in errors.items()}
 
 
+LONGEST = [
+    pytest.param(case, id=f"MHA-{case.label}")
+    for case in CATALOG["MHA"].test.resolve(CATALOG["MHA"], None)
+    if case.kwargs.get("seq_len", 0) >= 16384
+]
+
+
+@pytest.mark.parametrize("case", LONGEST)
+def test_longest_attention_cases_on_sampled_queries(cuda, case):
+    """The catalog's 16384-row attention cases, whose whole reference takes the host minutes: the
+    operator runs whole through its own call, and every head of a sample of queries (both ends, tile
+    edges, random rows) is judged by the operator's tolerance against the one-query reference of that
+    query over its keys -- the same operator at ``seq_len=1``, which the causal case is row by row."""
+    import torch
+
+    from iron_amd.bf16 import from_torch, to_torch
+    from iron_amd.common.verify import compare
+
+    cls = CATALOG["MHA"]
+    op = cls(**case.kwargs)
+    assert op.causal and not op.heads_interleaved and not op.kv_interleaved
+    v = vectors(op, seed=42, scale=1.0)
+    Q, Kc, Vc = (v.inputs[n] for n in ("Q", "K", "V"))
+    O = torch.zeros(op.O.host_shape, dtype=torch.bfloat16, device="cuda")
+    op(*(to_torch(a).cuda() for a in (Q, Kc, Vc)), O)
+    got = from_torch(O)
+    S = op.seq_len
+    rng = np.random.default_rng(1)
+    rows = sorted({0, 1, 63, 64, 127, 128, 8191, 8192, S - 129, S - 128, S - 1, *rng.integers(0, S, 9).tolist()})
+    for r in rows:
+        one = cls(num_heads=op.num_heads, num_KV_heads=op.num_KV_heads, seq_len=1, kv_len=r + 1, d=op.d)
+        want = np.asarray(one.reference(Q[:, r : r + 1], Kc[:, : r + 1], Vc[:, : r + 1])).reshape(op.num_heads, op.d)
+        verdict = compare(got[:, r], want, op.tolerance())
+        assert verdict, f"query {r}: {verdict.detail}"
+        assert np.all(np.abs(got[:, r] - want) <= 1e-2 + 1e-2 * np.abs(want)), f"query {r}"
+
+
 def test_operator_api_refusals(cuda):
     import torch
 

@@ -242,6 +242,73 @@ def test_gemm_residual_epilogue(cuda, M, Kdim, N, rows, scale):
     close(from_torch(Rd)[:lim], want[:lim], rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("bound", [None, 512, 1281])
+@pytest.mark.parametrize("cache", [False, True])
+def test_prefill_qkv_at_the_decoder_s_width(cuda, bound, cache):
+    """The fused pre-attention launch at Llama-3.2-1B's own sizes: a 2048-row chunk of hidden 2048,
+    32 query and 8 KV heads, whole and under the bounds a prompt leaves (512 rows: the one-head
+    tiles; 1281: the 192-wide ones), against the oracle's three GEMMs, then RoPE."""
+    rng = np.random.default_rng(93)
+    rows, E, H, G, D, L, start = 2048, 2048, 32, 8, 64, 4096, 777
+    x = bf(rng, rows, E)
+    Wq, Wk, Wv = bf(rng, H * D, E, scale=0.02), bf(rng, G * D, E, scale=0.02), bf(rng, G * D, E, scale=0.02)
+    table = round_bf16(ops.rope_angles(D, rows, 500000.0))
+    lim = rows if bound is None else bound
+    q, k, v = (ops.gemm(x[:lim], W, b_col_maj=True) for W in (Wq, Wk, Wv))
+    want_q = ops.rope(q.reshape(lim * H, D), table[:lim]).reshape(lim, H * D)
+    want_k = ops.rope(k.reshape(lim * G, D), table[:lim]).reshape(lim, G * D)
+    if bound is not None:
+        x[bound:] = np.nan
+    valid = None if bound is None else word(bound, cuda)
+    args = [dev(a, cuda) for a in (x, Wq, Wk, Wv, table)]
+    q_out = out_like((rows, H * D), cuda, fill=7.0)
+    if cache:
+        keys, values = (out_like((L, G * D), cuda, fill=3.0) for _ in range(2))
+        K.prefill_qkv_cache(*args, q_out, keys, values, rows=rows, hidden=E, heads=H, kv_heads=G, d=D,
+                            cache_rows=L, start=word(start, cuda), valid=valid)
+        k_got, v_got = from_torch(keys), from_torch(values)
+        for got in (k_got, v_got):
+            assert np.all(got[:start] == 3.0) and np.all(got[start + lim :] == 3.0)
+        k_got, v_got = k_got[start : start + lim], v_got[start : start + lim]
+    else:
+        k_out, v_out = (out_like((rows, G * D), cuda, fill=7.0) for _ in range(2))
+        K.prefill_qkv(*args, q_out, k_out, v_out, rows=rows, hidden=E, heads=H, kv_heads=G, d=D, valid=valid)
+        k_got, v_got = from_torch(k_out), from_torch(v_out)
+        assert np.all(k_got[lim:] == 7.0) and np.all(v_got[lim:] == 7.0)
+        k_got, v_got = k_got[:lim], v_got[:lim]
+    q_got = from_torch(q_out)
+    assert np.all(q_got[lim:] == 7.0)
+    close(q_got[:lim], want_q)
+    close(k_got, want_k)
+    close(v_got, v)
+
+
+@pytest.mark.parametrize("M,Kdim,N", [(2048, 2048, 8192), (2048, 8192, 2048), (2048, 2048, 2048), (2048, 2048, 512)])
+@pytest.mark.parametrize("rows", [512, 1281])
+def test_prompt_chunk_projections_under_a_row_bound(cuda, M, Kdim, N, rows):
+    """The launches a bounded prompt chunk takes at Llama-3.2-1B's widths (blocks choosing their tile
+    by the bound, the ranges of the bound served by two launches): the plain product and the one
+    with its residual, at the full depth of K, poison past the bound, nothing written past it."""
+    rng = np.random.default_rng(M + Kdim + N + rows)
+    A, B, R = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.02), bf(rng, M, N)
+    want = ops.gemm(A[:rows], B, b_col_maj=True)
+    A[rows:] = np.nan
+    C = out_like((M, N), cuda, fill=5.0)
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=M, N=N, K=Kdim, b_col_maj=True, valid=word(rows, cuda))
+    got = from_torch(C)
+    close(got[:rows], want)
+    assert np.all(got[rows:] == 5.0)
+    Rd = dev(R, cuda)
+    K.gemm_residual(dev(A, cuda), dev(B, cuda), Rd, Rd, M=M, N=N, K=Kdim, residual_scale=1.0, valid=word(rows, cuda))
+    got = from_torch(Rd)
+    # The product is rounded to bf16 before the sum, as the separate step stores it: where float32
+    # sums in another order round it the other way, the sum moves by the PRODUCT's last place,
+    # however small the sum itself comes out.
+    total = ops.add(want, R[:rows])
+    assert np.all(np.abs(got[:rows] - total) <= ATOL + RTOL * np.abs(total) + 2.0**-7 * np.abs(want))
+    assert np.array_equal(got[rows:], R[rows:])
+
+
 @pytest.mark.parametrize("b_col_maj", [False, True])
 def test_gemm_bounded_rows_and_k_do_not_read_the_poison(cuda, b_col_maj):
     """NaN past the bounds must not reach the output (test_gemm_bounded_k.py)."""
@@ -558,6 +625,31 @@ def test_mha_decode_llama_shape(cuda, L):
     want = ops.mha(Q, Kc, Vc, num_heads=H, num_KV_heads=G, seq_len=1, kv_len=L, d=d, scale=0.125,
                    heads_interleaved=True, kv_interleaved=True)
     close(O, want)
+
+
+def test_mha_decode_is_as_accurate_deep_in_a_32k_cache_as_near_its_start(cuda):
+    """The reference's long-context check (iron/tests/operators/test_mha_long_context.py:45-62): one
+    query of Llama-3.2-1B's packed heads over a 32768-row cache of 55 distinct rows tiled over its
+    length (every key block weighs alike and the outputs stay far from 0, so a running sum that loses
+    a block's share shows), at positions 1023 and 32703, within 4 % of the output's peak -- and,
+    float32 sums losing nothing of the kind here, within the stated bf16 tolerance as well."""
+    rng = np.random.default_rng(0)
+    H, G, d, L, distinct = 32, 8, 64, 32768, 55
+    Kc = round_bf16(np.resize(rng.standard_normal((distinct, G, d)) * 2, (L, G, d)).astype(np.float32))
+    Vc = round_bf16(np.resize(rng.standard_normal((distinct, G, d)), (L, G, d)).astype(np.float32))
+    Q = round_bf16(rng.standard_normal((1, H, d)).astype(np.float32))
+    ws = K.mha_decode_workspace(H, d, cuda)
+    Kd, Vd, Qd = dev(Kc, cuda), dev(Vc, cuda), dev(Q, cuda)
+    for position in (1023, L - 65):
+        O = out_like((1, H, d), cuda, fill=float("nan"))
+        K.mha_decode(Qd, Kd, Vd, O, heads=H, kv_heads=G, d=d, kv_len=L, kv_interleaved=True,
+                     kv_valid=word(position + 1, cuda), workspace=ws)
+        want = ops.mha(Q, Kc, Vc, num_heads=H, num_KV_heads=G, seq_len=1, kv_len=L, d=d, heads_interleaved=True,
+                       kv_interleaved=True, kv_valid=position + 1)
+        got = from_torch(O).reshape(want.shape)
+        peak = float(np.abs(want).max())
+        assert peak > 0.5 and np.abs(got - want).max() <= 0.04 * peak, (position, np.abs(got - want).max(), peak)
+        close(got, want)
 
 
 @pytest.mark.parametrize("H,G,d", [(32, 8, 64), (8, 8, 64), (24, 8, 128), (40, 8, 64), (4, 1, 256), (16, 8, 64), (12, 2, 64), (3, 1, 64)])
