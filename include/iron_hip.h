@@ -242,8 +242,9 @@ int iron_argmax_bf16(const uint16_t* logits, int n, int* token, int* record, int
  * lower index; candidate i weighs exp((l_i - l_0) / temperature) in float64 and the token is the
  * first whose running weight exceeds number * 2^-53 * total.  token, record, at, token_copy as
  * iron_argmax_bf16.  1 <= k_max <= 64; n <= 524288.  workspace: iron_sample_workspace_bytes(n)
- * bytes, 8-byte aligned, any contents (NULL allowed for n <= 2048).  One launch; launches on one
- * device must not overlap (they count their blocks in one device-wide word).
+ * bytes, 8-byte aligned (NULL allowed for n <= 2048); its first 16 bytes count the launch's blocks:
+ * zero before the workspace's first launch, left zero by every launch; the rest may hold anything.
+ * One launch; launches that share a workspace must not overlap.
  * Replaces Sample: iron/operators/sample.py:72-79,106-336 (its sample_ref is out of the
  * reference's tree; the arithmetic above is this library's own, fixed so a host computes the
  * same token bit for bit). */
@@ -260,15 +261,6 @@ int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_
  * The device-side carry/Emit of a decode loop (position += 1, kv_valid = position + 1):
  * iron/common/graph/carried.py:189-276, iron/operators/emit.py. */
 int iron_eval_words(int* words, int n_words, const int* exprs, int n, void* stream);
-
-/* Measurement aid (no counterpart in the reference; bench.py's MFMA ceiling): IRON_PROBE_BLOCKS
- * blocks of 4 waves run `iters` rounds of 16 independent 32x32x16 bf16 MFMAs from registers.
- * operands: operand_count bf16 values the fragments are drawn from, or NULL for constants.
- * sink: IRON_PROBE_BLOCKS*256 floats.  iron_probe_mfma_flops(iters) = flops of one launch. */
-#define IRON_PROBE_BLOCKS 512
-int iron_probe_mfma_bf16(const uint16_t* operands, int64_t operand_count, float* sink, int iters,
-                         void* stream);
-int64_t iron_probe_mfma_flops(int iters);
 
 #ifdef __cplusplus
 }

@@ -65,8 +65,6 @@ SIGNATURES = {
     "iron_sample_workspace_bytes": (c_int64, [c_int]),
     "iron_sample_bf16": (c_int, [_P, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P]),
     "iron_eval_words": (c_int, [_P, c_int, _P, c_int, _P]),
-    "iron_probe_mfma_bf16": (c_int, [_P, c_int64, _P, c_int, _P]),
-    "iron_probe_mfma_flops": (c_int64, [c_int]),
 }
 
 

@@ -151,8 +151,8 @@ class Select:
 
 class OperandDecl(_Member):
     def __init__(self, dims, *, fills, drains, dtype=bfloat16, obj_shape=None, per=None, depth=None,
-                 replicate=False, when=None, like=None, scratch=False):
-        self.dims, self.fills, self.drains, self.scratch = dims, fills, drains, scratch
+                 replicate=False, when=None, like=None, scratch=False, kept=False):
+        self.dims, self.fills, self.drains, self.scratch, self.kept = dims, fills, drains, scratch, kept
         self.dtype, self.obj_shape, self.per, self.depth = dtype, obj_shape, per, depth
         self.replicate, self.when, self.like = replicate, when, like
 
@@ -176,7 +176,9 @@ def InOut(*dims, **kw) -> Any:  # noqa: N802
 
 def Scratch(*dims, **kw) -> Any:  # noqa: N802
     """Device memory a kernel needs beside its operands (partial results): a graph places it
-    in the arena as a transient; a call outside a graph allocates it once."""
+    in the arena as a transient; a call outside a graph allocates it once.  ``kept=True``: memory
+    whose contents the kernel counts on finding as it left them (zero at first), which a graph
+    places among its residents instead, one per step."""
     return OperandDecl(dims, fills=False, drains=False, scratch=True, **kw)
 
 
@@ -190,6 +192,7 @@ class Operand:
     fills: bool
     drains: bool
     replicate: bool = False
+    kept: bool = False
 
     @property
     def host_shape(self) -> tuple[int, ...]:
@@ -348,7 +351,7 @@ class Operator:
             return None
         src = decl if decl.like is None else decl.like
         dtype = _value_of(self, src.dtype)
-        return Operand(decl.name, self._dims(src.dims), dtype, decl.fills, decl.drains, decl.replicate)
+        return Operand(decl.name, self._dims(src.dims), dtype, decl.fills, decl.drains, decl.replicate, decl.kept)
 
     @property
     def buffers(self) -> list[Operand]:

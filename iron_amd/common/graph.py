@@ -616,8 +616,11 @@ class Recorder:
                     h = dataclasses.replace(h, shape=tuple(seen_as))
                 outputs[b.name] = dataclasses.replace(h, valid=op.output_valid(b.name, inputs))
         result = [outputs[b.name] for b in declared_out]
-        for b in op.scratch:  # placed in the arena, live over this step only
-            outputs[b.name] = self.transient(b.shape, b.dtype, f"{cls.__name__.lower()}_{b.name}")
+        for b in op.scratch:  # placed in the arena, live over this step only -- or, kept, for good
+            if b.kept:
+                outputs[b.name] = self.resident(state(b.shape, b.dtype))
+            else:
+                outputs[b.name] = self.transient(b.shape, b.dtype, f"{cls.__name__.lower()}_{b.name}")
         for name, h in {**inputs, **outputs}.items():
             if h.index is not None:
                 width = max(h.elements // h.index_stride, 1)  # rows the view spans

@@ -17,9 +17,10 @@ constexpr int SAMPLE_SHARE = 2048;      // logits a block selects from: a 16-byt
 constexpr int SAMPLE_BLOCKS_MAX = 256;
 constexpr int SAMPLE_LIST = SAMPLE_SHARE;
 
-// Blocks done with their lists; the last one to come resets it, so it is zero between launches.
-// One per device: launches that overlap on a device (two streams) would share it.
-__device__ unsigned int sample_ticket;
+// Blocks done with their lists are counted in the first word of the caller's workspace (the lists
+// start SAMPLE_TICKET_BYTES in): zero before the workspace's first launch, and the last block to come
+// sets it back to zero, so launches that share no workspace share no counter.
+constexpr int SAMPLE_TICKET_BYTES = 16;
 
 // 16 raw bf16 bits -> a key whose unsigned order is the logits' order.
 __device__ __forceinline__ uint32_t order_key(uint32_t b) {
@@ -202,10 +203,12 @@ __device__ double exp_det(double z) {
 // lists: gridDim.x lists of SAMPLE_K_MAX entries, from each block's best, 0 past its last.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const bf16_t* __restrict__ logits, int n, const int* __restrict__ draws, int draws_words,
-    const int* __restrict__ row, int k_max, uint64_t* lists, int* __restrict__ token,
+    const int* __restrict__ row, int k_max, uint64_t* workspace, int* __restrict__ token,
     int* __restrict__ record, int record_len, const int* __restrict__ at,
     int* __restrict__ token_copy) {
   __shared__ SampleShared sh;
+  unsigned int* ticket = reinterpret_cast<unsigned int*>(workspace);
+  uint64_t* lists = workspace + SAMPLE_TICKET_BYTES / 8;
 
   // The draw row: {temperature (float32 bits), top-k, the 53-bit number's low and high word}.
   // A row outside the buffer, like a temperature that is not positive, is the greedy draw.
@@ -259,12 +262,16 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       publish(&lists[(size_t)blockIdx.x * SAMPLE_K_MAX + threadIdx.x], sh.cand[threadIdx.x]);
   }
   if (blocks > 1) {
-    // The lists are out (each thread has waited for its own stores); the block whose ticket is
-    // the last goes on with all of them.
+    // The lists are out: each thread's agent-scope stores have been acknowledged from past the
+    // XCD's L2 (the wait below counts them down) before the block's barrier, and the barrier comes
+    // before the ticket, so a block that sees the last ticket finds every list where its own
+    // agent-scope loads read: in device memory.  The ticket is relaxed on purpose: a release/acquire
+    // pair at agent scope would write back and invalidate the whole L2 on either side (the logits
+    // the head just wrote are dirty lines in it), which costs more than this kernel's other work.
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0)
-      sh.last_block = __hip_atomic_fetch_add(&sample_ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+      sh.last_block = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
                       (unsigned)blocks - 1;
     __syncthreads();
     if (!sh.last_block) return;
@@ -300,7 +307,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
       });
     }
-    if (threadIdx.x == 0) atomicExch(&sample_ticket, 0u);
+    if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
 
@@ -352,7 +359,7 @@ using namespace iron;
 static int sample_blocks(int n) { return (n + SAMPLE_SHARE - 1) / SAMPLE_SHARE; }
 
 extern "C" int64_t iron_sample_workspace_bytes(int n) {
-  return (int64_t)sample_blocks(n) * SAMPLE_K_MAX * 8;
+  return SAMPLE_TICKET_BYTES + (int64_t)sample_blocks(n) * SAMPLE_K_MAX * 8;
 }
 
 extern "C" int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,

@@ -408,7 +408,8 @@ def argmax(logits, token, *, n=None, record=None, at=None, token_copy=None):
 
 
 def sample_workspace(n, device="cuda"):
-    return torch.empty(lib().iron_sample_workspace_bytes(n) // 8, dtype=torch.int64, device=device)
+    """The draw's workspace, zeroed: its first words count a launch's blocks and start at zero."""
+    return torch.zeros(lib().iron_sample_workspace_bytes(n) // 8, dtype=torch.int64, device=device)
 
 
 def sample(logits, draws, token, *, n=None, row=None, k_max=64, workspace=None, record=None, at=None,
@@ -442,20 +443,3 @@ def eval_words(words, exprs, n=None):
     n = exprs.numel() // 9 if n is None else n  # nine words a record
     check(lib().iron_eval_words(ptr(words), words.numel(), ptr(exprs), n, current_stream()), "iron_eval_words")
 
-
-PROBE_BLOCKS = 512
-
-
-def probe_mfma(operands, sink, iters):
-    """Launch the register-only MFMA loop (a measurement aid); returns the flops of the launch."""
-    if operands is not None:
-        _dev(operands, "operands", torch.bfloat16)
-    _dev(sink, "sink", torch.float32)
-    if sink.numel() < PROBE_BLOCKS * 256:
-        raise ValueError(f"sink: {sink.numel()} floats, {PROBE_BLOCKS * 256} needed")
-    check(
-        lib().iron_probe_mfma_bf16(ptr(operands), 0 if operands is None else operands.numel(), ptr(sink), iters,
-                                   current_stream()),
-        "iron_probe_mfma_bf16",
-    )
-    return lib().iron_probe_mfma_flops(iters)

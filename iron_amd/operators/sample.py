@@ -64,8 +64,9 @@ class Sample(Operator):
     draws = In(steps, ROW_WORDS, dtype=np.int32)
     tokens = InOut(steps, dtype=np.int32)
     token = Out(1, dtype=np.int32)
-    # The blocks' candidate lists.
-    workspace = Scratch(workspace_words, dtype=np.float32)
+    # The blocks' candidate lists behind the word that counts the blocks, which every launch finds
+    # and leaves at zero: kept from call to call.
+    workspace = Scratch(workspace_words, dtype=np.float32, kept=True)
     # The word of `draws` the call's row starts at, and the record slot it writes.
     row = per_call(bounds=None)
     at = per_call(bounds=None)
