@@ -206,6 +206,17 @@ int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int heads, int kv_heads, int d, int kv_len, float scale, int window,
                          int kv_interleaved, const int* kv_valid, void* workspace, void* stream);
 int64_t iron_mha_decode_workspace_bytes(int heads, int d);
+/* iron_mha_decode_bf16 for callers that cannot allocate (code under HIP-graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same kernels, their split-KV partial results
+ * in a scratch array the library holds in device memory itself (iron_mha_decode_static_max_bytes()
+ * bytes on each GPU it runs on, until the process ends), so no workspace is passed and nothing is
+ * allocated or freed.  Refused (1) when iron_mha_decode_workspace_bytes(heads, d) exceeds that size.
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU race.  Nothing in it
+ * has to start at zero.  No counterpart in the reference. */
+int iron_mha_decode_static_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
+                                int heads, int kv_heads, int d, int kv_len, float scale, int window,
+                                int kv_interleaved, const int* kv_valid, void* stream);
+int64_t iron_mha_decode_static_max_bytes(void);
 /* One query over a window of a longer buffer of keys, as iron_mha_prefill_at_bf16. */
 int iron_mha_decode_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
                             int heads, int kv_heads, int d, int kv_len, float scale, int window,

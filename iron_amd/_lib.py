@@ -47,6 +47,11 @@ SIGNATURES = {
         [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, _P, _P],
     ),
     "iron_mha_decode_workspace_bytes": (c_int64, [c_int, c_int]),
+    "iron_mha_decode_static_bf16": (
+        c_int,
+        [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, _P],
+    ),
+    "iron_mha_decode_static_max_bytes": (c_int64, []),
     "iron_mha_prefill_at_bf16": (
         c_int,
         [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, _P, _P, c_int, _P],

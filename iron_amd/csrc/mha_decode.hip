@@ -11,6 +11,8 @@
 #include "../../include/iron_hip.h"
 #include "common.h"
 
+#include <mutex>
+
 namespace iron {
 
 constexpr int kMaxSplits = 128;
@@ -447,6 +449,59 @@ extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const 
                                     const int* kv_valid, void* workspace, void* stream) {
   return mha_decode(Q, K, V, O, heads, kv_heads, d, kv_len, scale, window, kv_interleaved, kv_valid, nullptr, 0,
                     workspace, stream);
+}
+
+// ---- the entry point that allocates nothing
+//
+// The split kernel's partial results in device memory the library itself holds: a file-scope array,
+// one copy per GPU, there from the moment the code object is loaded until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress, never an address: the device
+// address is asked for once per device, with that device current, and kept.
+namespace iron {
+constexpr int64_t kScratchBytes = 8 << 20;
+constexpr int kScratchDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static void* scratch_ptr[kScratchDevices];     // per device: the array's address there
+static std::mutex scratch_mutex;
+
+// The current device's copy of the array, or null with the reason set.
+static void* scratch_here() {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= kScratchDevices) {
+    set_error("mha_decode_static: no current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(scratch_mutex);
+  if (scratch_ptr[device] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("mha_decode_static: the scratch array has no address on device %d (%s)", device, hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_ptr[device] = p;
+  }
+  return scratch_ptr[device];
+}
+}  // namespace iron
+
+extern "C" int64_t iron_mha_decode_static_max_bytes(void) { return kScratchBytes; }
+
+extern "C" int iron_mha_decode_static_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                           uint16_t* O, int heads, int kv_heads, int d, int kv_len,
+                                           float scale, int window, int kv_interleaved,
+                                           const int* kv_valid, void* stream) {
+  IRON_REQUIRE(heads > 0 && d > 0, "mha_decode_static: heads (%d) and d (%d) must be positive", heads, d);
+  const int64_t need = iron_mha_decode_workspace_bytes(heads, d);
+  IRON_REQUIRE(need <= kScratchBytes,
+               "mha_decode_static: %d heads of width %d need %lld bytes of partial results; the library's own "
+               "scratch holds %lld (use iron_mha_decode_bf16 with a workspace of the caller's)",
+               heads, d, (long long)need, (long long)kScratchBytes);
+  void* ws = scratch_here();
+  if (ws == nullptr) return IRON_EINVAL;
+  return mha_decode(Q, K, V, O, heads, kv_heads, d, kv_len, scale, window, kv_interleaved, kv_valid, nullptr, 0, ws,
+                    stream);
 }
 
 extern "C" int iron_mha_decode_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,

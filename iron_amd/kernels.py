@@ -354,6 +354,25 @@ def mha_decode(
     )
 
 
+def mha_decode_static(Q, K, V, O, *, heads, kv_heads, d, kv_len, scale=None, window=None, kv_interleaved=False,
+                      kv_valid=None):
+    """``mha_decode`` with the split-KV partial results in the library's own device scratch: no
+    workspace, nothing allocated (for callers that cannot allocate); refused past its fixed size."""
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    _numel(_dev(Q, "Q"), heads * d, "Q")
+    _numel(_dev(O, "O"), heads * d, "O")
+    _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
+    _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
+    check(
+        lib().iron_mha_decode_static_bf16(
+            ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, kv_len, float(scale),
+            -1 if window is None else int(window), int(kv_interleaved),
+            ptr(_word(kv_valid, "kv_valid")), current_stream(),
+        ),
+        "iron_mha_decode_static_bf16",
+    )
+
+
 def gather_rows(table, ids, out, *, valid=None):
     _dev(table, "table", None)
     _dev(ids, "ids", torch.int32)
