@@ -114,26 +114,77 @@ def bench_library_reference(torch, dev, n, rng):
     return out
 
 
-def bench_mfma_ceiling(torch, K, dev, rng):
-    """What the MFMA units sustain from registers alone: with constant operands, and with operands
-    drawn like the GEMM's (N(0,1)*0.02) -- under the power cap the clock depends on the data."""
-    from iron_amd.bf16 import round_bf16, to_torch
+def bench_decode_kernels(torch, K, dev, n, rng):
+    """Each kernel the captured decode step of the Llama-3.2-1B shape launches, alone at its own shape:
+    a replayed HIP graph of back-to-back launches over distinct weights (more than the last-level
+    cache holds), timed with HIP events on the graph's stream.  ``per_step`` is how often a decode
+    step launches it; ``bytes`` the algorithmic bytes of one launch (its weights, vectors and cache
+    rows), ``frac_hbm`` those over the duration against the published HBM peak."""
+    E, F, H, G, D, V, L, pos = 2048, 8192, 32, 8, 64, 128256, 2048, 576
 
-    sink = torch.empty(K.PROBE_BLOCKS * 256, dtype=torch.float32, device=dev)
-    drawn = to_torch(round_bf16(rng.standard_normal(1 << 21, dtype=np.float32) * np.float32(0.02))).to(dev)
-    out = {}
-    for name, ops in (("constant", None), ("random", drawn)):
-        iters = 4000
-        flops = K.probe_mfma(ops, sink, iters)
-        torch.cuda.synchronize()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(3):
-            K.probe_mfma(ops, sink, iters)
-        stop.record()
-        stop.synchronize()
-        out[name] = round(3 * flops / (start.elapsed_time(stop) * 1e-3) / 1e12, 1)
-    return out
+    def drawn(*shape, scale=0.02):
+        return (torch.randn(*shape, device=dev) * scale).to(torch.bfloat16)
+
+    def pool(bytes_each, make):
+        return [make() for _ in range(max(2, min(96, int(np.ceil(640e6 / bytes_each)))))]
+
+    x, gain = drawn(E, scale=1.0), (torch.rand(E, device=dev) * 0.2 + 0.9).to(torch.bfloat16)
+    position = torch.tensor([pos], dtype=torch.int32, device=dev)
+    kv_valid = torch.tensor([pos + 1], dtype=torch.int32, device=dev)
+    angles = drawn(D, scale=1.0)
+    q, y, m = torch.empty(H * D, dtype=torch.bfloat16, device=dev), torch.empty(E, dtype=torch.bfloat16, device=dev), \
+        drawn(F, scale=1.0)
+    rows = []
+
+    def add(name, kernel, per_step, nbytes, launches):
+        us = graph_time_us(torch, launches, max(1, n // len(launches)))
+        rows.append({"name": name, "kernel": kernel, "per_step": per_step, "bytes": int(nbytes), "us": round(us, 3),
+                     "GBps": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+
+    # attention's first half: norm, q/k/v projections, RoPE, the cache rows
+    qkv_bytes = 2 * ((H + 2 * G) * D * E + 2 * E + (H + 2 * G) * D)
+    caches = pool(2 * L * G * D * 2, lambda: (drawn(L, G, D, scale=1.0), drawn(L, G, D, scale=1.0)))
+    ws = pool(qkv_bytes, lambda: (drawn(H * D, E), drawn(G * D, E), drawn(G * D, E)))
+    add("norm + q/k/v + RoPE + cache write", "decode_qkv_kernel<64,1>", 16, qkv_bytes,
+        [(lambda w=w, c=caches[i % len(caches)]: K.decode_qkv(x, gain, w[0], w[1], w[2], angles, q, c[0], c[1], eps=1e-5,
+                                                               hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
+                                                               position=position)) for i, w in enumerate(ws)])
+    del ws
+    # attention over the cache (one query, pos + 1 keys)
+    att_bytes = 2 * (pos + 1) * G * D * 2 + 2 * H * D * 2
+    wsp = K.mha_decode_workspace(H, D, dev)
+    o = torch.empty(1, H, D, dtype=torch.bfloat16, device=dev)
+    add(f"attention, one query over {pos + 1} keys", "mha_decode_single_kernel<64>", 16, att_bytes,
+        [(lambda c=c: K.mha_decode(q.reshape(1, H, D), c[0], c[1], o, heads=H, kv_heads=G, d=D, kv_len=L, scale=0.125,
+                                   kv_interleaved=True, kv_valid=kv_valid, workspace=wsp)) for c in caches])
+    del caches
+    # o projection + residual
+    ws = pool(2 * E * H * D, lambda: drawn(E, H * D))
+    add("o projection + residual", "gemv_fused_kernel<1,1,false,1>", 16, 2 * (E * H * D + H * D + 2 * E),
+        [(lambda w=w: K.gemv_fused(w, q, y, M=E, K=H * D, residual=x, epilogue=1)) for w in ws])
+    del ws
+    # norm + gate/up + SiLU * mul
+    ws = pool(4 * F * E, lambda: (drawn(F, E), drawn(F, E)))
+    mm = torch.empty(F, dtype=torch.bfloat16, device=dev)
+    add("norm + gate/up + SiLU*mul", "gemv_fused_kernel<2,1,true,2>", 16, 2 * (2 * F * E + 2 * E + F),
+        [(lambda w=w: K.gemv_fused(w[0], x, mm, M=F, K=E, W2=w[1], norm_w=gain, eps=1e-5, epilogue=2)) for w in ws])
+    del ws
+    # down projection + residual
+    ws = pool(2 * E * F, lambda: drawn(E, F))
+    add("down projection + residual", "gemv_fused_kernel<1,4,false,1>", 16, 2 * (E * F + F + 2 * E),
+        [(lambda w=w: K.gemv_fused(w, m, y, M=E, K=F, residual=x, epilogue=1)) for w in ws])
+    del ws
+    # final norm + head
+    ws = pool(2 * V * E, lambda: drawn(V, E))
+    logits = torch.empty(V, dtype=torch.bfloat16, device=dev)
+    add("final norm + LM head", "gemv_fused_kernel<4,1,true,0>", 1, 2 * (V * E + 2 * E + V),
+        [(lambda w=w: K.gemv_fused(w, x, logits, M=V, K=E, norm_w=gain, eps=1e-5, epilogue=0)) for w in ws])
+    del ws
+    torch.cuda.empty_cache()
+    total = sum(r["per_step"] * r["us"] for r in rows)
+    for r in rows:
+        r["share_of_listed_us"] = round(r["per_step"] * r["us"] / total, 4)
+    return rows
 
 
 def bench_attention(torch, K, dev, n, rng):
@@ -285,7 +336,7 @@ def prompt_probe(torch, dev, repeats=20):
     for _ in range(repeats):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for inputs, values in model.session._chunks(prompt, 0):
+        for inputs, values in model.session.chunk_calls(prompt, 0):
             model(*inputs, **values)
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
@@ -294,7 +345,7 @@ def prompt_probe(torch, dev, repeats=20):
                       "ttft_ms_median": round(1e3 * float(np.median(times)), 3)}))
 
 
-def bench_decoder(torch, dev, steps, warmup, with_cpu):
+def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
     """Llama-3.2-1B shape: a 512-token prompt prefill, then ``steps`` greedy decode steps as
     replays of the captured decode step (each starts from the token and position the last one
     carried on the device)."""
@@ -311,14 +362,36 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu):
 
     def prefill():
         carry = None
-        for inputs, values in session._chunks(prompt, 0):
-            _, carry = model(*inputs, **values)
+        for inputs, values in session.chunk_calls(prompt, 0):
+            logits, carry = model(*inputs, **values)
+        prefill.last = logits
         return carry
 
     carry = prefill()
+    # A copy now: the decode steps write their logits where the prompt's were.
+    prompt_logits = np.array(prefill.last.numpy()).reshape(-1)[: config.vocab_size]
     decode.start(**carry)
     decode.replay(max(warmup, 1))
     torch.cuda.synchronize()
+    if probe_steps:   # a decode-only run for a kernel trace or a counter run: nothing else is launched after this
+        carry = prefill()
+        decode.start(**carry)
+        decode.replay(probe_steps - 1)
+        torch.cuda.synchronize()
+        # ... and a plain copy of known size, which turns a counter run's FETCH_SIZE / WRITE_SIZE into bytes
+        from iron_amd import kernels as K
+
+        rows = PROBE_COPY_BYTES // 4096
+        src = torch.zeros(PROBE_COPY_BYTES // 4, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            K.copy_rows(src, dst, rows=rows, row_elems=1024, src_rows=rows, dst_rows=rows)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "decode", "prefill_tokens": 512, "decode_steps": probe_steps,
+                          "launches_per_step": decode.launches_per_call,
+                          "copy": {"launches": 2, "bytes_read": PROBE_COPY_BYTES, "bytes_written": PROBE_COPY_BYTES}}))
+        model.release()
+        return None, None
 
     t0 = time.perf_counter()
     carry = prefill()
@@ -351,16 +424,23 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu):
            "launches_per_prompt_chunk": model.prompt_chunk.launches_per_call, "first_tokens": [int(t) for t in tokens[:4]]}
     cpu = None
     if with_cpu:
-        cpu = cpu_decoder_baseline(torch, config, weights)
+        drawn = decode.read(model.drawn)[511 : 512 + steps]   # the prompt's draw, then each decode step's
+        cpu, out["checked"] = cpu_decoder_baseline(torch, config, weights, prompt, prompt_logits, [int(t) for t in drawn])
     model.release()
     return out, cpu
 
 
-def cpu_decoder_baseline(torch, config, weights, budget_s=12.0):
+def cpu_decoder_baseline(torch, config, weights, prompt, gpu_prompt_logits, gpu_tokens, budget_s=12.0):
     """The oracle's graph reference (the reference's CPU path: the graph run step by step through
-    each operator's numpy reference) timed on the host cores for a few decode steps of the same
-    16-layer model at position 512 (the prompt is not prefilled on the CPU: the cost of a decode
-    step does not depend on what the cache holds)."""
+    each operator's numpy reference) on the same 16-layer model and the same 512-token prompt.
+
+    First the check that makes the timed model a checked one: the host's logits after the prompt
+    against the GPU's by the reference's rule (within 5 % of the largest logit, the same argmax
+    where the top two are further apart than that: iron/lm/testing.py:182-206), and the GPU's first
+    drawn token against the host's logits.  Then decode steps from the GPU's own tokens are timed on
+    the host cores for about ``budget_s`` seconds, each compared with the GPU's next token the same way."""
+    import dataclasses
+
     import oracle
     from iron_amd.applications.llama import Llama
     from iron_amd.bf16 import from_torch
@@ -371,27 +451,48 @@ def cpu_decoder_baseline(torch, config, weights, budget_s=12.0):
     class HostLlama(OnHost, Llama):
         pass
 
+    def judge(host_logits, got_logits, got_token, what):
+        scale = float(np.abs(host_logits).max())
+        second, best = np.sort(host_logits)[-2:]
+        if got_logits is not None:
+            err = float(np.abs(got_logits - host_logits).max())
+            assert err <= 0.05 * scale, f"{what}: max |diff| {err:.4f} against |logits| {scale:.3f}"
+            if best - second > 0.05 * scale:
+                assert int(got_logits.argmax()) == int(host_logits.argmax()), f"{what}: argmax differs"
+        # the token the device drew is the host's best, or within the logits' tolerance of it
+        assert host_logits[got_token] >= best - 0.05 * scale, f"{what}: the drawn token {got_token} is not a best one"
+        return round(float(np.abs(got_logits - host_logits).max()) / scale, 5) if got_logits is not None else None
+
     host_weights = {n: from_torch(t) for n, t in weights.items()}
-    model = HostLlama(config, host_weights)
+    # The host's chunk is as long as the prompt: the rows past a bound are nobody's.
+    model = HostLlama(dataclasses.replace(config, prefill_chunk=len(prompt)), host_weights)
     model.load_versions()
-    carry = {"token": 1, "position": 512}
-    _, carry = model(**carry)  # records the graph and warms the caches
     t0 = time.perf_counter()
-    steps = 0
-    while time.perf_counter() - t0 < budget_s and carry["position"] < config.max_seq_len - 1:
-        _, carry = model(**carry)
+    host_logits = model.logits(prompt)
+    prefill_s = time.perf_counter() - t0
+    share = judge(host_logits, gpu_prompt_logits, gpu_tokens[0], "the prompt's logits")
+    history, steps, checked = list(map(int, prompt)), 0, 1
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < budget_s and steps + 1 < len(gpu_tokens):
+        history.append(gpu_tokens[steps])
+        row = model.logits(history)
         steps += 1
+        judge(row, None, gpu_tokens[steps], f"decode step {steps}")
+        checked += 1
     dt = time.perf_counter() - t0
-    return {"value": round(steps / dt, 3), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{steps} decode steps at positions 513.. of the same 16-layer model through the oracle's "
-                      f"graph reference, {dt:.1f} s wall; weights held as float32, prompt not prefilled on the CPU"}
+    cpu = {"value": round(steps / dt, 3), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"{steps} decode steps after the same 512-token prompt (prefilled on the host in {prefill_s:.1f} s) "
+                     f"of the same 16-layer model through the oracle's graph reference, teacher-forced on the GPU's "
+                     f"tokens, {dt:.1f} s wall; weights held as float32 (the reference widens bf16 on every call)"}
+    return cpu, {"rule": "within 5 % of the largest logit; same argmax where the top two are apart; each GPU token a best "
+                         "one of the host's logits", "prompt_logits_max_diff_share": share, "tokens_checked": checked}
 
 
 PROBE_COPY_BYTES = 512 << 20
-# HBM bytes one launch of the head GEMV moves, from hardware counters (FETCH_SIZE and WRITE_SIZE of
-# `--counter-probe`, each scaled by what the same counter reads for the probe's 512 MiB copy):
-# 513122 KiB fetched + 1002 KiB written.  The algorithmic figure is 525.6 MB.
-HEAD_GEMV_TRAFFIC_BYTES = (513122 + 1002) * 1024
+# HBM bytes one launch moves, by kernel, from hardware counters (FETCH_SIZE and WRITE_SIZE per
+# dispatch, each scaled by what the same counter reads for a plain copy of PROBE_COPY_BYTES): filled
+# from counter runs of `--decode-probe` / `--counter-probe`; a kernel without a reading reports null.
+DOMINANT_TRAFFIC_BYTES: dict[str, int] = {}
 
 
 def counter_probe(torch, K, dev, rng):
@@ -447,6 +548,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--counter-probe", action="store_true",
                     help="launch only the LM-head GEMV, a plain copy of known size and the MFMA kernels (for a rocprofv3 --pmc run) and exit")
+    ap.add_argument("--no-library", action="store_true",
+                    help="skip the vendor-library leg (torch.matmul / SDPA for scale): a kernel trace then lists this build's kernels only")
+    ap.add_argument("--decode-probe", type=int, default=0, metavar="N",
+                    help="prefill the 512-token prompt once, replay N decode steps and exit (for a rocprofv3 --kernel-trace or --pmc run)")
     ap.add_argument("--prompt-probe", action="store_true",
                     help="run only the decoder's 512-token prompt chunk, 20 times (for a rocprofv3 --kernel-trace run) and exit")
     args = ap.parse_args()
@@ -482,6 +587,9 @@ def main():
     if args.prompt_probe:
         prompt_probe(torch, dev)
         return 0
+    if args.decode_probe:
+        bench_decoder(torch, dev, args.steps, args.warmup, False, probe_steps=args.decode_probe)
+        return 0
 
     t_wall = time.perf_counter()
     n = args.kernel_launches
@@ -491,17 +599,16 @@ def main():
     gemm += [bench_gemm(torch, K, dev, max(20, n // 4), rng, True, M=m, N=nn, Kd=k)
              for m, nn, k in ((2048, 8192, 2048), (2048, 2048, 8192), (4096, 4096, 4096), (8192, 8192, 8192))]
     attention = bench_attention(torch, K, dev, n, rng)
-    mfma_ceiling = bench_mfma_ceiling(torch, K, dev, rng)
-    for g in gemm:
-        g["frac_sustained"] = round(g["TFLOPs"] / mfma_ceiling["random"], 4)
     pre_attention = bench_pre_attention(torch, K, dev, n)
     sample = bench_sample(torch, K, dev, n, rng)
-    library = bench_library_reference(torch, dev, n, rng)
+    library = None if args.no_library else bench_library_reference(torch, dev, n, rng)
+    decode_kernels = bench_decode_kernels(torch, K, dev, n, rng)
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     decoder, cpu = bench_decoder(torch, dev, args.steps, args.warmup, not args.no_cpu)
     wall = time.perf_counter() - t_wall
 
+    dominant = max(decode_kernels, key=lambda r: r["per_step"] * r["us"])
     sweep_bytes = sum(g["bytes"] for g in gemv)
     sweep_us = sum(g["us"] for g in gemv)
     head = gemv[-1]
@@ -523,18 +630,24 @@ def main():
                                "512-token prompt prefill, then greedy decode steps replayed as a HIP graph; "
                                "one step = one decoded token",
                    "prefill_tokens": 512, "decode_steps": args.steps},
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<4,4> (the 2048->128256 LM head, the largest launch of a "
-                                               "decode step)",
-                     "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["frac_hbm"], "traffic": HEAD_GEMV_TRAFFIC_BYTES},
+        "roofline": {"bound": "hbm", "kernel": dominant["kernel"], "what": dominant["name"],
+                     "why": f"the decode step's dominant kernel by time ({dominant['per_step']} launches a step, "
+                            f"{dominant['share_of_listed_us']:.0%} of the step's kernel time); timed alone at its shape "
+                            "over distinct weights with HIP events in this run",
+                     "achieved": dominant["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dominant["frac_hbm"],
+                     "us": dominant["us"], "algorithmic_bytes": dominant["bytes"],
+                     "traffic": DOMINANT_TRAFFIC_BYTES.get(dominant["kernel"]),
+                     "traffic_source": "a separate rocprofv3 --pmc run of `bench.py --decode-probe` (FETCH_SIZE + "
+                                       "WRITE_SIZE per dispatch, scaled by the same counters over a copy of known size); "
+                                       "not measured in this run"},
+        "decode_step_kernels": decode_kernels,
         "decoder": decoder,
         "gemv_sweep": {"GBps": round(sweep_bytes / sweep_us / 1e3, 1), "shapes": gemv},
         "gemm": gemm,
-        "mfma_sustained_TFLOPs": mfma_ceiling,
         "attention": attention,
         "pre_attention_block": pre_attention,
         "sample": sample,
-        "library_reference": library,
+        **({} if library is None else {"library_reference": library}),
         "bench_wall_s": round(wall, 1),
     }
     if cpu is not None:

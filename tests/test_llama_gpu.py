@@ -125,7 +125,7 @@ def test_a_carried_loop_runs_the_decode_steps_on_the_device(toy):
     prompt = np.random.default_rng(8).integers(0, SCALED.vocab_size, 40)
     want = toy.generate(prompt, 24)
     toy.session.forget(0)
-    ((ids,), values), = toy.session._chunks(prompt, 0)
+    ((ids,), values), = toy.session.chunk_calls(prompt, 0)
     loop = iron_amd.CarriedLoop(toy.prompt_chunk, toy.decode_step)
     assert list(loop.run(23, ids, **values)) == list(range(23))
     record = toy.decode_step.read(toy.drawn)

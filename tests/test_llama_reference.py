@@ -103,7 +103,7 @@ def test_a_token_outside_the_vocabulary_is_refused_before_any_dispatch(w, outsid
     broken[70] = outside
     with pytest.raises(IndexError, match=rf"\[{outside}\] are outside"):
         model.logits(broken)
-    np.testing.assert_array_equal(model.session._seen, tokens)
+    np.testing.assert_array_equal(model.session.cached, tokens)
 
 
 def test_a_model_runs_only_the_versions_it_loaded(w):

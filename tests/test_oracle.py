@@ -396,7 +396,7 @@ def test_sampler_draws_what_its_rows_draw():
     assert Sampler(0.0, 50).probabilities(x).argmax() == x.argmax()
     with pytest.raises(ValueError, match="not one the device draws"):
         Sampler(0.7, None).rows(1, 64)
-    with pytest.raises(ValueError, match="negative"):
+    with pytest.raises(ValueError, match="below zero"):
         Sampler(-1.0)
 
 
