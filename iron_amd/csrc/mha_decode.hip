@@ -18,6 +18,19 @@ namespace iron {
 constexpr int kMaxSplits = 128;
 constexpr int kSingleMaxKeys = 2048;  // caches up to this many rows take the one-launch kernel
 
+// 2^x for x <= 0 by the hardware's own instruction: a softmax weight small enough to be a denormal
+// counts as 0, which saves the library routine's rescaling around every call.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+typedef __bf16 bf16x2_v __attribute__((ext_vector_type(2)));
+// The dot product of two 16-byte runs of bf16.
+__device__ __forceinline__ float dot8(const uint4& a, const uint4& b) {
+  float d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, a.x), __builtin_bit_cast(bf16x2_v, b.x), 0.f, false);
+  d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, a.y), __builtin_bit_cast(bf16x2_v, b.y), d, false);
+  d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, a.z), __builtin_bit_cast(bf16x2_v, b.z), d, false);
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_v, a.w), __builtin_bit_cast(bf16x2_v, b.w), d, false);
+}
+
 // One wave's pass over key rows base + u*RW + rg for base = lo, lo + stride, ... while < hi, for
 // the G query heads q0.. of one KV head, then the merge of the wave's lane groups: on return every
 // lane holds the wave's (m, l) per head and acc = its 8 columns sub*8.. of the weighted V sum.
@@ -33,14 +46,11 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
   const int lane = threadIdx.x & 63;   // U = steps in flight
   const int sub = lane % LPR, rg = lane / LPR;
 
-  float qf[G][8];
+  // The queries stay packed bf16: a score is four two-element dot products (v_dot2c_f32_bf16: exact
+  // products, float32 sums) of a key's 16 bytes as they were loaded, scaled once at the end.
+  uint4 qp[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float t[8];
-    unpack8(*reinterpret_cast<const uint4*>(Q + (size_t)(q0 + g) * D + sub * 8), t);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) qf[g][i] = t[i] * scale_log2;
-  }
+  for (int g = 0; g < G; ++g) qp[g] = *reinterpret_cast<const uint4*>(Q + (size_t)(q0 + g) * D + sub * 8);
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     m[g] = -INFINITY;
@@ -65,13 +75,9 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
     float s[U][G];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      float kf[8];
-      unpack8(kv[u], kf);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        float d = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) d = fmaf(qf[g][i], kf[i], d);
+        float d = dot8(qp[g], kv[u]);
         if (LPR == 8) d = group8_sum(d);
         else if (LPR == 16) d = group16_sum(d);
         else {
@@ -79,7 +85,7 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
           d += __shfl_xor(d, 16, 64);
           if (LPR == 64) d += __shfl_xor(d, 32, 64);
         }
-        s[u][g] = live[u] ? d : -INFINITY;
+        s[u][g] = live[u] ? d * scale_log2 : -INFINITY;
       }
     }
 #pragma unroll
@@ -89,18 +95,23 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
       for (int u = 0; u < U; ++u) mx = fmaxf(mx, s[u][g]);
       // A lane group whose rows are all past the end keeps -inf; exp2(-inf - 0) = 0.
       const float ref = (mx == -INFINITY) ? 0.f : mx;
-      const float alpha = exp2f(m[g] - ref);
       float p[U];
       float ps = 0.f;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        p[u] = exp2f(s[u][g] - ref);
+        p[u] = fast_exp2(s[u][g] - ref);
         ps += p[u];
       }
-      l[g] = l[g] * alpha + ps;
-      m[g] = mx;
+      // The running sums are rescaled only on the steps where some lane's maximum moved: after a
+      // cache's first rows that is rare, and the rescaling is a third of a step's arithmetic.
+      if (__builtin_amdgcn_ballot_w64(mx != m[g]) != 0) {
+        const float alpha = fast_exp2(m[g] - ref);
+        l[g] *= alpha;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+        for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+      }
+      l[g] += ps;
+      m[g] = mx;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         float vf[8];
@@ -132,7 +143,7 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
   }
 }
 
-template <int D, int G>
+template <int D, int G, int U>
 __global__ __launch_bounds__(256) void mha_decode_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     float* __restrict__ part, int kv_len, float scale_log2, int window, long row_stride,
@@ -140,7 +151,10 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
   constexpr int LPR = D / 8, RW = 64 / LPR;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPR, rg = lane / LPR;
-  const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y;
+  // KV heads vary fastest over the grid: blocks that run together then read whole cache rows between
+  // them (all 1 KB of a row of 8 heads), not one head's 128 bytes of every row, which would keep a
+  // fraction of the memory channels busy and leave the rest idle.
+  const int split = blockIdx.y, nsplit = gridDim.y, kvh = blockIdx.x;
   if (kv_first) {   // the keys are a window of a longer buffer, rows *kv_first on (held inside it)
     const long first_row = max(0, min(*kv_first, kv_rows - kv_len));
     K += first_row * row_stride;
@@ -158,8 +172,8 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
   const int whi = min(min(wlo + chunk / 4, blo + chunk), kv_tokens);
 
   float m[G], l[G], acc[G][8];
-  decode_scan<D, G, 4, true>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, kvh * G, wlo, whi,
-                    4 * RW, row_stride, scale_log2, m, l, acc);
+  decode_scan<D, G, U, true>(Q, K + (size_t)kvh * head_stride, V + (size_t)kvh * head_stride, kvh * G, wlo, whi,
+                    U * RW, row_stride, scale_log2, m, l, acc);
 
   // Merge the 4 waves through LDS; wave 0 writes the block's partial.
   __shared__ float sm[4][G];
@@ -372,8 +386,15 @@ static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf1
                           int kv_heads, int kv_len, float scale_log2, int window, long row_stride,
                           long head_stride, const int* kv_valid, const int* kv_first, int kv_rows, int nsplit,
                           hipStream_t s) {
-  hipLaunchKernelGGL((mha_decode_kernel<D, G>), dim3(nsplit, kv_heads), dim3(256), 0, s, Q, K, V,
-                     part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
+  // A wave's share of its block's slice in one pass where it fits eight steps (every byte of the
+  // cache is then requested before any is needed), else four steps a pass.
+  constexpr int RW = 64 / (D / 8);
+  if (D <= 128 && G <= 4 && (kv_len + nsplit - 1) / nsplit > 4 * 4 * RW)
+    hipLaunchKernelGGL((mha_decode_kernel<D, G, 8>), dim3(kv_heads, nsplit), dim3(256), 0, s, Q, K, V,
+                       part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
+  else
+    hipLaunchKernelGGL((mha_decode_kernel<D, G, 4>), dim3(kv_heads, nsplit), dim3(256), 0, s, Q, K, V,
+                       part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
   hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D > kMaxSplits ? D : kMaxSplits), 0, s,
                      part, O, nsplit);
 }
@@ -406,6 +427,7 @@ static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, u
   // (beyond that the merge of the splits costs more than the extra parallelism gains).
   int nsplit = (kv_len + 127) / 128;
   nsplit = nsplit < 8 ? 8 : (nsplit > 64 ? 64 : nsplit);
+  if (kv_len > 64 * 256) nsplit = (kv_len + 255) / 256 > kMaxSplits ? kMaxSplits : (kv_len + 255) / 256;
   if (nsplit * 8 > kv_len) nsplit = kv_len >= 8 ? kv_len / 8 : 1;
   const float scale_log2 = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
