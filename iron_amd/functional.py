@@ -1,7 +1,8 @@
-"""Functions for a graph's body, under ``torch.nn.functional``'s names (iron/functional.py:30-129).
+"""``torch.nn.functional``-style recorders for a graph's body (the reference's iron/functional.py:30-129).
 
-Each records the operator steps that compute it and returns their handle.  Weights are a
-checkpoint's ``(out, in)``, as ``torch.nn.Linear`` stores them.
+Calling one of these inside a body appends the operator step(s) that compute it and hands back the
+result's handle.  Matrices are ``(out_features, in_features)``, the way ``torch.nn.Linear`` and every
+checkpoint store them, so both GEMV and GEMM read a weight row as one contiguous run of K.
 """
 
 from __future__ import annotations
@@ -15,56 +16,61 @@ from .operators.rms_norm import RMSNorm
 from .operators.rope import RoPE
 from .operators.silu import SiLU
 
-BF16_EPS = 2.0**-7  # bfloat16's machine epsilon
+BF16_EPS = 2.0**-7   # machine epsilon of bfloat16 (8 significand bits), the default norm epsilon
 
 
 def linear(x, weight, bias=None, *, precision: Precision = Precision.HIGHEST, **gemv):
-    """Return ``x @ weight.T``, plus ``bias`` on every row if given.
+    """``x @ weight.T (+ bias)``.
 
-    One row runs on GEMV, which always rounds once in float32; several rows run on the MFMA
-    GEMM reading the weight as stored (``b_col_maj``) -- at every ``precision`` the same
-    kernel: f32 partial sums, one rounding (the reference's flm.ProjectionGEMM at
-    MEDIUM/HIGH has no counterpart here).
+    Dispatch by row count: a single row (``(in,)`` or ``(1, in)``) records the bandwidth-bound
+    ``GEMV``, anything taller the MFMA ``GEMM`` with ``b_col_maj`` (the weight as stored).  Both
+    accumulate in float32 and round once whatever ``precision`` says: the reference's reduced-precision
+    projection kernels have no equivalent here, the field is only carried.  ``gemv`` passes tunables
+    to the single-row case.
 
     Raises:
-        ValueError: ``x`` of another rank, or GEMV tunables for several rows.
+        ValueError: ``x`` is neither a vector nor a matrix; or GEMV tunables came with several rows.
     """
-    if len(x.shape) not in (1, 2):
+    rank = len(x.shape)
+    if rank not in (1, 2):
         raise ValueError(f"linear(): x {tuple(x.shape)} is not (in,) or (rows, in)")
-    one_row = len(x.shape) == 1 or x.shape[0] == 1
-    if one_row:
-        y = GEMV.step(weight, x, **gemv)
-    elif gemv:
-        raise ValueError(f"linear(): {x.shape[0]} rows take no GEMV {sorted(gemv)}")
+    rows = 1 if rank == 1 else x.shape[0]
+    if rows > 1 and gemv:
+        raise ValueError(f"linear(): {rows} rows take no GEMV {sorted(gemv)}")
+    if rows == 1:
+        product = GEMV.step(weight, x, **gemv)
     else:
-        y = GEMM.step(x, weight, b_col_maj=True, precision=precision)
+        product = GEMM.step(x, weight, b_col_maj=True, precision=precision)
     if bias is None:
-        return y
-    # A row added to every row, also for GEMV's one-dimensional output.
-    rows = math.prod(y.shape) // bias.shape[0]
-    return (y.reshape(rows, bias.shape[0]) + bias).reshape(y.shape)
-
-
-def _last_axis(name: str, x, normalized_shape) -> None:
-    given = (normalized_shape,) if isinstance(normalized_shape, int) else tuple(normalized_shape)
-    if given != tuple(x.shape[-1:]):
-        raise ValueError(f"{name}(): normalized_shape {list(given)} is not the last axis of input "
-                         f"{list(x.shape)}; only ({x.shape[-1]},) is normalized")
+        return product
+    # Broadcast the bias over rows; a GEMV's flat output is viewed as one row for the purpose.
+    width = bias.shape[0]
+    as_rows = product.reshape(math.prod(product.shape) // width, width)
+    return (as_rows + bias).reshape(product.shape)
 
 
 def rms_norm(x, normalized_shape, weight=None, eps: float | None = None):
-    """``x`` over the RMS of its last axis, times ``weight`` if given; ``eps`` None is bf16's epsilon."""
-    _last_axis("rms_norm", x, normalized_shape)
-    if eps is None:
-        eps = BF16_EPS
-    return RMSNorm.step(x, weight=weight, epsilon=eps)
+    """RMS normalisation over the last axis (``normalized_shape`` must name exactly that axis),
+    scaled by ``weight`` when given.  ``eps=None`` means bfloat16's machine epsilon, as torch picks
+    the dtype's.
+
+    Raises:
+        ValueError: ``normalized_shape`` is not ``x``'s last axis.
+    """
+    wanted = (normalized_shape,) if isinstance(normalized_shape, int) else tuple(normalized_shape)
+    last = tuple(x.shape[-1:])
+    if wanted != last:
+        raise ValueError(f"rms_norm(): normalized_shape {list(wanted)} is not the last axis of input "
+                         f"{list(x.shape)}; only ({x.shape[-1]},) is normalized")
+    return RMSNorm.step(x, weight=weight, epsilon=BF16_EPS if eps is None else eps)
 
 
 def silu(x):
-    """Apply SiLU, ``x * sigmoid(x)``, as torch's."""
+    """``x * sigmoid(x)`` elementwise."""
     return SiLU.step(x)
 
 
 def rope(x, angles):
-    """``x`` ``(rows, head_dim)`` turned by RoPE, a row of ``angles`` per row."""
+    """Rotate the rows of ``x`` (``(rows, head_dim)``, two-halves convention) by ``angles``, whose
+    rows are spread evenly over ``x``'s."""
     return RoPE.step(x, angles)

@@ -1,7 +1,8 @@
-"""A decoder's shape (``DecoderConfig``) and its RoPE table (``rope_angles``).
+"""The numbers that define a decoder (``DecoderConfig``) and the rotary table they imply
+(``rope_angles``).
 
-Field names are a Hugging Face checkpoint's ``config.json``'s where it has one
-(iron/lm/config.py:23-42,184-267).
+Fields carry the names of a Hugging Face ``config.json`` wherever that file has the notion, so a
+config can be read from and written to one; the interface follows iron/lm/config.py:23-42,184-267.
 """
 
 from __future__ import annotations
@@ -17,29 +18,39 @@ from ..common.declare import Precision
 
 RopeScaling = Callable[[np.ndarray], np.ndarray]
 
+_ACTIVATIONS = ("silu", "gelu_pytorch_tanh", "gelu")
+
 
 def rope_angles(head_dim: int, context_length: int, rope_theta: float = 500000.0,
                 scaling: RopeScaling | None = None) -> np.ndarray:
-    """Return the RoPE table, ``(context_length, head_dim)`` float32, cos and sin interleaved.
+    """The rotary table: float32 ``(context_length, head_dim)``; column ``2i`` holds
+    ``cos(p * f_i)`` and column ``2i + 1`` holds ``sin(p * f_i)`` for position ``p``.
 
-    The frequency and the position are float32, their product float32; each transcendental
-    is evaluated in float64 and rounded once.
+    Precision recipe (it fixes the table bit for bit, so it is part of the contract): the exponent
+    ``2i / head_dim`` is float32; ``f_i = theta ** -exponent`` is evaluated in float64, passed through
+    ``scaling`` if any, then rounded to float32; ``p * f_i`` is a float32 product; cos and sin are
+    taken in float64 and rounded to float32 once.
     """
-    exponents = np.arange(0, head_dim, 2, dtype=np.float32) / np.float32(head_dim)
-    inv_freq = 1.0 / np.power(rope_theta, exponents.astype(np.float64))
+    pair = np.arange(head_dim // 2 + head_dim % 2, dtype=np.float32) * np.float32(2)
+    exponent = (pair / np.float32(head_dim)).astype(np.float64)
+    frequency = np.reciprocal(np.power(rope_theta, exponent))
     if scaling is not None:
-        inv_freq = scaling(inv_freq)
-    inv_freq = inv_freq.astype(np.float32)
-    freqs = np.outer(np.arange(context_length, dtype=np.float32), inv_freq)
-    angles = np.empty((context_length, head_dim), dtype=np.float32)
-    angles[:, ::2] = np.cos(freqs.astype(np.float64))
-    angles[:, 1::2] = np.sin(freqs.astype(np.float64))
-    return angles
+        frequency = scaling(frequency)
+    frequency = frequency.astype(np.float32)
+    position = np.arange(context_length, dtype=np.float32)
+    phase = (position[:, None] * frequency[None, :]).astype(np.float64)
+    table = np.stack((np.cos(phase), np.sin(phase)), axis=-1)
+    return table.reshape(context_length, -1)[:, :head_dim].astype(np.float32)
+
+
+def _required(field: dataclasses.Field) -> bool:
+    return field.default is dataclasses.MISSING and field.default_factory is dataclasses.MISSING
 
 
 @dataclasses.dataclass(frozen=True)
 class DecoderConfig:
-    """A decoder's shape. ``max_seq_len`` is the checkpoint's native context unless a caller lowers it."""
+    """Shape and options of a decoder.  ``max_seq_len`` starts as the checkpoint's native context
+    and is usually lowered by the caller (it sizes the KV caches and the rotary table)."""
 
     vocab_size: int
     hidden_size: int
@@ -60,88 +71,96 @@ class DecoderConfig:
     mlp_bias: bool = False
     sliding_window: int | None = None
 
-    # Where a checkpoint's config.json holds a field, where that is not the field's own name; None:
-    # nowhere -- a choice of this package, kept at its default by ``from_checkpoint`` and left out
-    # by ``to_json`` (iron/lm/config.py:68-183).
+    # field -> its key in config.json when that differs from the field's name.  None marks a field
+    # that is this package's own choice: never read from a checkpoint, never written to one.
     JSON = {"eps": "rms_norm_eps", "max_seq_len": "max_position_embeddings", "precision": None,
             "prefill_chunk": None}
 
+    def __post_init__(self):
+        fix = object.__setattr__           # the dataclass is frozen; these two are derived defaults
+        if self.head_dim is None:
+            fix(self, "head_dim", self.hidden_size // self.num_attention_heads)
+        if self.prefill_chunk > self.max_seq_len:
+            fix(self, "prefill_chunk", self.max_seq_len)
+        if self.hidden_act not in _ACTIVATIONS:
+            raise ValueError(f"{type(self).__name__}: hidden_act {self.hidden_act!r}: no operator here computes it")
+
+    # -- config.json in and out
+    @classmethod
+    def _json_key(cls, name: str) -> str | None:
+        return cls.JSON[name] if name in cls.JSON else name
+
     @classmethod
     def from_checkpoint(cls, path):
-        """The fields read from ``path``'s ``config.json``: ``path`` is that file, or a checkpoint's
-        directory or one of its files.
+        """Read ``config.json`` given that file, the checkpoint directory, or any file in it.
 
         Raises:
-            FileNotFoundError: no ``config.json`` is there.
-            ValueError: the file lacks a field that has no default.
+            FileNotFoundError: there is no ``config.json`` there.
+            ValueError: a field without a default is absent from it.
         """
-        path = Path(path)
-        if path.name != "config.json":
-            path = (path if path.is_dir() else path.parent) / "config.json"
-        return cls.from_json(json.loads(path.read_text()), path)
+        where = Path(path)
+        if where.name != "config.json":
+            where = (where if where.is_dir() else where.parent) / "config.json"
+        with open(where) as handle:
+            return cls.from_json(json.load(handle), where)
 
     @classmethod
     def from_json(cls, data: dict, source="config.json"):
-        """``from_checkpoint`` on ``data``, a ``config.json`` already parsed; ``source`` names it in an error."""
-        kwargs, missing = {}, []
-        for f in dataclasses.fields(cls):
-            key = cls.JSON.get(f.name, f.name)
+        """Build from an already parsed ``config.json``; ``source`` only labels error messages.
+        Hugging Face writes ``null`` for options left unset, which reads the same as absent."""
+        given, absent = {}, []
+        for field in dataclasses.fields(cls):
+            key = cls._json_key(field.name)
             if key is None:
                 continue
-            value = data.get(key)
-            if value is None:  # absent, or Hugging Face's null for an unset option
-                if f.default is dataclasses.MISSING and f.default_factory is dataclasses.MISSING:
-                    missing.append(key)
-                continue
-            kwargs[f.name] = cls.convert(f.name, value)
-        if missing:
-            raise ValueError(f"{source} lacks {missing}")
-        return cls(**kwargs)
+            raw = data.get(key)
+            if raw is not None:
+                given[field.name] = cls.convert(field.name, raw)
+            elif _required(field):
+                absent.append(key)
+        if absent:
+            raise ValueError(f"{source} lacks {absent}")
+        return cls(**given)
 
     @classmethod
     def convert(cls, name: str, value):
-        """A ``config.json`` value as the field holds it."""
-        if name == "rope_scaling":
-            kind = value.get("rope_type", value.get("type"))
-            if kind != "default":
-                raise ValueError(f"rope_scaling {value}: no RoPE table here builds it")
+        """Hook: a raw ``config.json`` value -> what the field stores.  The base class understands
+        only the trivial rotary scaling."""
+        if name != "rope_scaling":
+            return value
+        kind = value.get("rope_type", value.get("type"))
+        if kind == "default":
             return None
-        return value
+        raise ValueError(f"rope_scaling {value}: no RoPE table here builds it")
 
     def to_json(self) -> dict:
-        """The fields as ``config.json`` names them: ``from_json``'s inverse."""
+        """The inverse of ``from_json``: plain JSON values under ``config.json``'s keys."""
+        plain = (bool, int, float, str, tuple, dict)
         out = {}
-        for f in dataclasses.fields(self):
-            key = self.JSON.get(f.name, f.name)
-            value = getattr(self, f.name)
+        for field in dataclasses.fields(self):
+            key, value = self._json_key(field.name), getattr(self, field.name)
+            if key is None:
+                continue
             if dataclasses.is_dataclass(value) and not isinstance(value, type):
                 value = dataclasses.asdict(value)
-            if key is None or not isinstance(value, (bool, int, float, str, tuple, dict)):
-                continue
-            out[key] = list(value) if isinstance(value, tuple) else value
+            if isinstance(value, plain):
+                out[key] = list(value) if isinstance(value, tuple) else value
         return out
 
-    def __post_init__(self):
-        if self.head_dim is None:
-            object.__setattr__(self, "head_dim", self.hidden_size // self.num_attention_heads)
-        if self.prefill_chunk > self.max_seq_len:
-            object.__setattr__(self, "prefill_chunk", self.max_seq_len)
-        if self.hidden_act not in ("silu", "gelu_pytorch_tanh", "gelu"):
-            raise ValueError(f"{type(self).__name__}: hidden_act {self.hidden_act!r}: no operator here computes it")
-
+    # -- derived quantities
     @property
     def window(self) -> int | None:
-        """The positions before a query each layer attends to, ``sliding_window`` less the query's own."""
-        if self.sliding_window is None or self.sliding_window >= self.max_seq_len:
-            return None
-        return self.sliding_window - 1
+        """Earlier positions a query may see (its own excluded), or None when attention is global or
+        the window covers the whole context anyway."""
+        span = self.sliding_window
+        return None if span is None or span >= self.max_seq_len else span - 1
 
     @property
     def rope_width(self) -> int:
         return self.head_dim
 
     def angles(self) -> np.ndarray | None:
-        """The RoPE table, a row per position; None with no ``rope_theta``."""
+        """This config's rotary table (a row per position), or None for a model without RoPE."""
         if self.rope_theta is None:
             return None
         return rope_angles(self.rope_width, self.max_seq_len, self.rope_theta, self.rope_scaling)
