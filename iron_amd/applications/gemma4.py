@@ -1,13 +1,20 @@
-"""Gemma 4's text decoder on the shared decoder (iron/applications/gemma4/model.py:42-246).
+"""The text decoder of Gemma 4 (interface of iron/applications/gemma4/model.py:42-246).
 
-Sliding-window and global layers alternate as ``layer_types`` says; a global layer has its own
-head size and a RoPE that turns only the first quarter of its pairs; q, k and v are RMS-normed per
-head and attention is unscaled; every block's output is normed again before its residual
-(``SandwichLayer``); the last ``num_kv_shared_layers`` layers attend over an earlier layer's cache
-and may have a double-wide MLP; every layer gates in a per-layer input made of the token's own
-row of a per-layer table and a projection of the embeddings (``PleLayer``); the logits are capped
-by a tanh.  The vision and audio towers are not built: a multimodal checkpoint's text decoder
-loads from its ``model.language_model`` tensors.
+What sets it apart from the plain decoder, and where each piece lives:
+
+* layers are "sliding_attention" or "full_attention" by ``layer_types``.  Global layers have wider
+  heads (``global_head_dim``) and their own rotary table, of which only the first
+  ``partial_rotary_factor`` of the pairs turn -- the rest get frequency 0, i.e. the identity;
+* q, k and v are RMS-normed per head and the scores are not scaled (``Gemma4Layer``);
+* each block's output is normed before it joins the residual (``SandwichLayer``);
+* the last ``num_kv_shared_layers`` layers own no cache: they read the cache of the last earlier
+  layer of their kind, and may have a feed-forward twice as wide;
+* every layer adds a "per-layer input": the token's row of a per-layer table plus a projection of
+  the embeddings, gated into the hidden state (``PleLayer``);
+* the logits may be soft-capped with a tanh.
+
+Vision and audio towers are out of scope; a multimodal checkpoint's language model loads from the
+tensors under ``model.language_model``.
 """
 
 from __future__ import annotations
@@ -28,39 +35,46 @@ from ..operators.tanh import Tanh
 
 PREFIX = "model.language_model."
 
+_GLOBAL, _SLIDING = "full_attention", "sliding_attention"
 
-def _dig(data: dict, path: str):
-    for key in path.split("."):
-        if not isinstance(data, dict) or key not in data:
+
+def _walk(tree, dotted: str):
+    """``tree["a"]["b"]`` for ``"a.b"``, or None as soon as a level is missing."""
+    node = tree
+    for part in dotted.split("."):
+        node = node.get(part) if isinstance(node, dict) else None
+        if node is None:
             return None
-        data = data[key]
-    return data
+    return node
+
+
+def _kw(default=dataclasses.MISSING):
+    return dataclasses.field(kw_only=True) if default is dataclasses.MISSING else dataclasses.field(default=default, kw_only=True)
 
 
 @dataclasses.dataclass(frozen=True)
 class Gemma4Config(DecoderConfig):
-    """``DecoderConfig`` as a checkpoint's ``text_config`` holds it, with the global layers' heads
-    and RoPE, the shared caches, the per-layer inputs and the logits' cap."""
+    """The decoder's config as a Gemma 4 ``config.json`` spells it: most fields sit under
+    ``text_config`` (some nested deeper), the multimodal placeholder ids at the top level."""
 
-    precision: Precision = dataclasses.field(default=Precision.MEDIUM, kw_only=True)
+    precision: Precision = _kw(Precision.MEDIUM)
     hidden_act: str = "gelu_pytorch_tanh"
-    layer_types: tuple[str, ...] = dataclasses.field(kw_only=True)
-    global_head_dim: int = dataclasses.field(default=512, kw_only=True)
-    global_rope_theta: float = dataclasses.field(default=1000000.0, kw_only=True)
-    partial_rotary_factor: float = dataclasses.field(default=0.25, kw_only=True)
-    num_kv_shared_layers: int = dataclasses.field(default=0, kw_only=True)
-    use_double_wide_mlp: bool = dataclasses.field(default=False, kw_only=True)
-    ple_dim: int = dataclasses.field(default=256, kw_only=True)
-    final_logit_softcapping: float | None = dataclasses.field(default=None, kw_only=True)
-    # The placeholders a tower's soft tokens would replace, which the per-layer inputs read as the
-    # padding token.
-    pad_token_id: int = dataclasses.field(default=0, kw_only=True)
-    image_token_id: int | None = dataclasses.field(default=None, kw_only=True)
-    audio_token_id: int | None = dataclasses.field(default=None, kw_only=True)
-    video_token_id: int | None = dataclasses.field(default=None, kw_only=True)
+    layer_types: tuple[str, ...] = _kw()
+    global_head_dim: int = _kw(512)
+    global_rope_theta: float = _kw(1000000.0)
+    partial_rotary_factor: float = _kw(0.25)
+    num_kv_shared_layers: int = _kw(0)
+    use_double_wide_mlp: bool = _kw(False)
+    ple_dim: int = _kw(256)
+    final_logit_softcapping: float | None = _kw(None)
+    # Ids that stand for image / audio / video soft tokens.  Without towers they can only be treated
+    # as padding by the per-layer table, which is what the full model does with them too.
+    pad_token_id: int = _kw(0)
+    image_token_id: int | None = _kw(None)
+    audio_token_id: int | None = _kw(None)
+    video_token_id: int | None = _kw(None)
 
-    # Where ``text_config`` holds a field under another name or deeper; a leading "/" is the file's
-    # top level.
+    # field -> where config.json keeps it, relative to text_config; "/" in front = top level instead
     PATHS = {
         "eps": "rms_norm_eps", "max_seq_len": "max_position_embeddings", "hidden_act": "hidden_activation",
         "rope_theta": "rope_parameters.sliding_attention.rope_theta",
@@ -69,229 +83,253 @@ class Gemma4Config(DecoderConfig):
         "ple_dim": "hidden_size_per_layer_input",
         "image_token_id": "/image_token_id", "audio_token_id": "/audio_token_id", "video_token_id": "/video_token_id",
     }
-    NOT_JSON = ("precision", "prefill_chunk", "rope_scaling")
+    NOT_JSON = ("precision", "prefill_chunk", "rope_scaling")     # this package's own knobs
+
+    @classmethod
+    def _unsupported(cls, text: dict) -> str | None:
+        """The first thing ``text_config`` asks for that this decoder does not implement, if any."""
+        for flag in ("attention_k_eq_v", "enable_moe_block", "attn_logit_softcapping"):
+            if text.get(flag):
+                return f"{flag} {text[flag]!r}"
+        # "vision" limits bidirectional attention to image tokens, of which text has none
+        both_ways = text.get("use_bidirectional_attention")
+        if both_ways not in (None, False, "vision"):
+            return f"bidirectional attention {both_ways!r}"
+        vocab = text.get("vocab_size")
+        table_vocab = text.get("vocab_size_per_layer_input", vocab)
+        if table_vocab != vocab:
+            return f"vocab_size_per_layer_input {table_vocab} other than vocab_size {vocab}"
+        ropes = text.get("rope_parameters", {})
+        for kind, expected in ((_SLIDING, "default"), (_GLOBAL, "proportional")):
+            declared = ropes.get(kind, {}).get("rope_type", expected)
+            if declared != expected:
+                return f"{kind} RoPE {declared!r}"
+        return None
 
     @classmethod
     def from_json(cls, data: dict, source="config.json") -> "Gemma4Config":
-        """The fields of a parsed ``config.json`` (iron/applications/gemma4/model.py:89-125).
+        """Parse a ``config.json`` (iron/applications/gemma4/model.py:89-125).
 
         Raises:
-            ValueError: the file asks for what is not built here (keys equal to values, experts, an
-                attention soft-cap, bidirectional text, a per-layer vocabulary other than the
-                embedding's, RoPE other than the sliding layers' default and the global ones'
-                proportional), or lacks a field that has no default.
+            ValueError: it asks for a variant not built here (keys tied to values, experts, capped
+                attention scores, bidirectional text, a per-layer vocabulary of its own, other RoPE
+                kinds), or a field without a default is missing.
         """
         text = dict(data.get("text_config", {}))
-        for key in ("attention_k_eq_v", "enable_moe_block", "attn_logit_softcapping"):
-            if text.get(key):
-                raise ValueError(f"{source}: {key} {text[key]!r} is not built here")
-        # "vision" makes only image tokens bidirectional; text has none.
-        bidirectional = text.get("use_bidirectional_attention")
-        if bidirectional not in (None, False, "vision"):
-            raise ValueError(f"{source}: bidirectional attention {bidirectional!r} is not built here")
-        per_layer = text.get("vocab_size_per_layer_input", text.get("vocab_size"))
-        if per_layer != text.get("vocab_size"):
-            raise ValueError(f"{source}: vocab_size_per_layer_input {per_layer} other than vocab_size "
-                             f"{text.get('vocab_size')} is not built here")
-        rope = text.get("rope_parameters", {})
-        for kind, built in (("sliding_attention", "default"), ("full_attention", "proportional")):
-            got = rope.get(kind, {}).get("rope_type", built)
-            if got != built:
-                raise ValueError(f"{source}: {kind} RoPE {got!r} is not built here")
-        kwargs, missing = {}, []
-        for f in dataclasses.fields(cls):
-            if f.name in cls.NOT_JSON:
+        problem = cls._unsupported(text)
+        if problem is not None:
+            raise ValueError(f"{source}: {problem} is not built here")
+        found, absent = {}, []
+        for field in dataclasses.fields(cls):
+            if field.name in cls.NOT_JSON:
                 continue
-            path = cls.PATHS.get(f.name, f.name)
-            value = _dig(data, path[1:]) if path.startswith("/") else _dig(text, path)
-            if value is None:
-                if f.default is dataclasses.MISSING and f.default_factory is dataclasses.MISSING:
-                    missing.append(path)
-                continue
-            kwargs[f.name] = tuple(value) if f.name == "layer_types" else value
-        if missing:
-            raise ValueError(f"{source} lacks {missing}")
-        return cls(**kwargs)
+            where = cls.PATHS.get(field.name, field.name)
+            value = _walk(data, where[1:]) if where[0] == "/" else _walk(text, where)
+            if value is not None:
+                found[field.name] = tuple(value) if field.name == "layer_types" else value
+            elif field.default is dataclasses.MISSING and field.default_factory is dataclasses.MISSING:
+                absent.append(where)
+        if absent:
+            raise ValueError(f"{source} lacks {absent}")
+        return cls(**found)
 
     def to_json(self) -> dict:
-        """``from_json``'s inverse: the fields under ``text_config`` (or the top level) where a
-        checkpoint's ``config.json`` holds them."""
-        out: dict = {"text_config": {}}
-        for f in dataclasses.fields(self):
-            value = getattr(self, f.name)
-            if f.name in self.NOT_JSON or value is None:
+        """Back to ``config.json``'s layout: ``from_json(to_json())`` reproduces the config."""
+        document: dict = {"text_config": {}}
+        for field in dataclasses.fields(self):
+            value = getattr(self, field.name)
+            if value is None or field.name in self.NOT_JSON:
                 continue
-            path = self.PATHS.get(f.name, f.name)
-            at = out if path.startswith("/") else out["text_config"]
-            *parents, leaf = path.lstrip("/").split(".")
-            for key in parents:
-                at = at.setdefault(key, {})
-            at[leaf] = list(value) if isinstance(value, tuple) else value
-        return out
+            where = self.PATHS.get(field.name, field.name)
+            scope = document if where[0] == "/" else document["text_config"]
+            keys = where.lstrip("/").split(".")
+            for key in keys[:-1]:
+                scope = scope.setdefault(key, {})
+            scope[keys[-1]] = list(value) if isinstance(value, tuple) else value
+        return document
 
     def full(self, i: int) -> bool:
-        """Whether layer ``i`` is global."""
-        return self.layer_types[i] == "full_attention"
+        """True for a global ("full_attention") layer."""
+        return self.layer_types[i] == _GLOBAL
 
     def owner(self, i: int) -> int:
-        """The layer whose cache layer ``i`` attends over: its own, or for a shared layer the last
-        one of its kind before the shared ones."""
-        first = self.num_hidden_layers - self.num_kv_shared_layers
-        if i < first:
+        """Index of the layer whose KV cache layer ``i`` reads: itself, unless ``i`` is one of the
+        trailing shared layers -- then the last non-shared layer of the same kind.
+
+        Raises:
+            ValueError: a shared layer with no earlier layer of its kind.
+        """
+        own_caches = self.num_hidden_layers - self.num_kv_shared_layers
+        if i < own_caches:
             return i
-        owners = [j for j in range(first) if self.full(j) == self.full(i)]
-        if not owners:
-            raise ValueError(f"Gemma4Config: shared layer {i} has no earlier layer of its kind")
-        return owners[-1]
+        for j in range(own_caches - 1, -1, -1):
+            if self.full(j) == self.full(i):
+                return j
+        raise ValueError(f"Gemma4Config: shared layer {i} has no earlier layer of its kind")
 
 
 class Gemma4Decoder(Decoder):
-    """``Decoder`` and the per-layer inputs' token table, projection and norm."""
+    """The trunk plus what the per-layer inputs need: one wide token table (all layers' columns side
+    by side, as the checkpoint stores it), the projection of the embeddings, and its norm."""
 
     def __init__(self, c: Gemma4Config, layer):
         super().__init__(c, layer)
-        L, P, E = c.num_hidden_layers, c.ple_dim, c.hidden_size
-        # Dropped once the loaded table has been split into the layers'.
-        self.embed_tokens_per_layer = Embedding(c.vocab_size, L * P)
-        self.per_layer_model_projection = Linear(E, L * P, False, precision=c.precision)
-        self.per_layer_projection_norm = RMSNorm(P, c.eps)
+        all_layers = c.num_hidden_layers * c.ple_dim
+        # only a loading vehicle: split into per-layer tables and dropped in load_state_dict
+        self.embed_tokens_per_layer = Embedding(c.vocab_size, all_layers)
+        self.per_layer_model_projection = Linear(c.hidden_size, all_layers, False, precision=c.precision)
+        self.per_layer_projection_norm = RMSNorm(c.ple_dim, c.eps)
 
 
 class Gemma4Layer(PleLayer):
-    """Layer ``i``: unscaled attention over normed q, k and v -- a global layer's heads and whole
-    context where it is one, else within the window -- and a double-wide MLP on a shared layer
-    where ``use_double_wide_mlp``."""
+    """One Gemma 4 layer: per-head norms on q, k, v; scores used as they are (scale 1); global
+    layers with their own head width over the whole context, sliding ones within the window; a
+    shared layer optionally with the double-width feed-forward."""
 
     def __init__(self, c: Gemma4Config, i: int):
-        heads = dataclasses.replace(c, head_dim=c.global_head_dim) if c.full(i) else c
-        mlp = None
-        if c.use_double_wide_mlp and c.owner(i) != i:
-            mlp = GatedMLP(dataclasses.replace(c, intermediate_size=2 * c.intermediate_size))
-        super().__init__(c, i, Attention(heads, i, norms="qkv"), mlp, KVCache(heads, None if c.full(i) else c.window))
+        is_global, shared = c.full(i), c.owner(i) != i
+        head_config = dataclasses.replace(c, head_dim=c.global_head_dim) if is_global else c
+        wide_mlp = None
+        if shared and c.use_double_wide_mlp:
+            wide_mlp = GatedMLP(dataclasses.replace(c, intermediate_size=2 * c.intermediate_size))
+        cache = KVCache(head_config, None if is_global else c.window)
+        super().__init__(c, i, Attention(head_config, i, norms="qkv"), wide_mlp, cache)
         self.self_attn.scaling = 1.0
 
 
-def _host_array(array) -> np.ndarray:
-    """A loaded weight as a float32 array of bf16 values (a checkpoint hands over torch tensors)."""
-    if type(array).__module__.startswith("torch"):
-        return from_torch(array)
-    return np.asarray(array, dtype=np.float32)
+def _as_float32(weight) -> np.ndarray:
+    """float32 values of a loaded weight (numpy, or a torch bf16 tensor from a checkpoint)."""
+    if type(weight).__module__.split(".")[0] == "torch":
+        return from_torch(weight)
+    return np.asarray(weight, dtype=np.float32)
 
 
 class _StillPairs:
-    """Proportional RoPE: the pairs past ``turned`` stand still (frequency zero)."""
+    """The "proportional" RoPE of global layers as a frequency scaling: pairs from ``turned`` on get
+    frequency 0 and therefore never rotate."""
 
     def __init__(self, turned: int):
         self.turned = turned
 
     def __call__(self, inv_freq: np.ndarray) -> np.ndarray:
-        return np.where(np.arange(inv_freq.size) < self.turned, inv_freq, 0)
+        keep = np.arange(inv_freq.size) < self.turned
+        return np.where(keep, inv_freq, 0)
+
+
+def _drop_kv(attention) -> None:
+    attention.k_proj = attention.v_proj = attention.k_norm = None
 
 
 class Gemma4(CausalLM):
-    """Gemma 4's text decoder on ``config``'s shape and a checkpoint's ``weights`` (by tensor name;
-    the decoder's are under ``model.language_model``, the towers' are left out)."""
+    """Gemma 4's language model from a config and a checkpoint's tensors by name (those under
+    ``model.language_model`` are used, plus an untied ``lm_head`` if present; towers are ignored)."""
 
     config_class = Gemma4Config
     decoder_class = Gemma4Decoder
     layer_class = Gemma4Layer
 
     def __init__(self, config: Gemma4Config, weights):
-        text = {"model." + name[len(PREFIX):]: t for name, t in weights.items() if name.startswith(PREFIX)}
+        own = {"model." + name.removeprefix(PREFIX): tensor for name, tensor in weights.items()
+               if name.startswith(PREFIX)}
         if "lm_head.weight" in weights:
-            text["lm_head.weight"] = weights["lm_head.weight"]
-        super().__init__(config, text)
+            own["lm_head.weight"] = weights["lm_head.weight"]
+        super().__init__(config, own)
         c = config
-        turned = int(c.partial_rotary_factor * c.global_head_dim // 2)
-        rope = Rope(dataclasses.replace(c, head_dim=c.global_head_dim, rope_theta=c.global_rope_theta,
-                                        rope_scaling=_StillPairs(turned)))
-        for i, layer in enumerate(self.layers):
+        turning_pairs = int(c.partial_rotary_factor * c.global_head_dim // 2)
+        global_rope = Rope(dataclasses.replace(c, head_dim=c.global_head_dim, rope_theta=c.global_rope_theta,
+                                               rope_scaling=_StillPairs(turning_pairs)))
+        for i, block in enumerate(self.layers):
             if c.full(i):
-                layer.rope = rope
-            if c.owner(i) != i:
-                attention = layer.self_attn
-                attention.k_proj = attention.v_proj = attention.k_norm = None
-                layer.cache = self.layers[c.owner(i)].cache
+                block.rope = global_rope
+            source = c.owner(i)
+            if source != i:
+                _drop_kv(block.self_attn)
+                block.cache = self.layers[source].cache
 
     def load_state_dict(self, tree, *, path: str = "") -> None:
-        c, m = self.config, self.model
-        # A shared layer's k/v projections and k norm are never read: a checkpoint that ships them
-        # loads them (they are dropped once the caches are shared), one that does not need not.
-        for i, layer in enumerate(m.layers):
-            if c.owner(i) != i and f"{path}model.layers.{i}.self_attn.k_proj.weight" not in tree:
-                layer.self_attn.k_proj = layer.self_attn.v_proj = layer.self_attn.k_norm = None
+        c, trunk = self.config, self.model
+        # Checkpoints differ on whether shared layers still carry k/v weights they never use.  If
+        # they do, load them (they are dropped when the caches are wired up); if not, do not ask.
+        for i, block in enumerate(trunk.layers):
+            unused = c.owner(i) != i
+            if unused and f"{path}model.layers.{i}.self_attn.k_proj.weight" not in tree:
+                _drop_kv(block.self_attn)
         super().load_state_dict(tree, path=path)
-        P, E = c.ple_dim, c.hidden_size
-        scale = round_bf16(np.float32(np.sqrt(P)))
-        table = _host_array(m.embed_tokens_per_layer.weight.array)
-        placeholders = [t for t in (c.image_token_id, c.audio_token_id, c.video_token_id) if t is not None]
-        for i, layer in enumerate(m.layers):
-            # A layer's own columns, scaled, contiguous: one gather a layer.
-            rows = table[:, i * P : (i + 1) * P] * scale
-            rows[placeholders] = rows[c.pad_token_id]
-            layer.per_layer_embedding = iron.param(round_bf16(rows))
-            # The row every row of the layer's output is multiplied by.
-            scalar = _host_array(layer.layer_scalar.array)
-            layer.scale = iron.param(round_bf16(np.full(E, scalar[0], np.float32)))
-        m.embed_tokens_per_layer = None
+        width, hidden = c.ple_dim, c.hidden_size
+        gain = round_bf16(np.float32(np.sqrt(width)))
+        wide_table = _as_float32(trunk.embed_tokens_per_layer.weight.array)
+        soft_tokens = [t for t in (c.image_token_id, c.audio_token_id, c.video_token_id) if t is not None]
+        for i, block in enumerate(trunk.layers):
+            # this layer's columns, pre-scaled and contiguous, so a call gathers one row per token
+            table = wide_table[:, i * width : (i + 1) * width] * gain
+            table[soft_tokens] = table[c.pad_token_id]
+            block.per_layer_embedding = iron.param(round_bf16(table))
+            # layer_scalar as a constant row the layer's output is multiplied by
+            scalar = _as_float32(block.layer_scalar.array)[0]
+            block.scale = iron.param(round_bf16(np.full(hidden, scalar, dtype=np.float32)))
+        trunk.embed_tokens_per_layer = None
 
     def lookup(self, ids):
-        # The embedding times sqrt(hidden_size), a constant row in the weights' dtype.
+        """Embedding rows times sqrt(hidden_size) (recorded as a multiply by a constant row)."""
         return super().lookup(ids) * float(np.sqrt(self.config.hidden_size))
 
     def layer(self, call, i, w, x):
-        """Layer ``i`` on ``x``, its per-layer input made from the call's embeddings and ids."""
-        c, m, P = self.config, self.model, self.config.ple_dim
-        projection = m.per_layer_model_projection.weight[i * P : (i + 1) * P]
-        ple = F.linear(call.embeddings, projection, precision=c.precision)
+        """Layer ``i`` with its per-layer input: (projection of the embeddings, normed, plus the
+        token's table row) / sqrt(2)."""
+        c, trunk = self.config, self.model
+        width = c.ple_dim
+        columns = trunk.per_layer_model_projection.weight[i * width : (i + 1) * width]
+        projected = F.linear(call.embeddings, columns, precision=c.precision)
         rows = call.embeddings.elements // c.hidden_size
-        # The projection's hidden_size ** -0.5 folded into the norm's epsilon:
-        # RMSNorm(s * y, eps) is RMSNorm(y, eps / s ** 2).
-        ple = F.rms_norm(ple.reshape(rows, P), (P,), m.per_layer_projection_norm.weight, c.eps * c.hidden_size)
+        # The checkpoint's projection carries a factor hidden_size ** -0.5.  Since
+        # RMSNorm(s * y, eps) is RMSNorm(y, eps / s ** 2), it moves into the epsilon for free.
+        projected = F.rms_norm(projected.reshape(rows, width), (width,), trunk.per_layer_projection_norm.weight,
+                               c.eps * c.hidden_size)
         token = Copy.step(iron.weight(w.per_layer_embedding)[call.ids])
-        return w(x, call, (ple + token.reshape(ple.shape)) * 2**-0.5)
+        return w(x, call, (projected + token.reshape(projected.shape)) * 2**-0.5)
 
     def head(self, x):
-        """The tied head's logits, capped by a tanh where the config says."""
-        logits, cap = super().head(x), self.config.final_logit_softcapping
-        return logits if cap is None else Tanh.step(logits * (1 / cap)) * cap
+        """Logits, soft-capped as ``cap * tanh(logits / cap)`` when the config sets a cap."""
+        logits = super().head(x)
+        cap = self.config.final_logit_softcapping
+        if cap is None:
+            return logits
+        return Tanh.step(logits * (1 / cap)) * cap
+
+
+# per-layer tensors in the order the reference's toy draws them
+# (tests/applications/gemma4/reference/test.py:60-108); letters: E hidden, Q q width, K kv width,
+# D head width, M feed-forward width, P per-layer width
+_LAYER_TENSORS = (
+    ("self_attn.q_proj.weight", "QE"), ("self_attn.o_proj.weight", "EQ"), ("self_attn.q_norm.weight", "D"),
+    ("mlp.gate_proj.weight", "ME"), ("mlp.up_proj.weight", "ME"), ("mlp.down_proj.weight", "EM"),
+    ("per_layer_input_gate.weight", "PE"), ("per_layer_projection.weight", "EP"), ("layer_scalar", "1"),
+    # shipped for shared layers as well, though those never read them
+    ("self_attn.k_proj.weight", "KE"), ("self_attn.v_proj.weight", "KE"), ("self_attn.k_norm.weight", "D"),
+    ("input_layernorm.weight", "E"), ("post_attention_layernorm.weight", "E"),
+    ("pre_feedforward_layernorm.weight", "E"), ("post_feedforward_layernorm.weight", "E"),
+    ("post_per_layer_input_norm.weight", "E"),
+)
 
 
 def shapes(config: Gemma4Config) -> dict[str, tuple[int, ...]]:
-    """Each tensor of a Hugging Face Gemma 4 checkpoint's text decoder of ``config``'s shape, by
-    name, in the order the reference's toy draws them
-    (tests/applications/gemma4/reference/test.py:60-108)."""
+    """Name -> shape for the language model's tensors of a Hugging Face Gemma 4 checkpoint of this
+    config, in the order a seeded draw of the reference's toy follows."""
     c = config
-    L, E, P, V = c.num_hidden_layers, c.hidden_size, c.ple_dim, c.vocab_size
-    H, G = c.num_attention_heads, c.num_key_value_heads
-    model = PREFIX[:-1]
-    out = {
-        f"{model}.embed_tokens.weight": (V, E),
-        f"{model}.norm.weight": (E,),
-        f"{model}.embed_tokens_per_layer.weight": (V, L * P),
-        f"{model}.per_layer_model_projection.weight": (L * P, E),
-        f"{model}.per_layer_projection_norm.weight": (P,),
+    layers, hidden, width, vocab = c.num_hidden_layers, c.hidden_size, c.ple_dim, c.vocab_size
+    root = PREFIX.rstrip(".")
+    named = {
+        f"{root}.embed_tokens.weight": (vocab, hidden),
+        f"{root}.norm.weight": (hidden,),
+        f"{root}.embed_tokens_per_layer.weight": (vocab, layers * width),
+        f"{root}.per_layer_model_projection.weight": (layers * width, hidden),
+        f"{root}.per_layer_projection_norm.weight": (width,),
     }
-    for i in range(L):
-        D = c.global_head_dim if c.full(i) else c.head_dim
-        M = c.intermediate_size * (2 if c.use_double_wide_mlp and c.owner(i) != i else 1)
-        layer = f"{model}.layers.{i}"
-        out |= {
-            f"{layer}.self_attn.q_proj.weight": (H * D, E),
-            f"{layer}.self_attn.o_proj.weight": (E, H * D),
-            f"{layer}.self_attn.q_norm.weight": (D,),
-            f"{layer}.mlp.gate_proj.weight": (M, E),
-            f"{layer}.mlp.up_proj.weight": (M, E),
-            f"{layer}.mlp.down_proj.weight": (E, M),
-            f"{layer}.per_layer_input_gate.weight": (P, E),
-            f"{layer}.per_layer_projection.weight": (E, P),
-            f"{layer}.layer_scalar": (1,),
-            # A shared layer's too: the checkpoint ships them, the layer never reads them.
-            f"{layer}.self_attn.k_proj.weight": (G * D, E),
-            f"{layer}.self_attn.v_proj.weight": (G * D, E),
-            f"{layer}.self_attn.k_norm.weight": (D,),
-        }
-        out |= {f"{layer}.{norm}.weight": (E,) for norm in (
-            "input_layernorm", "post_attention_layernorm", "pre_feedforward_layernorm",
-            "post_feedforward_layernorm", "post_per_layer_input_norm")}
-    return out
+    for i in range(layers):
+        head = c.global_head_dim if c.full(i) else c.head_dim
+        doubled = c.use_double_wide_mlp and c.owner(i) != i
+        size = {"E": hidden, "P": width, "D": head, "1": 1, "Q": c.num_attention_heads * head,
+                "K": c.num_key_value_heads * head, "M": c.intermediate_size * (2 if doubled else 1)}
+        for tensor, letters in _LAYER_TENSORS:
+            named[f"{root}.layers.{i}.{tensor}"] = tuple(size[letter] for letter in letters)
+    return named

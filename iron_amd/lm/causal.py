@@ -1,9 +1,11 @@
-"""A decoder-only language model on the GPU, as one graph (iron/lm/causal.py:40-508).
+"""A decoder-only language model as ONE graph with two compiled versions sharing an arena.
 
-A call with no tensor is a decode step; ``prefill_chunk`` token ``ids`` are a prompt chunk
-from ``start``, of which a call runs the first ``rows``.  Both draw the next token on the
-device and carry it and ``position + 1`` into the next call.  The decode step is captured
-in a HIP graph that carries its own values, so a run of decode steps is a run of replays.
+Interface of the reference's iron/lm/causal.py:40-508 and iron/lm/model.py:321-597.  ``body`` is
+recorded twice: without ``ids`` it is the *decode step* (one token at ``position``), with
+``prefill_chunk`` ids it is a *prompt chunk* (``rows`` tokens from ``start``).  Either version ends
+by drawing the next token on the device and carrying ``token`` / ``position + 1`` forward.  On the
+GPU the decode step is captured in a HIP graph whose tail re-derives its own per-call words, so
+generating N tokens is N replays with no host round trip between them.
 """
 
 from __future__ import annotations
@@ -29,9 +31,11 @@ from .session import Session
 
 @dataclasses.dataclass(kw_only=True)
 class Call:
-    """One call's values, built once in ``body`` and read by every memory module
-    (``KVCache``, ``Rope``): a prompt chunk's ``rows`` from ``start``, or the decode step's
-    one at ``position``."""
+    """The per-call quantities of one recording, gathered once so that every stateful module
+    (caches, rotary tables) reads the same ones.  ``prompt`` tells the two versions apart; for a
+    decode step ``start`` is the position and ``rows`` is 1.  ``ropes`` memoises each rotary
+    table's rows for this call by table identity; ``embeddings`` is the layers' input, kept for
+    models whose layers look back at it."""
 
     prompt: bool
     start: Any
@@ -46,7 +50,8 @@ class Call:
 
 @dataclasses.dataclass
 class Stats:
-    """What a generation measured: seconds to the first token, tokens per second after it."""
+    """Timing of the last ``generate`` / ``stream``: time to first token (s), decode rate after it
+    (tokens/s), and how many tokens came out."""
 
     ttft: float = 0.0
     tokens_per_s: float = 0.0
@@ -54,235 +59,251 @@ class Stats:
 
 
 class Decoder(iron.Graph):
-    """A decoder's modules as a checkpoint's ``model`` names them."""
+    """The trunk under a checkpoint's ``model.`` prefix: embedding, layers, final norm."""
 
     def __init__(self, c: DecoderConfig, layer=DecoderLayer):
         self.embed_tokens = Embedding(c.vocab_size, c.hidden_size)
-        self.layers = [layer(c, i) for i in range(c.num_hidden_layers)]
+        self.layers = [layer(c, index) for index in range(c.num_hidden_layers)]
         self.norm = RMSNorm(c.hidden_size, c.eps)
 
 
+def _read_json(path: Path) -> dict:
+    return json.loads(path.read_text()) if path.exists() else {}
+
+
 class CausalLM(iron.Graph):
-    """A decoder on ``config``'s shape: ``model``, ``lm_head`` and ``rotary_emb``."""
+    """``model`` (the trunk), ``lm_head`` (tied to the embedding unless the config says otherwise)
+    and ``rotary_emb``.  Subclasses vary it through ``config_class`` / ``layer_class`` /
+    ``decoder_class`` and the hooks ``lookup``, ``layer``, ``head``."""
 
     decoder_class = Decoder
     layer_class = DecoderLayer
-    #: The config class ``from_checkpoint`` builds from a checkpoint's ``config.json``.
-    config_class = DecoderConfig
+    config_class = DecoderConfig      # what from_checkpoint parses config.json into
     checkpoint = None
     tokenizer = None
+    k_max = 64                        # candidates a device draw can weigh; Sampler.rows refuses a larger top-k
+
+    # ------------------------------------------------------------------ construction
+    def __init__(self, config: DecoderConfig, weights):
+        self.config = config
+        self.rotary_emb = Rope(config) if config.rope_theta is not None else None
+        rows = config.max_seq_len
+        self.draws = iron.state((rows, ROW_WORDS), np.int32)   # a draw row per position; all-zero = greedy
+        self.drawn = iron.state((rows,), np.int32)             # the device's record of what it drew where
+        self.sampled = False          # whether `draws` currently holds a sampler's rows
+        self.decode_step = self.prompt_chunk = None
+        self.holder = None            # the Session whose tokens the caches hold
+        self.session = Session(self)
+        self.stats = Stats()
+        self.model = self.decoder_class(config, self.layer_class)
+        self.layers = self.model.layers
+        for block in self.layers:
+            block.rope = self.rotary_emb
+        self.lm_head = Linear(config.hidden_size, config.vocab_size, False, precision=config.precision)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.model.embed_tokens.weight
+        self.load_state_dict(weights)
 
     @classmethod
     def from_checkpoint(cls, path, *, max_seq_len: int | None = None, **changes):
-        """The model of a checkpoint directory's files (``config.json``, ``model.safetensors`` or its
-        sharded index, ``tokenizer.json``), not yet loaded (iron/lm/model.py:321-388).
+        """Build (not yet compile) the model described by a local checkpoint directory:
+        ``config.json``, ``model.safetensors`` or a shard index, optionally ``tokenizer.json`` with
+        ``tokenizer_config.json`` / ``chat_template.jinja`` (iron/lm/model.py:321-388).  Nothing is
+        fetched from anywhere.
 
         Args:
-            path: the directory (nothing is downloaded here).
-            max_seq_len: the longest context served, at most the checkpoint's own.
-            changes: other config fields replaced (``prefill_chunk=...``).
+            max_seq_len: context to serve; may only shrink the checkpoint's own.
+            changes: further config overrides, e.g. ``prefill_chunk=512``.
 
         Raises:
-            ValueError: ``max_seq_len`` is past the checkpoint's own.
+            FileNotFoundError: ``path`` is not a directory.
+            ValueError: ``max_seq_len`` exceeds what the checkpoint supports.
         """
         from .checkpoint import Checkpoint, weights_file
         from .tokenizer import Tokenizer, TokenizerJson
 
-        directory = Path(path)
-        if not directory.is_dir():
-            raise FileNotFoundError(f"{directory} is not a checkpoint directory (repositories are not downloaded)")
-        config = cls.config_class.from_checkpoint(directory)
-        if max_seq_len is not None:
-            if max_seq_len > config.max_seq_len:
-                raise ValueError(f"max_seq_len {max_seq_len} is past the model's {config.max_seq_len}")
-            changes["max_seq_len"] = max_seq_len
-        if changes:
-            config = dataclasses.replace(config, **changes)
-        checkpoint = Checkpoint(weights_file(directory))
-        # On the device a bf16 tensor goes up as the file holds it; the host stand-in computes on arrays.
+        folder = Path(path)
+        if not folder.is_dir():
+            raise FileNotFoundError(f"{folder} is not a checkpoint directory (repositories are not downloaded)")
+        config = cls.config_class.from_checkpoint(folder)
+        if max_seq_len is not None and max_seq_len > config.max_seq_len:
+            raise ValueError(f"max_seq_len {max_seq_len} is past the model's {config.max_seq_len}")
+        overrides = dict(changes) if max_seq_len is None else {**changes, "max_seq_len": max_seq_len}
+        if overrides:
+            config = dataclasses.replace(config, **overrides)
+        checkpoint = Checkpoint(weights_file(folder))
+        # The GPU takes bf16 exactly as stored (torch views of the mapped file); only the host
+        # stand-in wants widened arrays to compute on.
         weights = checkpoint.state_dict(as_torch=not issubclass(cls, OnHost))
-        if config.tie_word_embeddings:
-            weights.pop("lm_head.weight", None)  # some exports repeat the tied matrix
+        if config.tie_word_embeddings and "lm_head.weight" in weights:
+            del weights["lm_head.weight"]       # some exporters write the tied matrix twice
         model = cls(config, weights)
         model.checkpoint = checkpoint
-        if (directory / "tokenizer.json").exists():
-            settings, jinja = directory / "tokenizer_config.json", directory / "chat_template.jinja"
-            found = json.loads(settings.read_text()) if settings.exists() else {}
-            template = jinja.read_text() if jinja.exists() else found.get("chat_template")
-            b = found.get("bos_token")
-            bos_token = (b["content"] if isinstance(b, dict) else b) or ""
-            model.tokenizer = Tokenizer(TokenizerJson(directory / "tokenizer.json"), template, bos_token)
+        vocabulary = folder / "tokenizer.json"
+        if vocabulary.exists():
+            settings = _read_json(folder / "tokenizer_config.json")
+            template_file = folder / "chat_template.jinja"
+            template = template_file.read_text() if template_file.exists() else settings.get("chat_template")
+            bos = settings.get("bos_token")
+            if isinstance(bos, dict):           # {"content": "<s>", ...} in older configs
+                bos = bos.get("content")
+            model.tokenizer = Tokenizer(TokenizerJson(vocabulary), template, bos or "")
         return model
 
     @classmethod
     def load(cls, path, *, max_seq_len: int | None = None, capture: bool = True, **changes):
-        """``from_checkpoint``'s model compiled and loaded, its weights uploaded."""
+        """``from_checkpoint`` followed by ``load_versions``: ready to generate."""
         model = cls.from_checkpoint(path, max_seq_len=max_seq_len, **changes)
         model.load_versions(capture=capture)
         return model
 
     @functools.cached_property
     def eos(self) -> set[int]:
-        """The tokens generation stops at: the checkpoint's ``eos_token_id``, one or a list, from its
-        ``generation_config.json`` or else its ``config.json``; none without either."""
+        """Token ids that end a generation: ``eos_token_id`` (a number or a list) from the
+        checkpoint's ``generation_config.json``, failing that its ``config.json``; empty for a model
+        built from arrays."""
         if self.checkpoint is None:
             return set()
-        directory = Path(self.checkpoint.path).parent
+        folder = Path(self.checkpoint.path).parent
         for name in ("generation_config.json", "config.json"):
-            file = directory / name
-            if file.exists():
-                eos = json.loads(file.read_text()).get("eos_token_id")
-                if eos is not None:
-                    return set(eos) if isinstance(eos, list) else {eos}
+            declared = _read_json(folder / name).get("eos_token_id")
+            if declared is not None:
+                return set(declared) if isinstance(declared, list) else {declared}
         return set()
-
-    #: The most candidates a draw on the device weighs (``Sampler.rows`` refuses a larger top-k).
-    k_max = 64
-
-    def __init__(self, config: DecoderConfig, weights):
-        self.config = config
-        self.rotary_emb = None if config.rope_theta is None else Rope(config)
-        # Zero until the host writes draws: a row of zeros is greedy.
-        self.draws = iron.state((config.max_seq_len, ROW_WORDS), np.int32)
-        self.drawn = iron.state((config.max_seq_len,), np.int32)
-        self.sampled = False  # the draw rows hold a sampler's, not zeros
-        self.prompt_chunk = None
-        self.decode_step = None
-        self.holder = None
-        self.session = Session(self)
-        self.stats = Stats()
-        self.model = self.decoder_class(config, self.layer_class)
-        for layer in self.model.layers:
-            layer.rope = self.rotary_emb
-        self.lm_head = Linear(config.hidden_size, config.vocab_size, False, precision=config.precision)
-        if config.tie_word_embeddings:
-            self.lm_head.weight = self.model.embed_tokens.weight
-        self.load_state_dict(weights)
-        self.layers = self.model.layers
 
     @property
     def recurrent(self) -> list:
-        """The states that restart only at some positions: the layers' ring caches."""
-        rings = {id(l.cache): l.cache for l in self.layers if getattr(l.cache, "ring", None) is not None}
-        return list(rings.values())
+        """State that cannot be rewound to an arbitrary position -- the ring caches -- each once even
+        where layers share it.  ``Session.resume`` asks these where a run may restart."""
+        seen: dict[int, Any] = {}
+        for block in self.layers:
+            if getattr(block.cache, "ring", None) is not None:
+                seen.setdefault(id(block.cache), block.cache)
+        return list(seen.values())
+
+    # ------------------------------------------------------------------ the recorded body
+    def lookup(self, ids):
+        """Hook: token ids -> embedding rows."""
+        return self.model.embed_tokens(ids)
 
     def layer(self, call, i: int, w, x):
-        """Layer ``i``, ``w``, on ``x``: a model whose layers take more than the call says what."""
+        """Hook: apply layer ``i`` (module ``w``) to ``x``; override where layers take extra inputs."""
         return w(x, call)
 
     def head(self, x):
-        """The final norm, then the output head (the embedding, if tied)."""
+        """Hook: final norm and output projection."""
         return self.lm_head(self.model.norm(x))
-
-    def lookup(self, ids):
-        return self.model.embed_tokens(ids)
 
     def body(self, ids=None, *, token: Carried[np.int32], position: Carried[np.int32],
              start: Scratchpad[np.int32] = np.int32(0), rows: Scratchpad[np.int32] = np.int32(1),
              rope_start: Scratchpad[np.int32] = np.int32(0)):
-        prompt = ids is not None
-        call = Call(prompt=prompt, start=start if prompt else position, rows=rows, position=position,
-                    rope_start=rope_start, ids=ids[:rows] if prompt else token, token=token)
-        if prompt:
-            return self.forward(self.lookup(call.ids), call)
-        return self.forward(self.lookup(token).reshape(1, self.config.hidden_size), call)
+        if ids is None:
+            call = Call(prompt=False, start=position, rows=rows, position=position, rope_start=rope_start,
+                        ids=token, token=token)
+            x = self.lookup(token).reshape(1, self.config.hidden_size)
+        else:
+            call = Call(prompt=True, start=start, rows=rows, position=position, rope_start=rope_start,
+                        ids=ids[:rows], token=token)
+            x = self.lookup(call.ids)
+        return self.forward(x, call)
 
     def forward(self, x, call: Call):
-        """The layers, the head and the draw over ``x``, the rows ``call`` runs."""
-        c = self.config
+        """Embeddings ``x`` through the layers, the head and the draw."""
         call.embeddings = x
-        for rope in (layer.rope for layer in self.layers):
-            if rope is not None and id(rope) not in call.ropes:
-                call.ropes[id(rope)] = rope.rows(call)
-        for i, layer in enumerate(self.layers):
-            x = self.layer(call, i, layer, x)
+        for block in self.layers:          # each distinct rotary table copies its rows once per call
+            table = block.rope
+            if table is not None and id(table) not in call.ropes:
+                call.ropes[id(table)] = table.rows(call)
+        for index, block in enumerate(self.layers):
+            x = self.layer(call, index, block, x)
         if call.prompt:
-            x = Copy.step(x[call.rows - 1]).reshape(1, c.hidden_size)  # the last row's logits alone
+            # only the chunk's last real row feeds the head
+            x = Copy.step(x[call.rows - 1]).reshape(1, self.config.hidden_size)
         return self.draw(self.head(x), call)
 
     def draw(self, logits, call: Call):
-        """``logits`` and the token drawn from them on the device, carried with the next position."""
-        c = self.config
-        _, drawn = Sample.step(logits.reshape(c.vocab_size), self.draws, self.drawn,
-                               row=call.position * ROW_WORDS, at=call.position, drawable=c.vocab_size,
-                               k_max=self.k_max)
-        return logits, iron.carry(token=drawn, position=call.position + 1)
+        """Draw from ``logits`` by this position's draw row; returns the logits and the carry."""
+        vocab = self.config.vocab_size
+        _, token = Sample.step(logits.reshape(vocab), self.draws, self.drawn, row=call.position * ROW_WORDS,
+                               at=call.position, drawable=vocab, k_max=self.k_max)
+        return logits, iron.carry(token=token, position=call.position + 1)
 
-    # -- versions ------------------------------------------------------------
+    # ------------------------------------------------------------------ versions
     def shapes(self) -> list[dict]:
-        """The input shapes of each version: the decode step's (none), then the prompt chunk's ids."""
-        return [{}, dict(ids=((self.config.prefill_chunk,), np.int32))]
+        """Input shapes per version: ``[decode step (no tensor), prompt chunk (ids)]``."""
+        return [{}, {"ids": ((self.config.prefill_chunk,), np.int32)}]
 
     def load_versions(self, *, capture: bool = True, check: bool = False, fuse: bool = True) -> None:
-        """Compile the decode step and the prompt chunk into one arena and load them.
-
-        ``fuse``: launch the decode step's runs of one-row steps as fused kernels.
-        """
-        decode_shapes, prompt_shapes = self.shapes()
+        """Compile both versions into the shared arena, upload the weights, capture the decode step.
+        ``fuse=False`` launches every recorded step on its own (what ``check=True`` implies);
+        ``capture=False`` keeps the decode step eager."""
+        for_decode, for_prompt = self.shapes()
         try:
-            decode = self.compile(capture=capture, check=check, fuse=fuse, **decode_shapes)
-            prompt = self.compile(capture=False, check=check, fuse=fuse, **prompt_shapes)
-            decode.load()
-            prompt.load()
+            decode = self.compile(capture=capture, check=check, fuse=fuse, **for_decode)
+            prompt = self.compile(capture=False, check=check, fuse=fuse, **for_prompt)
+            for version in (decode, prompt):
+                version.load()
         except Exception:
             self.release()
             raise
         self.use(decode, prompt)
 
     def use(self, decode, prompt) -> None:
-        self.decode_step, self.prompt_chunk = decode, prompt
-        self.holder = None
+        """Adopt two loaded versions; whatever the caches held belongs to nobody now."""
+        self.decode_step, self.prompt_chunk, self.holder = decode, prompt, None
 
     def release(self) -> None:
         self.decode_step = self.prompt_chunk = None
         super().release()
 
     def __call__(self, ids=None, **values):
-        """One call of the prompt version or else the decode step."""
+        """Inside a recording: record the body.  Otherwise run a loaded version -- the prompt chunk
+        when ``ids`` are given, else the decode step."""
         if iron.graph_recorder.get() is not None:
             return super().__call__(ids, **values)
         if self.decode_step is None:
             raise RuntimeError(f"{type(self).__name__}: load_versions() first")
-        if ids is None:
-            return self.decode_step(**values)
-        return self.prompt_chunk(ids, **values)
+        return self.decode_step(**values) if ids is None else self.prompt_chunk(ids, **values)
 
+    # ------------------------------------------------------------------ use
     def logits(self, tokens) -> np.ndarray:
-        """The logits after the last of ``tokens``, the whole history (``Session.logits``)."""
+        """Logits after the last of ``tokens`` (see ``Session.logits``)."""
         return self.session.logits(tokens)
 
-    def generate(self, prompt, max_tokens: int, sampler=None):
-        """Up to ``max_tokens`` tokens drawn on the device after ``prompt``, stopping after an
-        end-of-sequence token; fills ``stats``.  Token ids in, token ids out; a text (or a chat's
-        list of messages) in, the text drawn out (needs the checkpoint's tokenizer).  ``sampler``:
-        how each is drawn (``generation.Sampler``); None is greedy (iron/lm/model.py:506-545)."""
-        if _is_text(prompt):
-            drawn = [t for t in self.stream(prompt, max_tokens, sampler) if t not in self.eos]
-            return self.tokenizer.decode(drawn)
-        return list(self.stream(prompt, max_tokens, sampler))
-
-    def _ids(self, prompt):
+    def _prompt_ids(self, prompt):
         if not _is_text(prompt):
             return prompt
         if self.tokenizer is None:
             raise ValueError(f"{type(self).__name__}: a text prompt takes the checkpoint's tokenizer; none is loaded")
-        return self.tokenizer(prompt) if isinstance(prompt, str) else self.tokenizer.chat(prompt)
+        return self.tokenizer.chat(prompt) if isinstance(prompt, list) else self.tokenizer(prompt)
 
     def stream(self, prompt, max_tokens: int, sampler=None) -> Iterator[int]:
-        tokens = self._ids(prompt)
-        t0 = time.perf_counter()
-        first = None
-        n = 0
-        for token in self.session.draw(tokens, max_tokens, sampler):
-            n += 1
-            if first is None:
-                first = time.perf_counter()
+        """Yield drawn token ids one by one, stopping after an end-of-sequence id; records ``stats``."""
+        ids = self._prompt_ids(prompt)
+        began = time.perf_counter()
+        first_at, count = None, 0
+        for token in self.session.draw(ids, max_tokens, sampler):
+            now = time.perf_counter()
+            first_at = now if first_at is None else first_at
+            count += 1
             yield token
             if token in self.eos:
                 break
-        end = time.perf_counter()
-        self.stats = Stats(ttft=(first or end) - t0,
-                           tokens_per_s=(n - 1) / (end - first) if n > 1 and end > first else 0.0, tokens=n)
+        ended = time.perf_counter()
+        first_at = ended if first_at is None else first_at
+        decoding = ended - first_at
+        rate = (count - 1) / decoding if count > 1 and decoding > 0 else 0.0
+        self.stats = Stats(ttft=first_at - began, tokens_per_s=rate, tokens=count)
+
+    def generate(self, prompt, max_tokens: int, sampler=None):
+        """Generate up to ``max_tokens`` tokens on the device (iron/lm/model.py:506-545).  Ids in, ids
+        out (the end-of-sequence id included if one was drawn).  A string, or a chat as a list of
+        ``{"role", "content"}`` messages, goes through the checkpoint's tokenizer and comes back as
+        text without end-of-sequence tokens.  ``sampler=None`` draws greedily."""
+        tokens = list(self.stream(prompt, max_tokens, sampler))    # refuses a text prompt without a tokenizer
+        if not _is_text(prompt):
+            return tokens
+        return self.tokenizer.decode([t for t in tokens if t not in self.eos])
 
 
 def _is_text(prompt) -> bool:
