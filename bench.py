@@ -388,7 +388,7 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
             K.copy_rows(src, dst, rows=rows, row_elems=1024, src_rows=rows, dst_rows=rows)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "decode", "prefill_tokens": 512, "decode_steps": probe_steps,
-                          "launches_per_step": decode.launches_per_call,
+                          "launches_per_step": decode.launches_per_replay,
                           "copy": {"launches": 2, "bytes_read": PROBE_COPY_BYTES, "bytes_written": PROBE_COPY_BYTES}}))
         model.release()
         return None, None
@@ -420,7 +420,7 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
            "bytes_per_token": int(per_token), "GBps": round(per_token * tok_s / 1e9, 1),
            "frac_hbm": round(per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
            "steps_recorded": len(decode.recording.steps),
-           "launches_per_step": decode.launches_per_call,
+           "launches_per_step": decode.launches_per_replay,
            "launches_per_prompt_chunk": model.prompt_chunk.launches_per_call, "first_tokens": [int(t) for t in tokens[:4]]}
     cpu = None
     if with_cpu:

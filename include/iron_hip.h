@@ -71,12 +71,15 @@ int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const uint16_t* 
 /* Attention's first half for one token: n = RMSNorm(x) * norm_w; q = Wq n, k = Wk n, v = Wv n
  * (each rounded to bf16); q and k rotated by the RoPE row `angles` (d bf16, cos/sin interleaved,
  * two halves); q -> q_out (heads*d), k -> keys[*position], v -> values[*position], caches
- * (cache_rows, kv_heads, d).  Replaces RMSNorm, 3 GEMV, 2 RoPE and 2 Copy steps
- * (iron/lm/blocks.py:472-502,627-648). */
+ * (cache_rows, kv_heads, d).  With angle_row not NULL, `angles` is a whole RoPE table of angle_rows
+ * rows and the row is angles[*angle_row] (held inside the table): the step's copy of its table row
+ * (iron/lm/blocks.py:394-431) then needs no launch of its own.  Replaces RMSNorm, 3 GEMV, 2 RoPE and
+ * 2 Copy steps (iron/lm/blocks.py:472-502,627-648). */
 int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* Wq,
                          const uint16_t* Wk, const uint16_t* Wv, const uint16_t* angles,
                          uint16_t* q_out, uint16_t* keys, uint16_t* values, int hidden, int heads,
-                         int kv_heads, int d, int cache_rows, const int* position, void* stream);
+                         int kv_heads, int d, int cache_rows, const int* position, const int* angle_row,
+                         int angle_rows, void* stream);
 
 /* A prompt chunk's three projections and the rotation of q and k in one launch (no single
  * counterpart in the reference: replaces 3 GEMM and 2 RoPE steps, iron/lm/blocks.py:617-648, and
@@ -263,6 +266,16 @@ int64_t iron_sample_workspace_bytes(int n);
 int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,
                      const int* row, int k_max, void* workspace, int* token, int* record,
                      int record_len, const int* at, int* token_copy, void* stream);
+
+/* iron_sample_bf16 that ends a decode step: after the token is written (to token, record and
+ * token_copy), the same launch evaluates the n_exprs word expressions of iron_eval_words over
+ * words[0..n_words) -- the carried position and every word derived from it -- so a replayed step needs
+ * no launch of its own for them.  Replaces Sample followed by the carry's Emit
+ * (iron/operators/sample.py:106, iron/common/graph/carried.py:189-276). */
+int iron_sample_advance_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,
+                             const int* row, int k_max, void* workspace, int* token, int* record,
+                             int record_len, const int* at, int* token_copy, int* words, int n_words,
+                             const int* exprs, int n_exprs, void* stream);
 
 /* Evaluate n per-call word expressions in order, on the device, in one thread:
  *   words[e.dst] = (clamp(((words[e.src] * e.mul + e.add) >> e.shift), e.lo, e.hi) & e.mask) + e.post

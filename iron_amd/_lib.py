@@ -25,7 +25,7 @@ SIGNATURES = {
     "iron_gemv_fused_bf16": (c_int, [_P, _P, _P, _P, c_float, _P, c_float, _P, c_int, c_int, c_int, _P]),
     "iron_decode_qkv_bf16": (
         c_int,
-        [_P, _P, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P],
+        [_P, _P, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P, c_int, _P],
     ),
     "iron_prefill_qkv_bf16": (c_int, [_P] * 8 + [c_int] * 5 + [_P, _P]),
     "iron_prefill_qkv_cache_bf16": (c_int, [_P] * 8 + [c_int] * 6 + [_P, _P, _P]),
@@ -69,6 +69,8 @@ SIGNATURES = {
     "iron_softmax_bf16": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_float, _P, _P]),
     "iron_sample_workspace_bytes": (c_int64, [c_int]),
     "iron_sample_bf16": (c_int, [_P, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P]),
+    "iron_sample_advance_bf16": (c_int, [_P, c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, c_int, _P,
+                                         c_int, _P]),
     "iron_eval_words": (c_int, [_P, c_int, _P, c_int, _P]),
 }
 

@@ -42,6 +42,7 @@ class Fused:
     first: int
     count: int
     launch: Callable[[], None]
+    launches: int = 1      # 0: a step other launches made needless (nothing runs for it)
 
 
 class _Anything:
@@ -113,6 +114,8 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
         return ok and (x is None or _same(s.inputs["B"], x))
 
     fused: list[Fused] = []
+    # decode_qkv launches whose RoPE row is a copy of one table row: (producing step, args, kw)
+    rope_rows: list[tuple[int, dict, dict]] = []
     i = 0
     while i < len(steps):
         s = steps[i]
@@ -152,6 +155,9 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                     kw = dict(eps=float(s.op.epsilon), hidden=s.op.tile_size, heads=q.elements // d,
                               kv_heads=k.elements // d, d=d, cache_rows=kd.index_rows, position=word(kd.index))
                     got = Fused("decode_qkv", i, 8, lambda a=args, kw=kw: kernels.decode_qkv(**a, **kw))
+                    made_by = _row_copy(steps, i, rq.inputs["angles"], d)
+                    if made_by is not None:
+                        rope_rows.append((made_by, args, kw))
             # the gated MLP's first half
             if (got is None and len(rest) >= 4 and gemv_row(rest[0], n) and gemv_row(rest[1], n) and once(n, 2)
                     and (_name(rest[2]) == "SiLU" or (_name(rest[2]) == "GELU" and rest[2].op.approximate == "tanh"))
@@ -303,4 +309,32 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
             i += got.count
         else:
             i += 1
-    return fused
+    # A RoPE row copied out of its table for nobody but these launches: they read the table at the
+    # call's row themselves, and the copy is not launched.
+    for producer in sorted({p for p, _, _ in rope_rows}):
+        users = [(a, kw) for p, a, kw in rope_rows if p == producer]
+        row = steps[producer].outputs["dst"]
+        if reads[id(row.buffer)] != 2 * len(users) or any(f.first <= producer < f.first + f.count for f in fused):
+            continue
+        table = steps[producer].inputs["src"]
+        for a, kw in users:
+            a["angles"] = tensor(table).reshape(-1)[: table.index_rows * table.index_stride]
+            kw["angle_row"] = word(table.index)
+        fused.append(Fused("elided_rope_row", producer, 1, lambda: None, launches=0))
+    return sorted(fused, key=lambda f: f.first)
+
+
+def _row_copy(steps, before: int, row, width: int):
+    """The step before ``before`` that made ``row`` by copying one table row a per-call word names
+    (``Copy(table[position])``), or None."""
+    for j in range(before - 1, -1, -1):
+        s = steps[j]
+        if any(h.buffer is row.buffer for h in s.outputs.values()):
+            if _name(s) != "Copy":
+                return None
+            src, dst = s.inputs["src"], s.outputs["dst"]
+            ok = (_same(dst, row) and src.index is not None and src.ids is None and not src.valid and src.offset == 0
+                  and src.index_stride == width and src.elements == width and src.buffer.kind == "resident"
+                  and not s.values)
+            return j if ok else None
+    return None

@@ -1225,6 +1225,9 @@ class CompiledGraph:
                 if h.buffer is last.outputs["token"].buffer and h.offset == last.outputs["token"].offset:
                     self._carry_by_draw[len(self.recording.steps) - 1] = slot
                     self.carry_copies.remove((slot, h))
+        # ... and where the draw is the captured step's last launch and nothing else is carried from a
+        # buffer, it evaluates the tail's expressions too: the step ends without a launch for them.
+        self._tail_in_draw = bool(self.capture and self._carry_by_draw and self.n_tail and not self.carry_copies)
         self._launches = [self._bind(step) for step in self.recording.steps]
         self._fused = {}
         if self.fuse:
@@ -1256,6 +1259,8 @@ class CompiledGraph:
         slot = self._carry_by_draw.get(self.recording.steps.index(step)) if self._carry_by_draw else None
         if slot is not None:
             words = {**words, "__carry_token__": self.words[slot : slot + 1]}
+            if self._tail_in_draw:
+                words["__carry_eval__"] = (self.words, self.expr_table[EXPR_WORDS * self.n_derived :], self.n_tail)
         return built.launch, tensors, words
 
     def _run_steps(self) -> None:
@@ -1273,7 +1278,18 @@ class CompiledGraph:
     @property
     def launches_per_call(self) -> int:
         """Kernel-launching units a call runs (recorded steps less those fused away)."""
-        return len(self._launches) - sum(f.count - 1 for f in self._fused.values())
+        return len(self._launches) - sum(f.count - f.launches for f in self._fused.values())
+
+    @property
+    def launches_per_replay(self) -> int:
+        """Kernel launches one replay of the captured version makes: its steps' and, where the draw
+        does not end the step itself, the tail's (carried values, re-derived words)."""
+        if not self.capture:
+            return self.launches_per_call
+        if self._tail_in_draw:
+            return self.launches_per_call
+        tail = len(self.carry_copies) + (1 if self.n_tail else (2 if self.n_exprs > self.n_derived else 0))
+        return self.launches_per_call + tail
 
     def _derive(self) -> None:
         from .. import kernels
@@ -1288,6 +1304,8 @@ class CompiledGraph:
         for slot, h in self.carry_copies:
             kernels.copy_rows(self._tensor(h).view(-1)[:1], self.words[slot : slot + 1], rows=1, row_elems=1,
                               src_rows=1, dst_rows=1)
+        if self._tail_in_draw:
+            return
         if self.n_tail:
             kernels.eval_words(self.words, self.expr_table[EXPR_WORDS * self.n_derived :], self.n_tail)
         elif self.n_exprs > self.n_derived:

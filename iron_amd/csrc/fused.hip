@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
     const bf16_t* __restrict__ Wq, const bf16_t* __restrict__ Wk, const bf16_t* __restrict__ Wv,
     const bf16_t* __restrict__ angles, bf16_t* __restrict__ q_out, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, int K, int heads, int kv_heads, int cache_rows,
-    const int* __restrict__ position) {
+    const int* __restrict__ position, const int* __restrict__ angle_row, int angle_rows) {
   constexpr int HALF = D / 2;
   __shared__ float scratch4[4];
   __shared__ float part[4][2];
@@ -171,6 +171,8 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   else if (pair < q_pairs + k_pairs) { kind = 1; Wm = Wk; const int p = pair - q_pairs; const int h = p / HALF; j = p % HALF; r0 = h * D + j; r1 = r0 + HALF; }
   else { kind = 2; Wm = Wv; const int p = pair - q_pairs - k_pairs; r0 = 2 * p; r1 = r0 + 1; }
 
+  // `angles` is the step's row itself, or a whole table whose row a device word names (held inside).
+  if (angle_row != nullptr) angles += (size_t)max(0, min(*angle_row, angle_rows - 1)) * D;
   // What the block's last thread needs after the last barrier is requested first: the pair's
   // angle and the position word ride under the weights' trip to memory.
   const float c_ahead = bf16_to_f32(angles[2 * j]), s_ahead = bf16_to_f32(angles[2 * j + 1]);
@@ -250,7 +252,8 @@ extern "C" int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, f
                                     const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,
                                     const uint16_t* angles, uint16_t* q_out, uint16_t* keys,
                                     uint16_t* values, int hidden, int heads, int kv_heads, int d,
-                                    int cache_rows, const int* position, void* stream) {
+                                    int cache_rows, const int* position, const int* angle_row, int angle_rows,
+                                    void* stream) {
   IRON_REQUIRE(x && norm_w && Wq && Wk && Wv && angles && q_out && keys && values && position,
                "decode_qkv: null operand");
   IRON_REQUIRE(hidden > 0 && hidden % 8 == 0, "decode_qkv: hidden (%d) must be a positive multiple of 8", hidden);
@@ -259,13 +262,14 @@ extern "C" int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, f
   IRON_REQUIRE((((uintptr_t)x | (uintptr_t)norm_w | (uintptr_t)Wq | (uintptr_t)Wk | (uintptr_t)Wv) & 15) == 0,
                "decode_qkv: operands must be 16-byte aligned");
   IRON_REQUIRE(hidden <= 8192, "decode_qkv: hidden (%d) exceeds 8192", hidden);
+  IRON_REQUIRE(angle_row == nullptr || angle_rows > 0, "decode_qkv: a table of %d angle rows", angle_rows);
   const int pairs = heads * (d / 2) + 2 * kv_heads * (d / 2);
   const int ch = hidden <= 2048 ? 1 : (hidden <= 4096 ? 2 : 4);
   hipStream_t s = (hipStream_t)stream;
 #define IRON_QKV(DD, C)                                                                             \
   if (d == DD && ch == C)                                                                           \
     hipLaunchKernelGGL((decode_qkv_kernel<DD, C>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
-                       angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position);
+                       angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row, angle_rows);
   IRON_QKV(64, 1) IRON_QKV(64, 2) IRON_QKV(64, 4) IRON_QKV(128, 1) IRON_QKV(128, 2) IRON_QKV(128, 4)
 #undef IRON_QKV
   IRON_LAUNCH_CHECK();

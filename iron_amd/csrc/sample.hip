@@ -205,7 +205,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const bf16_t* __restrict__ logits, int n, const int* __restrict__ draws, int draws_words,
     const int* __restrict__ row, int k_max, uint64_t* workspace, int* __restrict__ token,
     int* __restrict__ record, int record_len, const int* __restrict__ at,
-    int* __restrict__ token_copy) {
+    int* __restrict__ token_copy, int* words, int n_words, const int* __restrict__ exprs, int n_exprs) {
   __shared__ SampleShared sh;
   unsigned int* ticket = reinterpret_cast<unsigned int*>(workspace);
   uint64_t* lists = workspace + SAMPLE_TICKET_BYTES / 8;
@@ -313,6 +313,19 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
   // The first wave: a candidate's weight a lane; every lane sums and walks them in order.
   if (threadIdx.x >= 64) return;
+  // The step's own tail, where the caller asks for it (the word expressions of iron_eval_words: the
+  // carried position, then every word derived from it and from the token drawn here).  Its operands
+  // are requested now, a word and an expression a lane, so that their trips to memory pass under the
+  // draw: evaluated one after the other from memory they would cost a trip each.
+  const bool tail = n_exprs > 0, tail_in_lds = tail && n_words <= 64 && n_exprs <= 64;
+  int my_word = 0, rec[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+  if (tail_in_lds) {
+    if ((int)threadIdx.x < n_words) my_word = words[threadIdx.x];
+    if ((int)threadIdx.x < n_exprs) {
+#pragma unroll
+      for (int f = 0; f < 9; ++f) rec[f] = exprs[9 * threadIdx.x + f];
+    }
+  }
   int tok = entry_index(sh.cand[0]);
   const float top = key_value((uint32_t)(sh.cand[0] >> 32));
   if (k > 1 && top - top == 0.f) {   // a finite best logit; else it draws itself
@@ -349,6 +362,38 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       const int where = at ? *at : 0;
       if (where >= 0 && where < record_len) record[where] = tok;
     }
+    if (tail && !tail_in_lds) {   // more words or expressions than a wave holds: one by one, from memory
+      for (int e = 0; e < n_exprs; ++e) {
+        const int* x = exprs + 9 * e;
+        const int dst = x[0], src = x[1];
+        if (dst < 0 || dst >= n_words || src < 0 || src >= n_words) continue;
+        long v = ((long)words[src] * x[2] + x[3]) >> x[4];
+        v = v < x[5] ? x[5] : (v > x[6] ? x[6] : v);
+        words[dst] = ((int)v & x[7]) + x[8];
+      }
+    }
+  }
+  if (tail_in_lds) {
+    // The words in LDS (the wave is alone by now), the token where the caller carries it, the
+    // expressions in order -- each from the lane that holds it -- and the words back, a lane each.
+    int* wl = reinterpret_cast<int*>(sh.best);
+    wl[threadIdx.x] = my_word;
+    const long slot = token_copy != nullptr ? (long)(token_copy - words) : -1;
+    if (threadIdx.x == 0 && slot >= 0 && slot < n_words) wl[slot] = tok;
+    for (int e = 0; e < n_exprs; ++e) {
+      int x[9];
+#pragma unroll
+      for (int f = 0; f < 9; ++f) x[f] = __builtin_amdgcn_readlane(rec[f], e);
+      if (threadIdx.x == 0 && x[0] >= 0 && x[0] < n_words && x[1] >= 0 && x[1] < n_words) {
+        long v = ((long)wl[x[1]] * x[2] + x[3]) >> x[4];
+        v = v < x[5] ? x[5] : (v > x[6] ? x[6] : v);
+        wl[x[0]] = ((int)v & x[7]) + x[8];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if ((int)threadIdx.x < n_words) words[threadIdx.x] = wl[threadIdx.x];
   }
 }
 
@@ -362,9 +407,9 @@ extern "C" int64_t iron_sample_workspace_bytes(int n) {
   return SAMPLE_TICKET_BYTES + (int64_t)sample_blocks(n) * SAMPLE_K_MAX * 8;
 }
 
-extern "C" int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,
-                                const int* row, int k_max, void* workspace, int* token, int* record,
-                                int record_len, const int* at, int* token_copy, void* stream) {
+static int sample_launch(const uint16_t* logits, int n, const int* draws, int draws_words, const int* row, int k_max,
+                         void* workspace, int* token, int* record, int record_len, const int* at, int* token_copy,
+                         int* words, int n_words, const int* exprs, int n_exprs, void* stream) {
   IRON_REQUIRE(logits && token, "sample: null operand");
   IRON_REQUIRE(n > 0 && sample_blocks(n) <= SAMPLE_BLOCKS_MAX, "sample: n (%d) must be from 1 to %d", n,
                SAMPLE_BLOCKS_MAX * SAMPLE_SHARE);
@@ -374,8 +419,25 @@ extern "C" int iron_sample_bf16(const uint16_t* logits, int n, const int* draws,
   IRON_REQUIRE(((uintptr_t)logits & 15) == 0, "sample: logits must be 16-byte aligned");
   IRON_REQUIRE(sample_blocks(n) == 1 || (workspace && ((uintptr_t)workspace & 7) == 0),
                "sample: %d logits take an 8-byte aligned workspace of iron_sample_workspace_bytes(n)", n);
+  IRON_REQUIRE(n_exprs == 0 || (words && exprs && n_words > 0 && n_exprs > 0),
+               "sample: %d word expressions take the words (%d of them) and the table", n_exprs, n_words);
   hipLaunchKernelGGL(sample_kernel, dim3(sample_blocks(n)), dim3(SAMPLE_THREADS), 0, (hipStream_t)stream,
                      logits, n, draws, draws_words, row, k_max, (uint64_t*)workspace, token, record,
-                     record_len, at, token_copy);
+                     record_len, at, token_copy, words, n_words, exprs, n_exprs);
   IRON_LAUNCH_CHECK();
+}
+
+extern "C" int iron_sample_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,
+                                const int* row, int k_max, void* workspace, int* token, int* record,
+                                int record_len, const int* at, int* token_copy, void* stream) {
+  return sample_launch(logits, n, draws, draws_words, row, k_max, workspace, token, record, record_len, at,
+                       token_copy, nullptr, 0, nullptr, 0, stream);
+}
+
+extern "C" int iron_sample_advance_bf16(const uint16_t* logits, int n, const int* draws, int draws_words,
+                                        const int* row, int k_max, void* workspace, int* token, int* record,
+                                        int record_len, const int* at, int* token_copy, int* words, int n_words,
+                                        const int* exprs, int n_exprs, void* stream) {
+  return sample_launch(logits, n, draws, draws_words, row, k_max, workspace, token, record, record_len, at,
+                       token_copy, words, n_words, exprs, n_exprs, stream);
 }

@@ -98,21 +98,27 @@ def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, r
 
 
 def decode_qkv(x, norm_w, Wq, Wk, Wv, angles, q_out, keys, values, *, eps, hidden, heads, kv_heads, d,
-               cache_rows, position):
-    """Attention's first half for one token: norm, q/k/v projections, RoPE, cache writes."""
+               cache_rows, position, angle_row=None):
+    """Attention's first half for one token: norm, q/k/v projections, RoPE, cache writes.  ``angles``
+    is the token's row of the RoPE table, or with ``angle_row`` (a device word) the whole table."""
     _numel(_dev(x, "x"), hidden, "x")
     _numel(_dev(norm_w, "norm_w"), hidden, "norm_w")
     _numel(_dev(Wq, "Wq"), heads * d * hidden, "Wq")
     _numel(_dev(Wk, "Wk"), kv_heads * d * hidden, "Wk")
     _numel(_dev(Wv, "Wv"), kv_heads * d * hidden, "Wv")
-    _numel(_dev(angles, "angles"), d, "angles")
+    _dev(angles, "angles")
+    if angle_row is None:
+        _numel(angles, d, "angles")
+    elif angles.numel() % d or angles.numel() < d:
+        raise ValueError(f"angles: a table of rows of {d}, got {angles.numel()} elements")
     _numel(_dev(q_out, "q_out"), heads * d, "q_out")
     _numel(_dev(keys, "keys"), cache_rows * kv_heads * d, "keys")
     _numel(_dev(values, "values"), cache_rows * kv_heads * d, "values")
     check(
         lib().iron_decode_qkv_bf16(ptr(x), ptr(norm_w), float(eps), ptr(Wq), ptr(Wk), ptr(Wv), ptr(angles),
                                    ptr(q_out), ptr(keys), ptr(values), hidden, heads, kv_heads, d, cache_rows,
-                                   ptr(_word(position, "position")), current_stream()),
+                                   ptr(_word(position, "position")), ptr(_word(angle_row, "angle_row")),
+                                   angles.numel() // d, current_stream()),
         "iron_decode_qkv_bf16",
     )
 
@@ -432,8 +438,10 @@ def sample_workspace(n, device="cuda"):
 
 
 def sample(logits, draws, token, *, n=None, row=None, k_max=64, workspace=None, record=None, at=None,
-           token_copy=None):
-    """The draw of ``draws``' row at word ``row`` (a device word, or None for the first row)."""
+           token_copy=None, advance=None):
+    """The draw of ``draws``' row at word ``row`` (a device word, or None for the first row).
+    ``advance``: ``(words, exprs, n)`` -- word expressions the same launch evaluates once the token is
+    written (``eval_words``'s, for the tail of a replayed decode step)."""
     n = logits.numel() if n is None else n
     _dev(logits, "logits")
     _dev(token, "token", torch.int32)
@@ -446,14 +454,19 @@ def sample(logits, draws, token, *, n=None, row=None, k_max=64, workspace=None, 
     need = lib().iron_sample_workspace_bytes(n)
     if workspace.numel() * workspace.element_size() < need:
         raise ValueError(f"workspace: {workspace.numel() * workspace.element_size()} bytes, need {need}")
-    check(
-        lib().iron_sample_bf16(
-            ptr(logits), n, ptr(draws), 0 if draws is None else draws.numel(), ptr(_word(row, "row")), k_max,
-            ptr(workspace), ptr(token), ptr(record), 0 if record is None else record.numel(),
-            ptr(_word(at, "at")), ptr(_word(token_copy, "token_copy")), current_stream(),
-        ),
-        "iron_sample_bf16",
-    )
+    common = (ptr(logits), n, ptr(draws), 0 if draws is None else draws.numel(), ptr(_word(row, "row")), k_max,
+              ptr(workspace), ptr(token), ptr(record), 0 if record is None else record.numel(),
+              ptr(_word(at, "at")), ptr(_word(token_copy, "token_copy")))
+    if advance is None:
+        check(lib().iron_sample_bf16(*common, current_stream()), "iron_sample_bf16")
+        return
+    words, exprs, count = advance
+    _dev(words, "words", torch.int32)
+    _dev(exprs, "exprs", torch.int32)
+    if exprs.numel() < 9 * count:
+        raise ValueError(f"exprs: {exprs.numel()} words hold fewer than {count} expressions of 9")
+    check(lib().iron_sample_advance_bf16(*common, ptr(words), words.numel(), ptr(exprs), count, current_stream()),
+          "iron_sample_advance_bf16")
 
 
 def eval_words(words, exprs, n=None):

@@ -3,7 +3,7 @@ hand-written HIP kernel."""
 
 from .axpy import AXPY
 from .clamp import Clamp
-from .copy import Copy
+from .copy import Copy, Gather, GatherWords
 from .elementwise_add import ElementwiseAdd, RowwiseAdd
 from .elementwise_mul import ElementwiseMul, RowwiseMul
 from .gelu import GELU
@@ -20,7 +20,8 @@ from .silu import SiLU
 from .softmax import Softmax
 from .tanh import Tanh
 
-__all__ = ["AXPY", "Clamp", "Copy", "ElementwiseAdd", "ElementwiseMul", "GELU", "GEMM", "GEMV", "LayerNorm", "MHA",
+__all__ = ["AXPY", "Clamp", "Copy", "ElementwiseAdd", "ElementwiseMul", "GELU", "GEMM", "GEMV", "Gather", "GatherWords",
+           "LayerNorm", "MHA",
            "RMSNorm", "ReLU", "RoPE", "RowwiseAdd", "RowwiseMul", "Sample", "Sigmoid", "SiLU", "Softmax", "Tanh"]
 
 #: Every operator by its class name (iron/operators/__init__.py:69-72).

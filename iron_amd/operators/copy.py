@@ -11,8 +11,10 @@ from __future__ import annotations
 import math
 from typing import Any
 
+import numpy as np
+
 from ..bf16 import bfloat16
-from ..common.declare import Built, In, Operator, Out, param, per_call
+from ..common.declare import Built, In, Operator, Out, param, per_call, tunable
 from ..common.testing import Case, Testing
 from ..common.verify import Tolerance
 
@@ -92,3 +94,99 @@ class Copy(Operator):
                               src_row=s_idx, dst_row=d_idx, valid=valid)
 
         return Built("iron_copy_rows", launch)
+
+
+class GatherWords(Operator):
+    """The step the reference records ahead of a ``Gather`` whose ids the device itself produced
+    (iron/operators/copy.py:380-470).  On the NPU it turns each id into DMA descriptor words.  A HIP
+    gather reads ids straight from memory, so here the control words ARE the ids: ``control``'s
+    first ``rows`` words receive them unchanged and the rest of the buffer is left alone.  The
+    address words of the reference (``base_lo`` / ``base_hi``) are accepted per call and unused."""
+
+    test = Testing([Case(dict(rows=16, table_rows=64, row_bytes=128, words=64))])
+
+    rows: int = param()
+    table_rows: int = param(array=True)
+    row_bytes: int = param(array=True)
+    words: int = param(default=lambda op: op.rows)
+    bounded: bool = param(default=False, array=True)
+
+    ids = In(rows, dtype=np.int32)
+    control = Out(words, dtype=np.int32)
+    base_lo = per_call(bounds=None)
+    base_hi = per_call(bounds=None)
+    valid_rows = per_call(bounds=rows)
+
+    def validate(self) -> None:
+        if not 1 <= self.rows <= self.words:
+            raise ValueError(f"GatherWords: rows ({self.rows}) must be from 1 to words ({self.words})")
+
+    def ops(self) -> int:
+        return 0
+
+    def tolerance(self) -> Tolerance:
+        return Tolerance.exact()
+
+    def build(self) -> Built:
+        from .. import kernels
+
+        rows = self.rows
+
+        def launch(t, words):
+            kernels.copy_rows(t["ids"].reshape(-1), t["control"].reshape(-1)[:rows], rows=rows, row_elems=1,
+                              src_rows=rows, dst_rows=rows, valid=words.get("valid_rows"))
+
+        return Built("iron_copy_rows", launch)
+
+
+class Gather(Operator):
+    """``y[i] = table[control[i]]`` for the first ``valid_rows`` of ``rows`` ids: the reference's
+    declared gather (iron/operators/copy.py:72-378), which ``Copy(table[ids])`` records implicitly.
+    ``control`` holds the ids in its first ``rows`` words (``GatherWords`` writes them, or the host).
+    A row whose id lies outside the table is left as it was.  ``feeds`` (pairs of shim columns on the
+    reference's device) is accepted and carried; one launch streams every row here."""
+
+    test = Testing([Case(dict(rows=16, table_rows=64, row=64)), Case(dict(rows=2048, table_rows=4096, row=2048), bench=True)])
+
+    rows: int = param()
+    table_rows: int = param()
+    row: int = param()
+    dtype: Any = param(default=bfloat16, repr=False)
+    words: int = param(default=lambda op: op.rows, repr=False)
+    feeds: int = tunable(default=1)
+
+    table = In(table_rows, row, dtype=dtype)
+    control = In(words, dtype=np.int32)
+    y = Out(rows, row, dtype=dtype)
+    valid_rows = per_call(bounds=rows)
+
+    def validate(self) -> None:
+        if self.rows < 1:
+            raise ValueError(f"Gather: rows ({self.rows}) must be at least 1")
+        if self.words < self.rows:
+            raise ValueError(f"Gather: {self.words} control words do not hold {self.rows} ids")
+        itemsize = 2 if self.dtype is bfloat16 else np.dtype(self.dtype).itemsize
+        if self.row * itemsize % 4:
+            raise ValueError(f"Gather: a row of {self.row} elements of {itemsize} bytes is not whole 32-bit words")
+
+    def word_source(self) -> GatherWords:
+        """The step that fills ``control`` from ids made on the device."""
+        itemsize = 2 if self.dtype is bfloat16 else np.dtype(self.dtype).itemsize
+        return GatherWords(rows=self.rows, table_rows=self.table_rows, row_bytes=self.row * itemsize,
+                           words=self.words)
+
+    def ops(self) -> int:
+        return 0   # a mover: its figure is bandwidth
+
+    def tolerance(self) -> Tolerance:
+        return Tolerance.exact()
+
+    def build(self) -> Built:
+        from .. import kernels
+
+        rows = self.rows
+
+        def launch(t, words):
+            kernels.gather_rows(t["table"], t["control"].reshape(-1)[:rows], t["y"], valid=words.get("valid_rows"))
+
+        return Built("iron_gather_rows", launch)

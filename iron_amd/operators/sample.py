@@ -112,9 +112,11 @@ class Sample(Operator):
                 ws = own.get("ws")
                 if ws is None:
                     ws = own["ws"] = kernels.sample_workspace(drawable, t["logits"].device)
-            # "__carry_token__": the scratchpad word a compiled loop carries the draw in, if it does.
+            # "__carry_token__": the scratchpad word a compiled loop carries the draw in, if it does;
+            # "__carry_eval__": the loop's word expressions, where the draw is the step's last launch.
             kernels.sample(t["logits"].reshape(-1), t["draws"].reshape(-1), t["token"].reshape(-1), n=drawable,
                            row=words.get("row"), k_max=k_max, workspace=ws, record=t["tokens"].reshape(-1),
-                           at=words.get("at"), token_copy=words.get("__carry_token__"))
+                           at=words.get("at"), token_copy=words.get("__carry_token__"),
+                           advance=words.get("__carry_eval__"))
 
         return Built("iron_sample_bf16", launch)

@@ -110,6 +110,24 @@ def copy(op, src):
     return np.array(src).reshape(op.shape)
 
 
+def gather(op, table, control, *, valid_rows=None):
+    """iron/operators/copy.py:72-378: the rows of ``table`` the first ``rows`` control words name;
+    rows past ``valid_rows`` are not written (zeros here)."""
+    ids = np.asarray(control).reshape(-1)[: op.rows].astype(np.int64)
+    n = op.rows if valid_rows is None else int(valid_rows)
+    y = np.zeros((op.rows, op.row), np.asarray(table).dtype)
+    y[:n] = np.asarray(table).reshape(op.table_rows, op.row)[ids[:n]]
+    return y
+
+
+def gather_words(op, ids, *, valid_rows=None, base_lo=0, base_hi=0):
+    """iron/operators/copy.py:380-470 as this build defines it: the ids themselves, first in ``control``."""
+    control = np.zeros(op.words, np.int32)
+    n = op.rows if valid_rows is None else int(valid_rows)
+    control[:n] = np.asarray(ids).reshape(-1)[:n]
+    return control
+
+
 def sample(op, logits, draws, tokens, *, row=0, at=0):
     """iron/operators/sample.py:72-79,324-333: the draw at ``draws`` word ``row``, recorded at ``at``."""
     words = np.asarray(draws).reshape(-1)[row : row + 4]
@@ -125,7 +143,7 @@ def install() -> None:
 
     REFERENCES.update(
         GEMM=gemm, GEMV=gemv, RMSNorm=rms_norm, SiLU=silu, ElementwiseMul=mul, ElementwiseAdd=add,
-        RoPE=rope, MHA=mha, Copy=copy, Sample=sample, RowwiseAdd=rowwise_add, RowwiseMul=rowwise_mul,
+        RoPE=rope, MHA=mha, Copy=copy, Gather=gather, GatherWords=gather_words, Sample=sample, RowwiseAdd=rowwise_add, RowwiseMul=rowwise_mul,
         GELU=gelu, ReLU=relu, Sigmoid=sigmoid, Tanh=tanh, Clamp=clamp, AXPY=axpy, LayerNorm=layer_norm,
         Softmax=softmax,
         # The host's draw, for iron_amd.lm.generation.Sampler's checks.

@@ -375,8 +375,12 @@ def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
     plain.load_versions(fuse=False)
     steps = len(fused.decode_step.recording.steps)
     assert plain.decode_step.launches_per_call == steps
-    # per layer 18 steps become 5 launches (qkv, attention, o+add, gate/up, down+add); the head 2 -> 1.
-    assert fused.decode_step.launches_per_call == 2 + 5 * SCALED.num_hidden_layers + 2
+    # per layer 18 steps become 5 launches (qkv, attention, o+add, gate/up, down+add); the head 2 -> 1;
+    # the RoPE row's copy is not launched (the projections read the table at the position themselves), and
+    # a replay ends with the draw, which evaluates the step's carried and derived words itself.
+    assert fused.decode_step.launches_per_call == 1 + 5 * SCALED.num_hidden_layers + 2
+    assert fused.decode_step.launches_per_replay == fused.decode_step.launches_per_call
+    assert plain.decode_step.launches_per_replay == steps
     # the prompt chunk: per layer the three projections, two rotations and two cache writes become
     # one launch, the feed-forward's SiLU and Mul another, each residual sum rides its projection's
     # epilogue, and the last row's final norm and head are one
@@ -435,6 +439,14 @@ def test_fused_kernels_against_the_oracle_at_llama_1b_width(cuda):
                  hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
                  position=torch.tensor([pos], dtype=torch.int32, device=cuda))
     close(q_out, ops.rope(ops.gemv(Wq, n).reshape(H, D), table[pos : pos + 1]).reshape(-1))
+    # ... and the same launch reading its row out of the whole table by a device word: the same bits
+    keys2, values2 = torch.zeros_like(keys), torch.zeros_like(values)
+    q2 = torch.empty_like(q_out)
+    K.decode_qkv(dev(x), dev(g), dev(Wq), dev(Wk), dev(Wv), dev(table), q2, keys2, values2, eps=1e-5,
+                 hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
+                 position=torch.tensor([pos], dtype=torch.int32, device=cuda),
+                 angle_row=torch.tensor([pos], dtype=torch.int32, device=cuda))
+    assert torch.equal(q2, q_out) and torch.equal(keys2, keys) and torch.equal(values2, values)
     kc, vc = from_torch(keys), from_torch(values)
     close(kc[pos], ops.rope(ops.gemv(Wk, n).reshape(G, D), table[pos : pos + 1]))
     close(vc[pos], ops.gemv(Wv, n).reshape(G, D))
