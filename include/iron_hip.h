@@ -121,6 +121,13 @@ int iron_rmsnorm_add_bf16(const uint16_t* x, const uint16_t* w, const uint16_t* 
 int iron_rope_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows, int cols,
                    int angle_rows, int two_halves, const int* valid, void* stream);
 
+/* The same over the first rotary_cols columns of rows row_cols wide (angles (angle_rows, rotary_cols));
+ * the columns past them are copied as they are.  (row_cols - rotary_cols) % 8 == 0.  A decoder whose
+ * RoPE covers part of each head: one launch for the reference's copy out, rotation and copy back
+ * (Attention.rotate, iron/lm/blocks.py:612-620). */
+int iron_rope_partial_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows, int row_cols,
+                           int rotary_cols, int angle_rows, int two_halves, const int* valid, void* stream);
+
 /* Elementwise over n elements (valid: elements computed), f32 math, one rounding each:
  *   silu: y = x*sigmoid(x)   mul: y = a*b   add: y = a+b
  *   silu_mul: y = bf16(bf16(silu(g)) * u)  -- SiLU then ElementwiseMul, rounded between,

@@ -32,6 +32,7 @@ SIGNATURES = {
     "iron_rmsnorm_bf16": (c_int, [_P, _P, _P, c_int, c_int, c_float, _P, _P]),
     "iron_rmsnorm_add_bf16": (c_int, [_P, _P, _P, _P, c_int, c_int, c_float, _P, _P]),
     "iron_rope_bf16": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P]),
+    "iron_rope_partial_bf16": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P]),
     "iron_silu_bf16": (c_int, [_P, _P, c_int64, _P, _P]),
     "iron_mul_bf16": (c_int, [_P, _P, _P, c_int64, _P, _P]),
     "iron_add_bf16": (c_int, [_P, _P, _P, c_int64, _P, _P]),

@@ -134,6 +134,7 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 ok = (
                     _same(rq.inputs["x"], q) and _same(rk.inputs["x"], k) and once(q) and once(k) and once(v)
                     and rq.op.two_halves and rk.op.two_halves and rq.op.angle_rows == 1 and rk.op.angle_rows == 1
+                    and rq.op.row == rq.op.cols and rk.op.row == rk.op.cols
                     and rk.op.cols == d and d in (64, 128) and not rq.values and not rk.values
                     and rq.inputs["angles"].buffer is rk.inputs["angles"].buffer and _plain(rq.inputs["angles"])
                     and _same(ck.inputs["src"], rk.outputs["y"]) and once(rk.outputs["y"])
@@ -199,7 +200,7 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 and M >= 64 and gq.op.K % 64 == 0 and gq.op.N % 128 == 0 and gk.op.N % 128 == 0
                 and gk.op.N == gv.op.N
                 and _same_view(rq.inputs["x"], q) and _same_view(rk.inputs["x"], k)
-                and all(r.op.two_halves and r.op.cols == d and r.op.angle_rows == M for r in (rq, rk))
+                and all(r.op.two_halves and r.op.cols == d and r.op.row == d and r.op.angle_rows == M for r in (rq, rk))
                 and rq.op.rows * d == M * gq.op.N and rk.op.rows * d == M * gk.op.N
                 and rq.inputs["angles"].buffer is rk.inputs["angles"].buffer
                 and _same_view(rq.inputs["angles"], rk.inputs["angles"])

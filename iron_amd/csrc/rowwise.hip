@@ -87,7 +87,7 @@ __global__ __launch_bounds__(256) void rope_kernel(const bf16_t* __restrict__ x,
                                                    const bf16_t* __restrict__ angles,
                                                    bf16_t* __restrict__ y, int rows, int cols,
                                                    int rows_per_angle,
-                                                   const int* __restrict__ valid) {
+                                                   const int* __restrict__ valid, int row_cols) {
   const int per_row = cols >> 4;  // threads a row takes
   const long t = (long)blockIdx.x * 256 + threadIdx.x;
   const long row = t / per_row;
@@ -101,8 +101,12 @@ __global__ __launch_bounds__(256) void rope_kernel(const bf16_t* __restrict__ x,
   unpack8(av[1], cs1);
   float c[8] = {cs0[0], cs0[2], cs0[4], cs0[6], cs1[0], cs1[2], cs1[4], cs1[6]};
   float s[8] = {cs0[1], cs0[3], cs0[5], cs0[7], cs1[1], cs1[3], cs1[5], cs1[7]};
-  const bf16_t* xr = x + (size_t)row * cols;
-  bf16_t* yr = y + (size_t)row * cols;
+  // A row is row_cols wide, of which the first cols turn; the rest passes through unchanged
+  // (a decoder whose RoPE covers part of each head), 16 bytes at a time over the row's threads.
+  const bf16_t* xr = x + (size_t)row * row_cols;
+  bf16_t* yr = y + (size_t)row * row_cols;
+  for (int c = cols + 8 * j; c < row_cols; c += 8 * per_row)
+    *reinterpret_cast<uint4*>(yr + c) = *reinterpret_cast<const uint4*>(xr + c);
   float a[8], b[8], oa[8], ob[8];
   if (TWO_HALVES) {
     const int half = cols >> 1;
@@ -254,13 +258,14 @@ extern "C" int iron_rmsnorm_add_bf16(const uint16_t* x, const uint16_t* w, const
   return rmsnorm(x, w, residual, y, rows, cols, eps, valid, stream);
 }
 
-extern "C" int iron_rope_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows,
-                              int cols, int angle_rows, int two_halves, const int* valid,
-                              void* stream) {
+static int rope_launch(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows, int row_cols, int cols,
+                       int angle_rows, int two_halves, const int* valid, void* stream) {
   IRON_REQUIRE(x && angles && y, "rope: null operand");
   IRON_REQUIRE(rows > 0 && cols > 0 && angle_rows > 0,
                "rope: rows (%d), cols (%d), angle_rows (%d) must be positive", rows, cols, angle_rows);
   IRON_REQUIRE(cols % 16 == 0, "rope: cols (%d) must be a multiple of 16", cols);
+  IRON_REQUIRE(row_cols >= cols && (row_cols - cols) % 8 == 0,
+               "rope: a row of %d columns of which %d turn: the rest must be a multiple of 8", row_cols, cols);
   IRON_REQUIRE(angle_rows <= rows && rows % angle_rows == 0,
                "rope: angle_rows (%d) must divide rows (%d)", angle_rows, rows);
   IRON_REQUIRE((((uintptr_t)x | (uintptr_t)angles | (uintptr_t)y) & 15) == 0,
@@ -270,11 +275,23 @@ extern "C" int iron_rope_bf16(const uint16_t* x, const uint16_t* angles, uint16_
   hipStream_t s = (hipStream_t)stream;
   if (two_halves)
     hipLaunchKernelGGL((rope_kernel<true>), dim3(blocks), dim3(256), 0, s, x, angles, y, rows, cols,
-                       rows / angle_rows, valid);
+                       rows / angle_rows, valid, row_cols);
   else
     hipLaunchKernelGGL((rope_kernel<false>), dim3(blocks), dim3(256), 0, s, x, angles, y, rows, cols,
-                       rows / angle_rows, valid);
+                       rows / angle_rows, valid, row_cols);
   IRON_LAUNCH_CHECK();
+}
+
+extern "C" int iron_rope_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows,
+                              int cols, int angle_rows, int two_halves, const int* valid,
+                              void* stream) {
+  return rope_launch(x, angles, y, rows, cols, cols, angle_rows, two_halves, valid, stream);
+}
+
+extern "C" int iron_rope_partial_bf16(const uint16_t* x, const uint16_t* angles, uint16_t* y, int rows,
+                                      int row_cols, int rotary_cols, int angle_rows, int two_halves,
+                                      const int* valid, void* stream) {
+  return rope_launch(x, angles, y, rows, row_cols, rotary_cols, angle_rows, two_halves, valid, stream);
 }
 
 extern "C" int iron_silu_bf16(const uint16_t* x, uint16_t* y, int64_t n, const int* valid,

@@ -183,17 +183,20 @@ def rmsnorm(x, w, y, *, rows, cols, eps, valid=None, residual=None):
     )
 
 
-def rope(x, angles, y, *, rows, cols, angle_rows, two_halves=True, valid=None):
-    _numel(_dev(x, "x"), rows * cols, "x")
+def rope(x, angles, y, *, rows, cols, angle_rows, two_halves=True, valid=None, row_cols=None):
+    """``cols`` columns of each row turn; ``row_cols`` (default: the same) is the whole row, whose
+    remaining columns pass through."""
+    row_cols = cols if row_cols is None else row_cols
+    _numel(_dev(x, "x"), rows * row_cols, "x")
     _numel(_dev(angles, "angles"), angle_rows * cols, "angles")
-    _numel(_dev(y, "y"), rows * cols, "y")
-    check(
-        lib().iron_rope_bf16(
-            ptr(x), ptr(angles), ptr(y), rows, cols, angle_rows, int(two_halves),
-            ptr(_word(valid, "valid")), current_stream(),
-        ),
-        "iron_rope_bf16",
-    )
+    _numel(_dev(y, "y"), rows * row_cols, "y")
+    if row_cols == cols:
+        check(lib().iron_rope_bf16(ptr(x), ptr(angles), ptr(y), rows, cols, angle_rows, int(two_halves),
+                                   ptr(_word(valid, "valid")), current_stream()), "iron_rope_bf16")
+    else:
+        check(lib().iron_rope_partial_bf16(ptr(x), ptr(angles), ptr(y), rows, row_cols, cols, angle_rows,
+                                           int(two_halves), ptr(_word(valid, "valid")), current_stream()),
+              "iron_rope_partial_bf16")
 
 
 def _binary(name):

@@ -70,11 +70,14 @@ class DecoderConfig:
     attention_bias: bool = False
     mlp_bias: bool = False
     sliding_window: int | None = None
+    # Partial rotary: RoPE turns only the first ``rotary_dim`` columns of each head (None: all of them).
+    # Not a config.json field; a model's own config class sets it from whatever its checkpoint calls it.
+    rotary_dim: int | None = None
 
     # field -> its key in config.json when that differs from the field's name.  None marks a field
     # that is this package's own choice: never read from a checkpoint, never written to one.
     JSON = {"eps": "rms_norm_eps", "max_seq_len": "max_position_embeddings", "precision": None,
-            "prefill_chunk": None}
+            "prefill_chunk": None, "rotary_dim": None}
 
     def __post_init__(self):
         fix = object.__setattr__           # the dataclass is frozen; these two are derived defaults
@@ -82,6 +85,10 @@ class DecoderConfig:
             fix(self, "head_dim", self.hidden_size // self.num_attention_heads)
         if self.prefill_chunk > self.max_seq_len:
             fix(self, "prefill_chunk", self.max_seq_len)
+        if self.rotary_dim is not None and not (0 < self.rotary_dim <= self.head_dim and self.rotary_dim % 16 == 0
+                                                and (self.head_dim - self.rotary_dim) % 8 == 0):
+            raise ValueError(f"{type(self).__name__}: rotary_dim {self.rotary_dim} of head_dim {self.head_dim}: a "
+                             "multiple of 16 that leaves a multiple of 8")
         if self.hidden_act not in _ACTIVATIONS:
             raise ValueError(f"{type(self).__name__}: hidden_act {self.hidden_act!r}: no operator here computes it")
 
@@ -157,7 +164,8 @@ class DecoderConfig:
 
     @property
     def rope_width(self) -> int:
-        return self.head_dim
+        """Width of the rotary table: the columns of a head that turn."""
+        return self.rotary_dim or self.head_dim
 
     def angles(self) -> np.ndarray | None:
         """This config's rotary table (a row per position), or None for a model without RoPE."""

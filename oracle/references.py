@@ -92,8 +92,14 @@ def rowwise_mul(op, x, row):
 
 
 def rope(op, x, angles):
-    """iron/operators/rope.py:167-184."""
-    return ops.rope(x, angles, two_halves=op.two_halves)
+    """iron/operators/rope.py:167-184; with a row wider than the table, the first columns turn and the
+    rest pass through (the reference's Attention.rotate, iron/lm/blocks.py:612-620)."""
+    x = np.asarray(x)
+    if op.row == op.cols:
+        return ops.rope(x, angles, two_halves=op.two_halves)
+    y = np.array(x, dtype=np.float32).reshape(op.rows, op.row)
+    y[:, : op.cols] = ops.rope(y[:, : op.cols], angles, two_halves=op.two_halves)
+    return y
 
 
 def mha(op, Q, K, V):

@@ -362,6 +362,29 @@ def test_rmsnorm_bound(cuda):
     assert np.all(got[5:] == 3.0)
 
 
+@pytest.mark.parametrize("rows,row,cols,angle_rows,halves", [(64, 128, 32, 2, True), (32, 64, 32, 1, True), (96, 256, 64, 96, True),
+                                                             (40, 80, 16, 5, False), (2048 * 8, 64, 32, 2048, True)])
+def test_rope_over_the_first_columns_of_each_row(cuda, rows, row, cols, angle_rows, halves):
+    """Partial rotary: the first ``cols`` columns of a ``row``-wide row turn exactly as a row of that
+    width would, the rest come through bit for bit; rows past a bound are left alone."""
+    rng = np.random.default_rng(rows + row)
+    x = bf(rng, rows, row)
+    table = round_bf16(ops.rope_angles(cols, angle_rows + 3, 10000.0))[3:]
+    bound = rows - rows // 3
+    y = out_like((rows, row), cuda, fill=9.0)
+    K.rope(dev(x, cuda), dev(table, cuda), y, rows=rows, cols=cols, angle_rows=angle_rows, two_halves=halves,
+           valid=word(bound, cuda), row_cols=row)
+    got = from_torch(y)
+    want = ops.rope(x[:, :cols], table, two_halves=halves)
+    close(got[:bound, :cols], want[:bound])
+    assert np.array_equal(got[:bound, cols:], x[:bound, cols:]) and np.all(got[bound:] == 9.0)
+    # ... and the turned columns are the bits the whole-row launch gives a row of that width
+    narrow = out_like((rows, cols), cuda)
+    K.rope(dev(np.ascontiguousarray(x[:, :cols]), cuda), dev(table, cuda), narrow, rows=rows, cols=cols,
+           angle_rows=angle_rows, two_halves=halves)
+    assert np.array_equal(got[:bound, :cols], from_torch(narrow)[:bound])
+
+
 @pytest.mark.parametrize("rows,cols,weighted,bound", [(1, 2048, True, None), (64, 512, True, 40), (7, 8192, False, None)])
 def test_rmsnorm_with_its_residual(cuda, rows, cols, weighted, bound):
     """The normed rows added to a residual in the norm's own pass: bit for bit the norm launch

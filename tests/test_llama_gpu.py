@@ -263,7 +263,10 @@ def test_refusals_before_any_dispatch(toy):
     # a window short enough against the context that the layers keep rings (128 rows, wrapped by the 200-token prompt)
     dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=2, head_dim=64, intermediate_size=1024,
          sliding_window=20, max_seq_len=1024),
-], ids=["d128", "twelve_heads_untied", "multi_query_window", "ring"])
+    # RoPE over the first half of each head only (partial rotary): one RoPE step turns 32 of 64 columns
+    dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=2, head_dim=64, intermediate_size=1024,
+         rotary_dim=32),
+], ids=["d128", "twelve_heads_untied", "multi_query_window", "ring", "partial_rotary"])
 def test_other_decoder_shapes_match_the_host_reference(cuda, shape):
     """Shapes off the benchmark's: every fused path either takes the shape or leaves the steps as
     recorded; either way the GPU's logits are the host reference's, prompt (in two chunks) and decode."""

@@ -215,3 +215,37 @@ def test_a_profile_in_the_reference_s_format_fills_the_open_tunables_of_recorded
     both.add(GEMV, K=Q, tile_size_input=4)
     with pytest.raises(ValueError, match="ambiguous"):
         both.tunables_for(GEMV, dict(M=E, K=Q))
+
+
+def test_partial_rotary_narrows_the_table_and_turns_the_leading_columns_in_one_step():
+    """``rotary_dim``: the angle table is that wide (iron/tests/common/test_decoder.py:51-66), the
+    weights keep the whole head, and q and k each take ONE RoPE step over rows a head wide of which
+    the leading columns turn (the reference copies them out, rotates and copies back,
+    iron/lm/blocks.py:612-620); the step's reference is the rotation of those columns alone."""
+    import dataclasses
+
+    import oracle
+    from iron_amd.bf16 import round_bf16
+    from iron_amd.lm.config import rope_angles
+    from oracle import ops
+
+    oracle.install()
+    model = small(rotary_dim=32)
+    cfg = model.config
+    assert cfg.rope_width == 32 and cfg.angles().shape == (cfg.max_seq_len, 32)
+    assert np.array_equal(cfg.angles(), rope_angles(32, cfg.max_seq_len, cfg.rope_theta, cfg.rope_scaling))
+    assert model.layers[0].self_attn.q_proj.weight.shape == (cfg.num_attention_heads * cfg.head_dim, cfg.hidden_size)
+    assert small().config.rotary_dim is None and small().config.rope_width == cfg.head_dim
+    for shapes in model.shapes():
+        t = model.record(**shapes)
+        ropes = [s.op for s in t.steps if type(s.op).__name__ == "RoPE"]
+        assert len(ropes) == 2 * cfg.num_hidden_layers
+        assert all(op.cols == 32 and op.row == cfg.head_dim for op in ropes)
+    op = ropes[0]
+    rng = np.random.default_rng(0)
+    x = round_bf16(rng.standard_normal((op.rows, op.row)).astype(np.float32))
+    table = round_bf16(rope_angles(32, op.angle_rows, cfg.rope_theta))
+    got = np.asarray(op.reference(x, table)).reshape(op.rows, op.row)
+    assert np.array_equal(got[:, :32], ops.rope(x[:, :32], table)) and np.array_equal(got[:, 32:], x[:, 32:])
+    with pytest.raises(ValueError, match="rotary_dim"):
+        dataclasses.replace(cfg, rotary_dim=40)
