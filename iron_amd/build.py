@@ -29,6 +29,12 @@ FLAGS = [
     "-target-feature",
     "-Xclang",
     "-packed-fp32-ops",
+    # The first 16 dwords of a kernel's arguments arrive in SGPRs with the wave instead of by a
+    # scalar load the kernel's first instructions wait for: about a memory trip off every launch of a
+    # chain of short dependent kernels.  (A kernel keeps a prologue that loads them for hardware
+    # that does not preload.)
+    "-mllvm",
+    "-amdgpu-kernarg-preload-count=16",
 ]
 
 

@@ -129,6 +129,12 @@ __device__ __forceinline__ int bound_or(const int* p, int whole) {
 #define IRON_GLOBAL_PTR(p) ((const void __attribute__((address_space(1)))*)(p))
 #define IRON_LDS_PTR(p) ((void __attribute__((address_space(3)))*)(p))
 
+// Rows of a matrix from `base` on as a raw buffer (no stride, 2 GiB of reach, 32-bit data): what a
+// buffer load into LDS addresses with a 32-bit offset a lane.  `base` must be uniform over the wave.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stage_rows(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+
 __device__ __forceinline__ void block_barrier() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();

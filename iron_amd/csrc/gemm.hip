@@ -373,36 +373,49 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
   }
   const int n0 = tn * NT_BN;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // The wave's number is uniform, so what depends on it (LDS destinations, the rows it loads) stays
+  // in scalar registers.
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane >> 3, pch = lane & 7;
-  const bf16_t* a_src[INST];
-  const bf16_t* b_src[INST];
+  // Loads are buffer loads straight into LDS.  The buffer is the tile's rows from the stage's k on
+  // (rebuilt once a stage with scalar instructions); a lane's place in it never changes, so it is a
+  // constant 32-bit vector offset and a load costs one scalar add (its LDS destination) on top of
+  // itself -- no vector ALU work between two MFMAs.
+  int a_voff[INST], b_voff[INST];
 #pragma unroll
   for (int i = 0; i < INST; ++i) {
     const int r = (wave * INST + i) * 8 + lrow;
     const int lch = pch ^ ((r >> 1) & 7);
     // Rows past the end re-read the last row; what they produce is never stored.
-    a_src[i] = A + (size_t)min(m0 + r, M - 1) * K + lch * 8;
+    a_voff[i] = (int)(((size_t)(min(m0 + r, M - 1) - m0) * K + lch * 8) * 2);
     if constexpr (!B_KN) {
-      b_src[i] = B + (size_t)min(n0 + r, N - 1) * K + lch * 8;
+      b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
     } else {
       const int kr = (wave * INST + i) * 4 + (lane >> 4);       // k row of the tile
       const int lc = (lane & 15) ^ ((kr & 7) << 1);               // logical 16-byte chunk (8 n)
-      b_src[i] = B + (size_t)kr * N + n0 + lc * 8;
+      b_voff[i] = (int)(((size_t)kr * N + lc * 8) * 2);
     }
   }
+  const bf16_t* a_tile = A + (size_t)m0 * K;
+  const bf16_t* b_tile = B_KN ? B + n0 : B + (size_t)n0 * K;
+  // One load of the 2*INST a wave issues per stage (A's first, then B's).
+  auto issue_one = [&](char* st, int kt, int idx) {
+    const int k0 = kt * BK;
+    if (idx < INST) {
+      const __amdgpu_buffer_rsrc_t rows = stage_rows(a_tile + k0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16,
+                                               (int)a_voff[idx], 0, 0, 0);
+    } else {
+      const __amdgpu_buffer_rsrc_t rows = stage_rows(b_tile + (B_KN ? (size_t)k0 * N : (size_t)k0));
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024),
+                                               16, (int)b_voff[idx - INST], 0, 0, 0);
+    }
+  };
   auto issue = [&](int kt, int buf) {
     char* st = smem_nt + buf * NT_STAGE_BYTES;
-    const int k0 = kt * BK;
 #pragma unroll
-    for (int i = 0; i < INST; ++i)
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_src[i] + k0),
-                                       IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < INST; ++i)
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(b_src[i] + (B_KN ? (size_t)k0 * N : (size_t)k0)),
-                                       IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + i) * 1024), 16, 0, 0);
+    for (int idx = 0; idx < 2 * INST; ++idx) issue_one(st, kt, idx);
   };
 
   f32x16 acc[T][T];
@@ -452,17 +465,6 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
 #pragma unroll
   for (int i = 0; i < T; ++i) tr_n[i] = wn * 64 + i * 32 + (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
 
-  // One load of the 2*INST a wave issues per stage (A's first, then B's).
-  auto issue_one = [&](char* st, int kt, int idx) {
-    const int k0 = kt * BK;
-    if (idx < INST)
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_src[idx] + k0),
-                                       IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16, 0, 0);
-    else
-      __builtin_amdgcn_global_load_lds(
-          IRON_GLOBAL_PTR(b_src[idx - INST] + (B_KN ? (size_t)k0 * N : (size_t)k0)),
-          IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
-  };
   auto read_frag_pair = [&](const char* st, int ks, int i, bf16x8& a, bf16x8& b, TrFrag& t) {
     const int j = ks * 2 + kh;
     a = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
@@ -673,7 +675,7 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
   const int m0 = tm * Q3_BM;
   if (m0 >= Mv) return;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane >> 3, pch = lane & 7;
   // Head g of the concatenated list: its weight rows and where its 64 columns go.
   auto head_weight = [&](int g) {
@@ -681,26 +683,34 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
     if (g < heads + kv_heads) return qkv.Bk + (size_t)(g - heads) * 64 * K;
     return qkv.Bv + (size_t)(g - heads - kv_heads) * 64 * K;
   };
-  const bf16_t* a_src[A_INST];
-  const bf16_t* b_src[B_INST];
+  // Buffer loads straight into LDS (see gemm_nt_body): the activations' tile rows are one buffer;
+  // the eight weight rows of an instruction lie in one head, so each of a wave's weight
+  // instructions has its own buffer, which starts at its first row.  The stage's k is the scalar
+  // offset, a lane's place the constant vector offset.
+  const __amdgpu_buffer_rsrc_t a_rows = stage_rows(A + (size_t)m0 * K);
+  __amdgpu_buffer_rsrc_t b_rows[B_INST];
+  int a_voff[A_INST], b_voff[B_INST];
 #pragma unroll
   for (int i = 0; i < A_INST; ++i) {
     const int r = (wave * A_INST + i) * 8 + lrow;
-    a_src[i] = A + (size_t)min(m0 + r, M - 1) * K + (pch ^ ((r >> 1) & 7)) * 8;
+    a_voff[i] = (int)(((size_t)(min(m0 + r, M - 1) - m0) * K + (pch ^ ((r >> 1) & 7)) * 8) * 2);
   }
 #pragma unroll
   for (int i = 0; i < B_INST; ++i) {
-    const int r = (wave * B_INST + i) * 8 + lrow;   // row of the tile's weight rows: head r / 64, its row r % 64
-    b_src[i] = head_weight(tn * HPT + r / 64) + (size_t)(r % 64) * K + (pch ^ ((r >> 1) & 7)) * 8;
+    const int r0 = (wave * B_INST + i) * 8;   // first of the instruction's rows among the tile's weight rows: head r0 / 64, its row r0 % 64
+    const int r = r0 + lrow;
+    b_rows[i] = stage_rows(head_weight(tn * HPT + r0 / 64) + (size_t)(r0 % 64) * K);
+    b_voff[i] = (int)(((size_t)lrow * K + (pch ^ ((r >> 1) & 7)) * 8) * 2);
   }
   auto issue_one = [&](char* st, int kt, int idx) {
-    const int k0 = kt * BK;
+    const int k_off = kt * BK * 2;
     if (idx < A_INST)
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_src[idx] + k0),
-                                       IRON_LDS_PTR(st + (wave * A_INST + idx) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rows, IRON_LDS_PTR(st + (wave * A_INST + idx) * 1024), 16,
+                                               (int)a_voff[idx], k_off, 0, 0);
     else
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(b_src[idx - A_INST] + k0),
-                                       IRON_LDS_PTR(st + Q3_A_BYTES + (wave * B_INST + idx - A_INST) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rows[idx - A_INST],
+                                               IRON_LDS_PTR(st + Q3_A_BYTES + (wave * B_INST + idx - A_INST) * 1024), 16,
+                                               (int)b_voff[idx - A_INST], k_off, 0, 0);
   };
 
   f32x16 acc[NACC];
@@ -990,7 +1000,7 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   const int m0 = tm * BIG_BM, n0 = tn * BIG_BN;
   if (m0 >= Mv) return;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS and global bases stay in scalar registers
   const int wm = wave / (WAVES / 2), wn = wave % (WAVES / 2);
   // Loader: instruction i of a wave moves rows (wave*INST + i)*RPI .. ; lane -> (row, physical
   // chunk); the logical chunk it fetches is the physical one swizzled by the row.
@@ -1001,18 +1011,21 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
     const int r = par * RPI + lrow;
     ld_off[par] = (unsigned)(((size_t)lrow * K + (pch ^ ((r >> 1) & (CPR - 1))) * 8) * 2);
   }
-  const char* a_base = reinterpret_cast<const char*>(A + (size_t)(m0 + wave * INST * RPI) * K);
-  const char* b_base = reinterpret_cast<const char*>(B + (size_t)(n0 + wave * INST * RPI) * K);
-  const size_t inst_stride = (size_t)RPI * K * 2;
+  // Loads go out as buffer loads straight into LDS: the rows a wave fetches are one buffer, the
+  // lane's place within an instruction's rows is the (constant) vector offset and the instruction's
+  // rows and the stage's k are the scalar offset, so a load costs two scalar adds and no vector ALU
+  // work between two MFMAs.
+  const __amdgpu_buffer_rsrc_t a_rows = stage_rows(A + (size_t)(m0 + wave * INST * RPI) * K);
+  const __amdgpu_buffer_rsrc_t b_rows = stage_rows(B + (size_t)(n0 + wave * INST * RPI) * K);
+  const int inst_stride = RPI * K * 2;
   auto issue_one = [&](char* st, int kt, int idx) {
-    const size_t k_off = (size_t)kt * KB * 2;
+    const int k_off = kt * KB * 2;
     if (idx < INST)
-      __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(a_base + idx * inst_stride + k_off + ld_off[idx & 1]),
-                                       IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rows, IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16,
+                                               (int)ld_off[idx & 1], idx * inst_stride + k_off, 0, 0);
     else
-      __builtin_amdgcn_global_load_lds(
-          IRON_GLOBAL_PTR(b_base + (idx - INST) * inst_stride + k_off + ld_off[idx & 1]),
-          IRON_LDS_PTR(st + A_BYTES + (wave * INST + idx - INST) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rows, IRON_LDS_PTR(st + A_BYTES + (wave * INST + idx - INST) * 1024),
+                                               16, (int)ld_off[idx & 1], (idx - INST) * inst_stride + k_off, 0, 0);
   };
 
   f32x16 acc[4][TN];
@@ -1217,6 +1230,8 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   IRON_REQUIRE(A && B && C, "gemm: null operand");
   IRON_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: M (%d), N (%d), K (%d) must be positive", M, N, K);
   IRON_REQUIRE(K % 8 == 0, "gemm: K (%d) must be a multiple of 8 (16-byte loads)", K);
+  IRON_REQUIRE(K <= (1 << 22) && N <= (1 << 22),
+               "gemm: K (%d) and N (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", K, N);
   IRON_REQUIRE((((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) == 0,
                "gemm: operands must be 16-byte aligned");
   IRON_REQUIRE(b_col_maj || N % 8 == 0,
@@ -1263,6 +1278,8 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
 extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
                                        int N, int K, float residual_scale, const int* valid, void* stream) {
   IRON_REQUIRE(A && B && R && C, "gemm_residual: null operand");
+  IRON_REQUIRE(K <= (1 << 22) && N <= (1 << 22),
+               "gemm_residual: K (%d) and N (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", K, N);
   IRON_REQUIRE(M >= 64 && N >= 64 && K > 0 && K % BK == 0,
                "gemm_residual: M (%d) and N (%d) at least 64, K (%d) a positive multiple of %d", M, N, K, BK);
   IRON_REQUIRE((((uintptr_t)A | (uintptr_t)B | (uintptr_t)R | (uintptr_t)C) & 15) == 0,
@@ -1292,6 +1309,7 @@ static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk
                "prefill_qkv: rows (%d) at least 64; heads (%d) and kv_heads (%d) positive and even "
                "(whole 128-column tiles)", rows, heads, kv_heads);
   IRON_REQUIRE(hidden > 0 && hidden % BK == 0, "prefill_qkv: hidden (%d) must be a positive multiple of %d", hidden, BK);
+  IRON_REQUIRE(hidden <= (1 << 22), "prefill_qkv: hidden (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", hidden);
   IRON_REQUIRE((((uintptr_t)x | (uintptr_t)Wq | (uintptr_t)Wk | (uintptr_t)Wv | (uintptr_t)angles |
                  (uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)v_out) & 15) == 0,
                "prefill_qkv: operands must be 16-byte aligned");

@@ -54,7 +54,10 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   extern __shared__ __align__(1024) char smem_all[];   // SPLIT * STAGES * STAGE bytes
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int half = (tid >> 6) >> 2, wave = (tid >> 6) & 3;   // which tiles, and which 32 queries
+  // Which tiles, and which 32 queries -- uniform over the wave, so what depends on them (LDS
+  // destinations, the rows a wave loads) stays in scalar registers.
+  const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = wave_id >> 2, wave = wave_id & 3;
   char* smem = smem_all + half * (STAGES * STAGE);            // this half's stage buffers
   const int col = lane & 31, g = lane >> 5;
   // Blocks are dispatched in id order, so the id runs over the query blocks from the last (under a
@@ -127,33 +130,35 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
     const bf16_t* Kh = K + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
     const bf16_t* Vh = V + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
 
-    // Loader: load i of a wave covers tile rows (wave*INST + i)*RPI .. ; lane -> (row, physical
-    // chunk), and fetches the logical chunk that the row's swizzle maps there.  Rows past the
-    // last key re-read it: finite values that the mask below turns into zero weights.
+    // Loader: buffer loads straight into LDS.  Load i of a wave covers tile rows
+    // (wave*INST + i)*RPI .. ; lane -> (row, physical chunk), and fetches the logical chunk that
+    // the row's swizzle maps there.  The buffer is the tile's rows of this head up to the last key
+    // (rebuilt per tile with scalar instructions): a lane's place in it is a constant 32-bit
+    // offset, and rows past the last key -- only the last tile can hold any -- lie outside the
+    // buffer and read as zeros, which the mask below turns into zero weights.
     const int l_row = lane / CPR, l_pch = lane % CPR;
-    // Per load: where tile 0's row starts (K and V share it), the same for the last tile with rows
-    // past the last key clamped to it, and the swizzled column of K and of V.
-    long row0[INST], row_last[INST];
-    int k_col[INST], v_col[INST];
+    const int row_bytes = (int)kv_row_stride * 2;
+    int k_voff[INST], v_voff[INST];
 #pragma unroll
     for (int i = 0; i < INST; ++i) {
       const int r = (wave * INST + i) * RPI + l_row;
-      row0[i] = (long)(kv_lo + r) * kv_row_stride;
-      row_last[i] = (long)min(kv_lo + (ntiles - 1) * BKV + r, kv_tokens - 1) * kv_row_stride;
-      k_col[i] = (l_pch ^ ((r >> 1) & 7)) * 8;
-      v_col[i] = (l_pch ^ ((r & 3) << 1)) * 8;
+      k_voff[i] = r * row_bytes + (l_pch ^ ((r >> 1) & 7)) * 16;
+      v_voff[i] = r * row_bytes + (l_pch ^ ((r & 3) << 1)) * 16;
     }
-    const long tile_stride = (long)BKV * kv_row_stride;
     auto issue = [&](int tile, int buf) {
       char* st = smem + buf * STAGE;
-      const bool last = tile == ntiles - 1;   // only the last tile can hold rows past the last key
+      const int first = kv_lo + tile * BKV;
+      const int reach = (min(BKV, kv_tokens - first) - 1) * row_bytes + ROWB;   // bytes up to the last key's row end
+      const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<bf16_t*>(Kh + (long)first * kv_row_stride), 0, reach, 0x00020000);
+      const __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<bf16_t*>(Vh + (long)first * kv_row_stride), 0, reach, 0x00020000);
 #pragma unroll
       for (int i = 0; i < INST; ++i) {
-        const long row = last ? row_last[i] : row0[i] + tile * tile_stride;
-        __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(Kh + row + k_col[i]),
-                                         IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(IRON_GLOBAL_PTR(Vh + row + v_col[i]),
-                                         IRON_LDS_PTR(st + TILE + (wave * INST + i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rows, IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16,
+                                                 (int)k_voff[i], 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rows, IRON_LDS_PTR(st + TILE + (wave * INST + i) * 1024), 16,
+                                                 (int)v_voff[i], 0, 0, 0);
       }
     };
     // Always STAGES-1 tiles in flight before the loop and one more each iteration (past the end
@@ -403,6 +408,7 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
   const long q_head = q_interleaved ? d : (long)seq * d;
   const long kv_row = kv_interleaved ? (long)kv_heads * d : d;
   const long kv_head = kv_interleaved ? d : (long)kv_len * d;
+  IRON_REQUIRE(kv_row <= (1L << 20), "mha_prefill: a key row spans %ld values, more than the 2^20 a tile's 32-bit offsets reach", kv_row);
   const float scale_log2 = scale * 1.4426950408889634f;
   if (d == 512) {
     IRON_REQUIRE(seq <= 65535, "mha_prefill: at d = 512 seq (%d) is a grid dimension, at most 65535", seq);
