@@ -492,7 +492,13 @@ PROBE_COPY_BYTES = 512 << 20
 # HBM bytes one launch moves, by kernel, from hardware counters (FETCH_SIZE and WRITE_SIZE per
 # dispatch, each scaled by what the same counter reads for a plain copy of PROBE_COPY_BYTES): filled
 # from counter runs of `--decode-probe` / `--counter-probe`; a kernel without a reading reports null.
-DOMINANT_TRAFFIC_BYTES: dict[str, int] = {}
+DOMINANT_TRAFFIC_BYTES: dict[str, int] = {
+    "gemv_fused_kernel<2,1,true,2>": 67_358_000,     # norm + gate/up + SiLU*mul: 67.227 MB fetched + 0.131 written
+    "gemv_fused_kernel<1,4,false,1>": 33_788_000,    # down projection + residual: 33.755 + 0.033
+    "gemv_fused_kernel<4,1,true,0>": 526_460_000,    # final norm + LM head: 525.43 + 1.03
+    "decode_qkv_kernel<64,1>": 12_750_000,           # norm + q/k/v + RoPE + cache rows: 12.70 + 0.05
+    "gemv_fused_kernel<1,1,false,1>": 8_500_000,     # o projection + residual: 8.47 + 0.03
+}
 
 
 def counter_probe(torch, K, dev, rng):

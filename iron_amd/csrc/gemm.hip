@@ -964,6 +964,16 @@ constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stage
 #define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
 constexpr int BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
 
+// acc += a b on the 16x16x32 MFMA, the accumulator held in place in accumulation registers.  As a
+// builtin, sixty-four 4-register accumulators live across a loop make the register allocator
+// rotate them through copies (some 200 moves an iteration); a tied operand leaves it no choice.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void mfma_16x16x32_in_place(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+               : "+a"(acc)
+               : "v"(__builtin_bit_cast(i32x4, a)), "v"(__builtin_bit_cast(i32x4, b)));
+}
+
 template <int WAVES, int KB>
 __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                 bf16_t* __restrict__ C, int M, int N, int K,
@@ -977,7 +987,6 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   constexpr int STAGES = KB == 64 ? 2 : 4;   // 128 KB either way
   constexpr int INST = BIG_BM / RPI / WAVES; // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int TN = 8 / WAVES * 2;          // 32-column MFMA tiles a wave owns along n (4 or 2)
-  constexpr int KSTEPS = KB / 16;
   extern __shared__ __align__(16) char smem_big[];
   const int Mv = bound_or(valid, M);
   if (Mv <= run_above || Mv > run_upto) return;
@@ -1028,72 +1037,85 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
                                                16, (int)ld_off[idx & 1], (idx - INST) * inst_stride + k_off, 0, 0);
   };
 
-  f32x16 acc[4][TN];
+  // The product runs on 16x16x32 MFMAs (a k-step is 32 wide, two a stage): on random operands the
+  // part sustains about a sixth more of them than of the 32x32x16 form, at the same registers and
+  // the same LDS reads per flop.  A wave's 128 x 128 is 8 x NT tiles of 16 x 16.
+  constexpr int NT = TN * 2;                 // 16-column tiles a wave owns along n
+  f32x4 acc[8][NT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
   const int nk = K / KB;
-  static_assert(KB == 64, "the loop below is written for two 64-wide stages");
-  // A stage's 2 INST loads go out in two halves of INST: the first under the last k-step of the
+  static_assert(KB == 64 && INST == 8 && TN == 4, "the loop below is written for two 64-wide stages and four waves");
+  // A stage's 2 INST loads go out in two halves of INST: the first under the last quarter of the
   // stage two before it (right after that stage's barrier freed the buffer), the second under the
-  // first k-step of the stage before it; two k-steps later, at that stage's barrier, all have landed.
+  // first quarter of the stage before it; two quarters later, at that stage's barrier, all have landed.
   auto issue_half = [&](char* st, int kt, int half, int slot) { issue_one(st, kt, half * INST + slot); };
 #pragma unroll
   for (int idx = 0; idx < 2 * INST; ++idx) issue_one(smem_big, 0, idx);
 #pragma unroll
   for (int slot = 0; slot < INST; ++slot) issue_half(smem_big + STAGE_BYTES, min(1, nk - 1), 0, slot);
 
-  const int fr = lane & 31, kh = lane >> 5;
-  const int swz = (fr >> 1) & (CPR - 1);   // tile rows are multiples of 32 apart: one swizzle for all
-  const int a_row = (wm * 128 + fr) * ROWB, b_row = A_BYTES + (wn * TN * 32 + fr) * ROWB;
-  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[4], bf16x8 (&bfr)[TN]) {
-    const int c = ((ks * 2 + kh) ^ swz) << 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(st + a_row + i * 32 * ROWB + c);
-#pragma unroll
-    for (int i = 0; i < TN; ++i) bfr[i] = *reinterpret_cast<const bf16x8*>(st + b_row + i * 32 * ROWB + c);
+  // Fragments: lane -> row fr of a 16-row tile, 16-byte chunk kq of the k-step's four.
+  const int fr = lane & 15, kq = lane >> 4;
+  const int swz = (fr >> 1) & (CPR - 1);   // tile rows are multiples of 16 apart: one swizzle for all
+  const int a_row = (wm * 128 + fr) * ROWB, b_row = A_BYTES + (wn * NT * 16 + fr) * ROWB;
+  auto a_frag = [&](const char* st, int ks, int i) {
+    return *reinterpret_cast<const bf16x8*>(st + a_row + i * 16 * ROWB + (((ks * 4 + kq) ^ swz) << 4));
+  };
+  auto b_frag = [&](const char* st, int ks, int j) {
+    return *reinterpret_cast<const bf16x8*>(st + b_row + j * 16 * ROWB + (((ks * 4 + kq) ^ swz) << 4));
   };
 
   wait_vmcnt<INST>();   // stage 0 has landed once only stage 1's first half is out
   block_barrier();
-  bf16x8 af[2][4], bfr[2][TN];
-  read_frags(smem_big, 0, af[0], bfr[0]);
+  bf16x8 af[2][8], bfr[2][NT];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) af[0][i] = a_frag(smem_big, 0, i);
+#pragma unroll
+  for (int j = 0; j < NT; ++j) bfr[0][j] = b_frag(smem_big, 0, j);
   for (int kt = 0; kt < nk; ++kt) {
     // Past the end the last stage is fetched again (into buffers nobody reads any more) rather than
     // branch: a branch would end the scheduling region and undo the interleaving below.
     const int k1 = min(kt + 1, nk - 1), k2 = min(kt + 2, nk - 1);
     char* st = smem_big + (kt % STAGES) * STAGE_BYTES;          // this stage; then stage kt+2's buffer
     char* nst = smem_big + ((kt + 1) % STAGES) * STAGE_BYTES;   // stage kt+1's
+    // A stage is two k-steps of 64 MFMAs, scheduled as four quarters of 32 (tile rows 0..3 and 4..7
+    // of a k-step).  Source order is issue order (nothing crosses a sched_barrier): after an MFMA
+    // one fragment read or one load goes out.
+    //   quarter 0: the second k-step's B fragments, and the second half of stage kt+1's loads
+    //   quarter 1: the second k-step's A fragments
+    //   quarter 2: nothing -- then the stage's one barrier: every wave's loads of stage kt+1 have
+    //              landed and nobody reads stage kt any more (the last quarter's fragments are in registers)
+    //   quarter 3: stage kt+1's first fragments, and the first half of stage kt+2's loads
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-      const bool last = ks + 1 == KSTEPS;
-      if (last) {
-        // The one barrier of the stage, before its last k-step (whose fragments are in registers):
-        // after it every wave's loads of stage kt+1 have landed and nobody reads stage kt any more.
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        wait_vmcnt<0>();
-        block_barrier();
-      }
-      const char* from = last ? nst : st;
-      const int c = (((last ? 0 : ks + 1) * 2 + kh) ^ swz) << 4;
-      // Source order is issue order (nothing crosses a sched_barrier): after each MFMA one of the
-      // next k-step's fragment reads (the next stage's first, under the last k-step) or one load goes out.
+    for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 8; ++i) {
+        const int quarter = ks * 2 + (i >> 2), q = i & 3;   // q: the quarter's tile row
+        if (quarter == 3 && q == 0) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          wait_vmcnt<0>();
+          block_barrier();
+        }
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < NT; ++j) {
+          mfma_16x16x32_in_place(acc[i][j], bfr[ks][j], af[ks][i]);
           __builtin_amdgcn_sched_barrier(0);
-          if (j == 0) af[nxt][i] = *reinterpret_cast<const bf16x8*>(from + a_row + i * 32 * ROWB + c);
-          if (j == 1 && i < TN) bfr[nxt][i] = *reinterpret_cast<const bf16x8*>(from + b_row + i * 32 * ROWB + c);
-          if (j & 1) {
-            if (last) issue_half(st, k2, 0, i * (TN / 2) + (j >> 1));
-            if (ks == 0) issue_half(nst, k1, 1, i * (TN / 2) + (j >> 1));
+          // A k-step's first MFMAs need all of its B fragments and its first A fragment: B's are read first.
+          if (quarter == 0) {
+            if (j < 2) bfr[1][2 * q + j] = b_frag(st, 1, 2 * q + j);
+            if (j == 3 || j == 5) issue_half(nst, k1, 1, 2 * q + (j == 5));
+          } else if (quarter == 1) {
+            if (j < 2) af[1][2 * q + j] = a_frag(st, 1, 2 * q + j);
+          } else if (quarter == 3) {
+            if (j < 4 && q < 2) bfr[0][4 * q + j] = b_frag(nst, 0, 4 * q + j);
+            if (j < 4 && q >= 2) af[0][4 * (q - 2) + j] = a_frag(nst, 0, 4 * (q - 2) + j);
+            if (j == 5 || j == 7) issue_half(st, k2, 0, 2 * q + (j == 7));
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -1104,21 +1126,18 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   wait_vmcnt<0>();   // the last iteration's idle fetch must land before LDS is reused
   block_barrier();   // every wave is done reading the stages
 
-  // Output through LDS: a wave lays its 128 x (32 TN) tile out row-major (rows padded by 16 bytes,
+  // Output through LDS: a wave lays its 128 x (16 NT) tile out row-major (rows padded by 16 bytes,
   // which spreads both the 8-byte writes below and the 16-byte reads over all banks) and stores
   // whole 16-byte pieces, so a row of the tile leaves as one contiguous segment.
-  // acc[i][j][e]: row fr of A tile i, column 8*(e/4) + 4*kh + e%4 of B tile j.
+  // acc[i][j][e]: row fr of A tile i, column 4*kq + e of B tile j.
   constexpr int OROWB = BIG_OUT_ROW_BYTES(TN);
   char* ot = smem_big + wave * (128 * OROWB);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<uint2*>(ot + (i * 32 + fr) * OROWB + (j * 32 + 8 * q + 4 * kh) * 2) =
-            make_uint2(pack_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
-                       pack_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
+    for (int j = 0; j < NT; ++j)
+      *reinterpret_cast<uint2*>(ot + (i * 16 + fr) * OROWB + (j * 16 + 4 * kq) * 2) =
+          make_uint2(pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]));
   // The tile is private to the wave, whose LDS operations execute in order: no block barrier,
   // only a fence to keep the compiler from moving the reads above other lanes' writes.
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
