@@ -135,6 +135,16 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t stage_rows(const void* base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
 }
 
+// acc += a b on the 16x16x32 MFMA, the accumulator held in place in accumulation registers.  As a
+// builtin, sixty-four 4-register accumulators live across a loop make the register allocator
+// rotate them through copies (some 200 moves an iteration); a tied operand leaves it no choice.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void mfma_16x16x32_in_place(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+               : "+a"(acc)
+               : "v"(__builtin_bit_cast(i32x4, a)), "v"(__builtin_bit_cast(i32x4, b)));
+}
+
 __device__ __forceinline__ void block_barrier() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();

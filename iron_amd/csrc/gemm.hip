@@ -600,6 +600,242 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
     }
 }
 
+// The 128 x 128 tile on 16x16x32 MFMAs, B as (N,K): the loop of gemm_nt_body with a wave's 64 x 64 as
+// 4 x 4 tiles of 16 x 16 (two 32-wide k-steps a stage; the part sustains more of these MFMAs under
+// its power limit than of the 32x32x16 form), accumulators tied in place, and the output staged
+// through LDS so that it leaves as whole 128-byte row segments (16 bytes a lane) instead of 8-byte
+// pieces of 16 rows an instruction -- the epilogue of the direct form took 3.3 us of a 2048^3
+// product's 20.  Same operands, bounds, fused-projection tail and residual epilogue as gemm_nt_body.
+template <bool QKV>
+__device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
+                                               bf16_t* __restrict__ C_, int M, int N_, int K,
+                                               const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                               int patched, int run_above, int run_upto, const QkvTail& qkv) {
+  constexpr int NT_BM = 128, NT_BN = 128;
+  constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
+  constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
+  constexpr int LOADS = 2 * INST;
+  static_assert(BK == 64 && INST == 4, "two 32-wide k-steps a stage, eight loads a wave");
+  extern __shared__ __align__(16) char smem_nt[];
+  const int Mv = bound_or(valid, M);
+  if (Mv <= run_above || Mv > run_upto) return;
+
+  int tm, tn;
+  const int bid = blockIdx.x;
+  if (patched) {
+    const int xcd = bid & 7, loc = bid >> 3;
+    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
+    const int patches_n = tiles_n >> 2;
+    tm = (patch / patches_n) * 8 + (within & 7);
+    tn = (patch % patches_n) * 4 + (within >> 3);
+  } else {
+    constexpr int BAND = 8;
+    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
+    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
+    tm = first + in_band % height;
+    tn = in_band / height;
+  }
+  const int m0 = tm * NT_BM;
+  if (m0 >= Mv) return;
+  const bf16_t* B = B_;
+  bf16_t* C = C_;
+  int N = N_, which = 0;
+  if constexpr (QKV) {
+    const int q_tiles = N_ / NT_BN, kv_tiles = qkv.kv_n / NT_BN;
+    if (tn >= q_tiles) {
+      which = tn < q_tiles + kv_tiles ? 1 : 2;
+      tn -= q_tiles + (which - 1) * kv_tiles;
+      B = which == 1 ? qkv.Bk : qkv.Bv;
+      C = which == 1 ? qkv.Ck : qkv.Cv;
+      N = qkv.kv_n;
+    }
+  }
+  const int n0 = tn * NT_BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane >> 3, pch = lane & 7;
+  int a_voff[INST], b_voff[INST];
+#pragma unroll
+  for (int i = 0; i < INST; ++i) {
+    const int r = (wave * INST + i) * 8 + lrow;
+    const int lch = pch ^ ((r >> 1) & 7);
+    // Rows past the end re-read the last row; what they produce is never stored.
+    a_voff[i] = (int)(((size_t)(min(m0 + r, M - 1) - m0) * K + lch * 8) * 2);
+    b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
+  }
+  const bf16_t* a_tile = A + (size_t)m0 * K;
+  const bf16_t* b_tile = B + (size_t)n0 * K;
+  auto issue_one = [&](char* st, int kt, int idx) {
+    const int k0 = kt * BK;
+    if (idx < INST) {
+      const __amdgpu_buffer_rsrc_t rows = stage_rows(a_tile + k0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16,
+                                               (int)a_voff[idx], 0, 0, 0);
+    } else {
+      const __amdgpu_buffer_rsrc_t rows = stage_rows(b_tile + k0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024),
+                                               16, (int)b_voff[idx - INST], 0, 0, 0);
+    }
+  };
+
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+
+  // Where this lane stores: rows r0 + lane / 8 of the wave's 64 (r0 = 0, 8, ..), 8 columns from 8 (lane % 8).
+  const int out_row = lane >> 3, out_col = (lane & 7) * 8;
+  const int out_n = n0 + wn * 64 + out_col;
+  // A residual's pieces this lane will add in the epilogue are requested now, so that their
+  // latency passes under the whole product instead of at its end (N a multiple of 8: 16-byte pieces).
+  uint4 res[8];
+  const bool res_ahead = !QKV && qkv.residual != nullptr && (N & 7) == 0;
+  if constexpr (!QKV) {
+    if (res_ahead) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int m = min(m0 + wm * 64 + r * 8 + out_row, M - 1);
+        res[r] = *reinterpret_cast<const uint4*>(qkv.residual + (size_t)m * N + min(out_n, N - 8));
+      }
+    }
+  }
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int s = 0; s < NT_STAGES - 1; ++s)
+#pragma unroll
+    for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_nt + s * NT_STAGE_BYTES, min(s, nk - 1), idx);
+
+  // Fragments: lane -> row fr of a 16-row tile, 16-byte chunk kq of the k-step's four.
+  const int fr = lane & 15, kq = lane >> 4;
+  const int swz = (fr >> 1) & 7;   // tile rows are multiples of 16 apart: one swizzle for all
+  const int a_row = (wm * 64 + fr) * 128, b_row = NT_A_BYTES + (wn * 64 + fr) * 128;
+  auto a_frag = [&](const char* st, int ks, int i) {
+    return *reinterpret_cast<const bf16x8*>(st + a_row + i * 16 * 128 + (((ks * 4 + kq) ^ swz) << 4));
+  };
+  auto b_frag = [&](const char* st, int ks, int j) {
+    return *reinterpret_cast<const bf16x8*>(st + b_row + j * 16 * 128 + (((ks * 4 + kq) ^ swz) << 4));
+  };
+
+  wait_vmcnt<(NT_STAGES - 2) * LOADS>();   // stage 0 has landed once only the two younger ones are out
+  block_barrier();
+  bf16x8 af[2][4], bfr[2][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { bfr[0][i] = b_frag(smem_nt, 0, i); af[0][i] = a_frag(smem_nt, 0, i); }
+  for (int kt = 0; kt < nk; ++kt) {
+    // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
+    // (into buffers nobody reads any more) rather than branch: every iteration issues the same
+    // loads, which keeps the wait counts exact and the scheduling region whole.
+    const int kn = min(kt + NT_STAGES - 1, nk - 1);
+    char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
+    const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
+    const char* st1 = smem_nt + ((kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      if (ks == 1) {
+        // The stage's one barrier, before its second k-step (whose fragments are in registers): of
+        // the loads in flight the oldest LOADS are stage kt+1's (then stage kt+2's, and the 4 issued
+        // so far for stage kt+3); after it nobody reads stage kt any more.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_vmcnt<LOADS + 4>();
+        block_barrier();
+      }
+      const char* from = ks == 0 ? st : st1;
+      const int nks = ks ^ 1;
+      // Source order is issue order (nothing crosses a sched_barrier): after an MFMA one fragment
+      // read of the next k-step (B's first: its first MFMAs need all of them) or one load goes out.
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          mfma_16x16x32_in_place(acc[i][j], bfr[ks][j], af[ks][i]);
+          __builtin_amdgcn_sched_barrier(0);
+          const int slot = i * 4 + j;
+          if (slot < 4) bfr[nks][slot] = b_frag(from, nks, slot);
+          else if (slot < 8) af[nks][slot - 4] = a_frag(from, nks, slot - 4);
+          else if (slot & 1) issue_one(nst, kn, ks * 4 + (slot - 9) / 2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+  }
+
+  wait_vmcnt<0>();   // the idle fetches of the last iterations land ...
+  block_barrier();   // ... in every wave, and every wave is done with the stages, before LDS is reused
+
+  if constexpr (QKV) {
+    if (which < 2) {
+      // acc[i][j][e] and acc[i][j + 2][e] are columns c and c + 32 of the wave's head, c = 16 j + 4 kq + e,
+      // of row m = 16 i + fr: the pair RoPE turns by the angle row's (cos, sin) number c.
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = min(m0 + wm * 64 + i * 16 + fr, M - 1);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          float cs[8];
+          unpack8(*reinterpret_cast<const uint4*>(qkv.angles + (size_t)m * 64 + 2 * (16 * j + 4 * kq)), cs);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float x1 = round_bf16(acc[i][j][e]), x2 = round_bf16(acc[i][j + 2][e]);
+            const float c = cs[2 * e], sn = cs[2 * e + 1];
+            acc[i][j][e] = x1 * c - x2 * sn;
+            acc[i][j + 2][e] = x2 * c + x1 * sn;
+          }
+        }
+      }
+    }
+  }
+
+  // Output through LDS: the wave lays its 64 x 64 out row-major (rows padded by 16 bytes, which
+  // spreads the 8-byte writes and the 16-byte reads over the banks) and each lane then owns 8
+  // consecutive columns of a row: a row of the tile leaves as one 128-byte segment.
+  constexpr int OROWB = 64 * 2 + 16;
+  char* ot = smem_nt + wave * (64 * OROWB);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<uint2*>(ot + (i * 16 + fr) * OROWB + (j * 16 + 4 * kq) * 2) =
+          make_uint2(pack_bf16(acc[i][j][0], acc[i][j][1]), pack_bf16(acc[i][j][2], acc[i][j][3]));
+  // The tile is private to the wave, whose LDS operations execute in order: no block barrier,
+  // only a fence to keep the compiler from moving the reads above other lanes' writes.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const bool whole = (N & 7) == 0 && out_n + 8 <= N;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int row = r * 8 + out_row, m = m0 + wm * 64 + row;
+    uint4 v = *reinterpret_cast<const uint4*>(ot + row * OROWB + out_col * 2);
+    if (m >= Mv || out_n >= N) continue;
+    bf16_t* p = C + (size_t)m * N + out_n;
+    if constexpr (!QKV) {
+      if (qkv.residual != nullptr) {   // the product rounded as it would be stored, then scale * it + residual
+        float x[8], rf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        unpack8(v, x);
+        if (whole) {
+          unpack8(res_ahead ? res[r] : *reinterpret_cast<const uint4*>(qkv.residual + (size_t)m * N + out_n), rf);
+        } else {
+          for (int e = 0; e < 8 && out_n + e < N; ++e) rf[e] = bf16_to_f32(qkv.residual[(size_t)m * N + out_n + e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = fmaf(qkv.residual_scale, x[e], rf[e]);
+        v = pack8(x);
+      }
+    }
+    if (whole) {
+      *reinterpret_cast<uint4*>(p) = v;
+    } else {
+      const bf16_t* h = reinterpret_cast<const bf16_t*>(&v);
+      for (int e = 0; e < 8 && out_n + e < N; ++e) p[e] = h[e];
+    }
+  }
+}
+
+
 template <bool B_KN, bool QKV, int T>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
                                                       const bf16_t* __restrict__ B,
@@ -608,7 +844,10 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       int tiles_n, int patched, int run_above,
                                                       int run_upto, QkvTail qkv) {
   if constexpr (QKV) to_cache_rows(qkv, valid, M);
-  gemm_nt_body<B_KN, QKV, T>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+  if constexpr (T == 2 && !B_KN)
+    gemm_nt16_body<QKV>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+  else
+    gemm_nt_body<B_KN, QKV, T>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
 }
 
 template <bool B_KN, bool QKV = false, int T = 2>
@@ -851,7 +1090,7 @@ __global__ __launch_bounds__(256) void qkv_either_kernel(const bf16_t* __restric
       qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, -1, INT_MAX, qkv);
   } else {
     if ((int)blockIdx.x < narrow.tiles_m * narrow.tiles_n)
-      gemm_nt_body<false, true, 2>(A, Bq, Cq, M, heads * 64, K, valid, narrow.tiles_m, narrow.tiles_n, narrow.patched,
+      gemm_nt16_body<true>(A, Bq, Cq, M, heads * 64, K, valid, narrow.tiles_m, narrow.tiles_n, narrow.patched,
                                    -1, INT_MAX, qkv);
   }
 }
@@ -963,16 +1202,6 @@ constexpr int BIG_WAVES = IRON_BIG_WAVES;
 constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stages of half-line rows) measured 13 % slower
 #define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
 constexpr int BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
-
-// acc += a b on the 16x16x32 MFMA, the accumulator held in place in accumulation registers.  As a
-// builtin, sixty-four 4-register accumulators live across a loop make the register allocator
-// rotate them through copies (some 200 moves an iteration); a tied operand leaves it no choice.
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void mfma_16x16x32_in_place(f32x4& acc, const bf16x8& a, const bf16x8& b) {
-  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
-               : "+a"(acc)
-               : "v"(__builtin_bit_cast(i32x4, a)), "v"(__builtin_bit_cast(i32x4, b)));
-}
 
 template <int WAVES, int KB>
 __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
@@ -1184,7 +1413,7 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
       gemm_nt256_body<BIG_WAVES, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched, -1, INT_MAX);
   } else if (Mv > few128) {
     if (bid < t128.tiles_m * t128.tiles_n)
-      gemm_nt_body<false, false, 2>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX,
+      gemm_nt16_body<false>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX,
                                     QkvTail{});
   } else {
     if (bid < t64.tiles_m * t64.tiles_n)
