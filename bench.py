@@ -54,6 +54,17 @@ def graph_time_us(torch, launches, replays):
     return start.elapsed_time(stop) * 1e3 / (replays * len(launches))
 
 
+def verified(torch, what, got, want, rtol=1e-2, atol=1e-2):
+    """The timed kernel's own output against a float32 evaluation of the same product on the same
+    operands (torch on the GPU, over the rows sampled): the bar of the parity tests, |diff| <= atol +
+    rtol |want|.  Raises if it fails, so a number in the line is a number of a checked result."""
+    got, want = got.float(), want.float()
+    excess = ((got - want).abs() - (atol + rtol * want.abs())).max().item()
+    if not excess <= 0.0:
+        raise AssertionError(f"bench self-check failed: {what}: |diff| exceeds {atol} + {rtol}|want| by {excess:.4g}")
+    return int(got.numel())
+
+
 def bench_gemv(torch, K, dev, Kdim, N, steps, rng):
     """One decode GEMV shape over a pool of distinct weights larger than the last-level cache."""
     from iron_amd.bf16 import round_bf16, to_torch
@@ -67,9 +78,12 @@ def bench_gemv(torch, K, dev, Kdim, N, steps, rng):
     launches = [(lambda W=W: K.gemv(W, x, y, M=N, K=Kdim)) for W in pool]
     reps = max(1, steps // len(launches))
     us = graph_time_us(torch, launches, reps)
+    rows = torch.from_numpy(rng.choice(N, size=min(N, 4096), replace=False)).to(dev)
+    checked = verified(torch, f"gemv {Kdim}->{N}", y[rows], pool[-1][rows].float() @ x.float())
     algo = 2 * (N * Kdim + Kdim + N)
     return {"K": Kdim, "N": N, "us": round(us, 3), "GBps": round(algo / us / 1e3, 1),
-            "frac_hbm": round(algo / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": algo, "copies": copies}
+            "frac_hbm": round(algo / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": algo, "copies": copies,
+            "checked_outputs": checked}
 
 
 def bench_gemm(torch, K, dev, steps, rng, b_col_maj, M=2048, N=2048, Kd=2048):
@@ -81,9 +95,13 @@ def bench_gemm(torch, K, dev, steps, rng, b_col_maj, M=2048, N=2048, Kd=2048):
     C = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
     launches = [lambda: K.gemm(A, B, C, M=M, N=N, K=Kd, b_col_maj=b_col_maj)] * 20
     us = graph_time_us(torch, launches, max(1, steps // 20))
+    rows = torch.from_numpy(np.sort(rng.choice(M, size=64, replace=False))).to(dev)
+    Bf = B.float()
+    checked = verified(torch, f"gemm {M}x{N}x{Kd}", C[rows], A[rows].float() @ (Bf.t() if b_col_maj else Bf))
     flops = 2.0 * M * N * Kd
     return {"M": M, "N": N, "K": Kd, "b_col_maj": b_col_maj, "us": round(us, 3),
-            "TFLOPs": round(flops / us / 1e6, 1), "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)}
+            "TFLOPs": round(flops / us / 1e6, 1), "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "checked_outputs": checked}
 
 
 def bench_library_reference(torch, dev, n, rng):
@@ -196,15 +214,25 @@ def bench_attention(torch, K, dev, n, rng):
     def rand(*shape):
         return torch.randn(shape, device=dev, dtype=torch.float32).to(torch.bfloat16)
 
+    def attend(q, keys, values):
+        """One query row of every head over `keys` / `values` (rows, G, D) in float32: (H, D)."""
+        qf = q.float().reshape(G, H // G, D)
+        scores = torch.einsum("ghd,lgd->ghl", qf, keys.float()) * 0.125
+        return torch.einsum("ghl,lgd->ghd", torch.softmax(scores, dim=-1), values.float()).reshape(H, D)
+
     for S in (512, 2048, 8192):
         Q, Kc, Vc = rand(S, H, D), rand(S, G, D), rand(S, G, D)
         O = torch.empty_like(Q)
         launches = [lambda: K.mha_prefill(Q, Kc, Vc, O, heads=H, kv_heads=G, d=D, seq=S, kv_len=S, scale=0.125,
                                           q_interleaved=True, kv_interleaved=True)] * 10
         us = graph_time_us(torch, launches, max(1, n // (10 * max(1, S // 512))))
+        checked = 0
+        for i in sorted({0, 63, 64, S // 2 - 1, S - 129, S - 1}):   # query rows, every head: keys 0..i
+            checked += verified(torch, f"prefill attention S={S} row {i}", O[i], attend(Q[i], Kc[: i + 1], Vc[: i + 1]))
         flops = 4.0 * H * D * S * (S + 1) / 2
         out["prefill"].append({"S": S, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
-                               "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)})
+                               "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                               "checked_outputs": checked})
     for L in (1024, 4096, 16384):
         copies = max(2, min(64, int(np.ceil(400e6 / (L * G * D * 4)))))
         Q = rand(1, H, D)
@@ -214,9 +242,11 @@ def bench_attention(torch, K, dev, n, rng):
         launches = [(lambda a=a, b=b: K.mha_decode(Q, a, b, O, heads=H, kv_heads=G, d=D, kv_len=L, scale=0.125,
                                                    kv_interleaved=True, workspace=ws)) for a, b in zip(Ks, Vs)]
         us = graph_time_us(torch, launches, max(1, n // len(launches)))
+        checked = verified(torch, f"decode attention L={L}", O[0], attend(Q[0], Ks[-1], Vs[-1]))
         algo = 2 * L * G * D * 2 + 2 * H * D * 2
         out["decode"].append({"L": L, "us": round(us, 2), "GBps": round(algo / us / 1e3, 1),
-                              "frac_hbm": round(algo / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": algo})
+                              "frac_hbm": round(algo / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": algo,
+                              "checked_outputs": checked})
     return out
 
 
@@ -235,6 +265,12 @@ def bench_sample(torch, K, dev, n, rng):
         row = torch.from_numpy(np.ascontiguousarray(draw_row(t, k, 1234567890123))).to(dev)
         launches = [lambda row=row: K.sample(logits, row, token, workspace=ws)] * 20
         out[name] = round(graph_time_us(torch, launches, max(1, n // 20)), 2)
+        drawn = int(token.item())
+        if k == 1 and drawn != int(torch.argmax(logits.float()).item()):
+            raise AssertionError(f"bench self-check failed: the greedy draw {drawn} is not the largest logit's index")
+        if not 0 <= drawn < vocab or logits[drawn].float() < torch.topk(logits.float(), k).values[-1]:
+            raise AssertionError(f"bench self-check failed: the draw {drawn} is not among the top {k}")
+    out["checked"] = "greedy = argmax; the sampled token among the top k"
     return out
 
 
@@ -266,12 +302,16 @@ def bench_pre_attention(torch, K, dev, n):
         K.prefill_qkv(n_, Wq, Wk, Wv, ang, qr, kr, v, rows=S, hidden=E, heads=H, kv_heads=G, d=D)
 
     us = graph_time_us(torch, [block] * 4, max(1, n // 8))
+    stepwise = [t.clone() for t in (qr, kr, v)]
     us_fused = graph_time_us(torch, [fused] * 4, max(1, n // 8))
+    checked = sum(verified(torch, f"fused projections, output {i}", got, want)
+                  for i, (got, want) in enumerate(zip((qr, kr, v), stepwise)))
     flops = 2.0 * S * E * (H + 2 * G) * D
     return {"us": round(us_fused, 2), "TFLOPs": round(flops / us_fused / 1e6, 1), "kernels": 2,
             "note": "RMSNorm, then one launch for the three projections with RoPE in its epilogue "
                     "(what the compiled prompt chunk runs)",
             "unfused": {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1), "kernels": 6},
+            "checked_outputs": checked,
             "bytes_unfused": 71_600_000, "bytes_fused_min": 33_600_000}
 
 
