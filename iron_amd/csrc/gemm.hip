@@ -1185,15 +1185,18 @@ static int launch_gemm(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N
 }
 
 
-// Large problems, B (N,K): 256x256x64 tiles, two 64 KB stages fed straight into LDS, 4 waves each
-// owning 128x128 of the tile (16 MFMA tiles, 256 accumulator registers).  Against the 128x128
-// kernel a wave reads half as many LDS bytes and a CU pulls half as many global bytes per flop --
-// the 64 B/clk a CU can move from L2 into LDS is what bounds the smaller tile.  A wave is alone on
-// its SIMD, so its own instruction stream interleaves the next k-step's fragment reads and a
-// quarter of the next stage's loads with the 16 MFMAs of a k-step.
+// Large problems, B (N,K): 256x256x64 tiles, two 64 KB stages fed straight into LDS.  Against the
+// 128x128 kernel a CU pulls half as many global bytes per flop -- the 64 B/clk a CU can move from L2
+// into LDS is what bounds the smaller tile.  Eight waves, two a SIMD, each owning 128 x 64 of the
+// tile (32 accumulator tiles of 16 x 16, 128 accumulation registers): one's loads and fragment reads
+// issue under the other's MFMAs (2048 x 8192 x 2048 60.5 -> 56.5 us, 4096^3 111 -> 107.5 against four
+// waves of 128 x 128; 8192^3 the same).  Within a wave the instruction stream still interleaves the
+// next k-step's fragment reads and the next stages' loads with the MFMAs.  Where the blocks of one
+// launch choose their tile size by a row bound (gemm_either_kernel) the large tile is four waves of
+// 128 x 128, as every other tiling of that launch is four waves.
 constexpr int BIG_BM = 256, BIG_BN = 256;
 #ifndef IRON_BIG_WAVES
-#define IRON_BIG_WAVES 4
+#define IRON_BIG_WAVES 8   // the stand-alone launch: two waves a SIMD, each 128 x 64 of the tile (4: one, 128 x 128)
 #endif
 constexpr int BIG_WAVES = IRON_BIG_WAVES;
 #ifndef IRON_BIG_KB
@@ -1279,7 +1282,7 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
   const int nk = K / KB;
-  static_assert(KB == 64 && INST == 8 && TN == 4, "the loop below is written for two 64-wide stages and four waves");
+  static_assert(KB == 64 && (WAVES == 4 || WAVES == 8), "the loop below is written for two 64-wide stages and four or eight waves");
   // A stage's 2 INST loads go out in two halves of INST: the first under the last quarter of the
   // stage two before it (right after that stage's barrier freed the buffer), the second under the
   // first quarter of the stage before it; two quarters later, at that stage's barrier, all have landed.
@@ -1313,14 +1316,19 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
     const int k1 = min(kt + 1, nk - 1), k2 = min(kt + 2, nk - 1);
     char* st = smem_big + (kt % STAGES) * STAGE_BYTES;          // this stage; then stage kt+2's buffer
     char* nst = smem_big + ((kt + 1) % STAGES) * STAGE_BYTES;   // stage kt+1's
-    // A stage is two k-steps of 64 MFMAs, scheduled as four quarters of 32 (tile rows 0..3 and 4..7
-    // of a k-step).  Source order is issue order (nothing crosses a sched_barrier): after an MFMA
-    // one fragment read or one load goes out.
+    // A stage is two k-steps of 8 NT MFMAs, scheduled as four quarters (tile rows 0..3 and 4..7 of
+    // a k-step).  Source order is issue order (nothing crosses a sched_barrier): after an MFMA one
+    // fragment read or one load goes out.  A k-step's first MFMAs need all of its B fragments and
+    // its first A fragment, so B's are read first.
     //   quarter 0: the second k-step's B fragments, and the second half of stage kt+1's loads
     //   quarter 1: the second k-step's A fragments
     //   quarter 2: nothing -- then the stage's one barrier: every wave's loads of stage kt+1 have
     //              landed and nobody reads stage kt any more (the last quarter's fragments are in registers)
     //   quarter 3: stage kt+1's first fragments, and the first half of stage kt+2's loads
+    constexpr int SLOTS = 4 * NT;                              // MFMAs of a quarter
+    constexpr int Q0_EVERY = (SLOTS - NT) / INST;              // quarter 0: a load every so many slots once B is read
+    constexpr int Q3_FIRST = NT + 8, Q3_EVERY = (SLOTS - Q3_FIRST) / INST;
+    static_assert(Q0_EVERY >= 1 && Q3_EVERY >= 1, "a quarter has a slot for each of its reads and loads");
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
@@ -1335,16 +1343,17 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
         for (int j = 0; j < NT; ++j) {
           mfma_16x16x32_in_place(acc[i][j], bfr[ks][j], af[ks][i]);
           __builtin_amdgcn_sched_barrier(0);
-          // A k-step's first MFMAs need all of its B fragments and its first A fragment: B's are read first.
+          const int slot = q * NT + j;
           if (quarter == 0) {
-            if (j < 2) bfr[1][2 * q + j] = b_frag(st, 1, 2 * q + j);
-            if (j == 3 || j == 5) issue_half(nst, k1, 1, 2 * q + (j == 5));
+            if (slot < NT) bfr[1][slot] = b_frag(st, 1, slot);
+            else if ((slot - NT) % Q0_EVERY == 0 && (slot - NT) / Q0_EVERY < INST) issue_half(nst, k1, 1, (slot - NT) / Q0_EVERY);
           } else if (quarter == 1) {
-            if (j < 2) af[1][2 * q + j] = a_frag(st, 1, 2 * q + j);
+            if (slot < 8) af[1][slot] = a_frag(st, 1, slot);
           } else if (quarter == 3) {
-            if (j < 4 && q < 2) bfr[0][4 * q + j] = b_frag(nst, 0, 4 * q + j);
-            if (j < 4 && q >= 2) af[0][4 * (q - 2) + j] = a_frag(nst, 0, 4 * (q - 2) + j);
-            if (j == 5 || j == 7) issue_half(st, k2, 0, 2 * q + (j == 7));
+            if (slot < NT) bfr[0][slot] = b_frag(nst, 0, slot);
+            else if (slot < Q3_FIRST) af[0][slot - NT] = a_frag(nst, 0, slot - NT);
+            else if ((slot - Q3_FIRST) % Q3_EVERY == 0 && (slot - Q3_FIRST) / Q3_EVERY < INST)
+              issue_half(st, k2, 0, (slot - Q3_FIRST) / Q3_EVERY);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -1406,11 +1415,11 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
                                                           int M, int N, int K, const int* __restrict__ valid,
                                                           Tiling t256, Tiling t128, Tiling t64, int few256,
                                                           int few128) {
-  static_assert(BIG_WAVES == 4, "the blocks of this launch are four waves");
+  // The blocks of this launch are four waves whatever the stand-alone large-tile launch uses.
   const int Mv = bound_or(valid, M), bid = blockIdx.x;
   if (BIG && Mv > few256) {
     if (bid < t256.tiles_m * t256.tiles_n)
-      gemm_nt256_body<BIG_WAVES, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched, -1, INT_MAX);
+      gemm_nt256_body<4, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched, -1, INT_MAX);
   } else if (Mv > few128) {
     if (bid < t128.tiles_m * t128.tiles_n)
       gemm_nt16_body<false>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX,
@@ -1431,7 +1440,7 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   const Tiling t256{BIG ? M / BIG_BM : 0, BIG ? N / BIG_BN : 0, BIG ? patched_order(M / BIG_BM, N / BIG_BN) : 0};
   const Tiling t128{(rows128 + 127) / 128, n128, patched_order((rows128 + 127) / 128, n128)};
   const Tiling t64{(rows64 + 63) / 64, n64, patched_order((rows64 + 63) / 64, n64)};
-  constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
+  constexpr size_t out_bytes = (size_t)4 * 128 * BIG_OUT_ROW_BYTES(4);   // this launch's large tiles are four waves'
   constexpr size_t lds256 = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
   constexpr size_t lds128 = (size_t)NT_STAGES * 256 * BK * 2;
   constexpr size_t lds = BIG ? (lds256 > lds128 ? lds256 : lds128) : lds128;
