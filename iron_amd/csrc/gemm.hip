@@ -1206,7 +1206,7 @@ constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stage
 #define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
 constexpr int BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
 
-template <int WAVES, int KB>
+template <int WAVES, int KB, bool B_KN = false>
 __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                 bf16_t* __restrict__ C, int M, int N, int K,
                                                 const int* __restrict__ valid, int tiles_m, int tiles_n,
@@ -1257,16 +1257,30 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   // rows and the stage's k are the scalar offset, so a load costs two scalar adds and no vector ALU
   // work between two MFMAs.
   const __amdgpu_buffer_rsrc_t a_rows = stage_rows(A + (size_t)(m0 + wave * INST * RPI) * K);
-  const __amdgpu_buffer_rsrc_t b_rows = stage_rows(B + (size_t)(n0 + wave * INST * RPI) * K);
+  // B as (K,N) lands as stored: the stage's 64 k-rows of 256 columns (512 bytes a row, two rows an
+  // instruction), a row's 32 chunks XORed with kn_swizzle(row) so that the transposing reads below
+  // find the four rows of a 16-lane group, and the groups of a pass, in different banks.
+  const __amdgpu_buffer_rsrc_t b_rows =
+      stage_rows(B_KN ? B + n0 + (size_t)(wave * INST * 2) * N : B + (size_t)(n0 + wave * INST * RPI) * K);
+  auto kn_swizzle = [](int k) { return ((k & 3) << 1) | (((k >> 3) & 3) << 3); };
+  int kn_off[INST];   // (K,N): this lane's 16 bytes within instruction idx's two rows
+#pragma unroll
+  for (int idx = 0; idx < INST; ++idx) {
+    const int kr = (wave * INST + idx) * 2 + (lane >> 5);   // the lane's k-row of the stage
+    kn_off[idx] = (int)(((size_t)(lane >> 5) * N + ((lane & 31) ^ kn_swizzle(kr)) * 8) * 2);
+  }
   const int inst_stride = RPI * K * 2;
   auto issue_one = [&](char* st, int kt, int idx) {
     const int k_off = kt * KB * 2;
     if (idx < INST)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rows, IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16,
                                                (int)ld_off[idx & 1], idx * inst_stride + k_off, 0, 0);
-    else
+    else if constexpr (!B_KN)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rows, IRON_LDS_PTR(st + A_BYTES + (wave * INST + idx - INST) * 1024),
                                                16, (int)ld_off[idx & 1], (idx - INST) * inst_stride + k_off, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rows, IRON_LDS_PTR(st + A_BYTES + (wave * INST + idx - INST) * 1024),
+                                               16, (int)kn_off[idx - INST], ((idx - INST) * 2 + kt * KB) * N * 2, 0, 0);
   };
 
   // The product runs on 16x16x32 MFMAs (a k-step is 32 wide, two a stage): on random operands the
@@ -1302,6 +1316,32 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   auto b_frag = [&](const char* st, int ks, int j) {
     return *reinterpret_cast<const bf16x8*>(st + b_row + j * 16 * ROWB + (((ks * 4 + kq) ^ swz) << 4));
   };
+  // (K,N): the B operand of tile j wants, for column n = 16 j + fr, the k-step's k = 8 kq .. + 7.  A
+  // transposing read hands a 16-lane group the 4 x 16 block its lanes point at (4 k-rows, each
+  // lane 4 columns) turned round: the lane gets 4 k of one column.  Rows 8 kq .. + 3 and 8 kq + 4 .. + 7.
+  const int tr_k = 8 * kq + ((lane & 15) >> 2), tr_n = wn * NT * 16 + 4 * (lane & 3);
+  const unsigned kn_base = (unsigned)(size_t)IRON_LDS_PTR(smem_big) + A_BYTES;
+  auto b_frag_kn = [&](int stage_bytes, int ks, int j, TrFrag& t) {
+    const int k = ks * 32 + tr_k, n = tr_n + j * 16;   // kn_swizzle(k + 4) = kn_swizzle(k): k % 8 < 4
+    const unsigned at = kn_base + stage_bytes + (((n >> 3) ^ kn_swizzle(k)) << 4) + ((n & 4) << 1);
+    t.lo = lds_read_tr16(at + k * 512);
+    t.hi = lds_read_tr16(at + (k + 4) * 512);
+  };
+  TrFrag tfb[2][NT];
+  // The compiler does not count the transposing reads: a k-step's B fragments pass through this
+  // wait (every LDS read issued so far) before they are joined into operands.
+  auto join_b = [&](int ks, bf16x8 (&b)[NT]) {
+    if constexpr (NT == 4)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tfb[ks][0].lo), "+v"(tfb[ks][0].hi), "+v"(tfb[ks][1].lo), "+v"(tfb[ks][1].hi),
+                                             "+v"(tfb[ks][2].lo), "+v"(tfb[ks][2].hi), "+v"(tfb[ks][3].lo), "+v"(tfb[ks][3].hi));
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tfb[ks][0].lo), "+v"(tfb[ks][0].hi), "+v"(tfb[ks][1].lo), "+v"(tfb[ks][1].hi),
+                                             "+v"(tfb[ks][2].lo), "+v"(tfb[ks][2].hi), "+v"(tfb[ks][3].lo), "+v"(tfb[ks][3].hi),
+                                             "+v"(tfb[ks][4].lo), "+v"(tfb[ks][4].hi), "+v"(tfb[ks][5].lo), "+v"(tfb[ks][5].hi),
+                                             "+v"(tfb[ks][6].lo), "+v"(tfb[ks][6].hi), "+v"(tfb[ks][7].lo), "+v"(tfb[ks][7].hi));
+#pragma unroll
+    for (int j = 0; j < NT; ++j) b[j] = tr_join(tfb[ks][j]);
+  };
 
   wait_vmcnt<INST>();   // stage 0 has landed once only stage 1's first half is out
   block_barrier();
@@ -1309,7 +1349,10 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
 #pragma unroll
   for (int i = 0; i < 8; ++i) af[0][i] = a_frag(smem_big, 0, i);
 #pragma unroll
-  for (int j = 0; j < NT; ++j) bfr[0][j] = b_frag(smem_big, 0, j);
+  for (int j = 0; j < NT; ++j) {
+    if constexpr (B_KN) b_frag_kn(0, 0, j, tfb[0][j]);
+    else bfr[0][j] = b_frag(smem_big, 0, j);
+  }
   for (int kt = 0; kt < nk; ++kt) {
     // Past the end the last stage is fetched again (into buffers nobody reads any more) rather than
     // branch: a branch would end the scheduling region and undo the interleaving below.
@@ -1329,8 +1372,10 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
     constexpr int Q0_EVERY = (SLOTS - NT) / INST;              // quarter 0: a load every so many slots once B is read
     constexpr int Q3_FIRST = NT + 8, Q3_EVERY = (SLOTS - Q3_FIRST) / INST;
     static_assert(Q0_EVERY >= 1 && Q3_EVERY >= 1, "a quarter has a slot for each of its reads and loads");
+    const int st_bytes = (kt % STAGES) * STAGE_BYTES, nst_bytes = ((kt + 1) % STAGES) * STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
+      if constexpr (B_KN) join_b(ks, bfr[ks]);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int quarter = ks * 2 + (i >> 2), q = i & 3;   // q: the quarter's tile row
@@ -1345,13 +1390,17 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
           __builtin_amdgcn_sched_barrier(0);
           const int slot = q * NT + j;
           if (quarter == 0) {
-            if (slot < NT) bfr[1][slot] = b_frag(st, 1, slot);
-            else if ((slot - NT) % Q0_EVERY == 0 && (slot - NT) / Q0_EVERY < INST) issue_half(nst, k1, 1, (slot - NT) / Q0_EVERY);
+            if (slot < NT) {
+              if constexpr (B_KN) b_frag_kn(st_bytes, 1, slot, tfb[1][slot]);
+              else bfr[1][slot] = b_frag(st, 1, slot);
+            } else if ((slot - NT) % Q0_EVERY == 0 && (slot - NT) / Q0_EVERY < INST) issue_half(nst, k1, 1, (slot - NT) / Q0_EVERY);
           } else if (quarter == 1) {
             if (slot < 8) af[1][slot] = a_frag(st, 1, slot);
           } else if (quarter == 3) {
-            if (slot < NT) bfr[0][slot] = b_frag(nst, 0, slot);
-            else if (slot < Q3_FIRST) af[0][slot - NT] = a_frag(nst, 0, slot - NT);
+            if (slot < NT) {
+              if constexpr (B_KN) b_frag_kn(nst_bytes, 0, slot, tfb[0][slot]);
+              else bfr[0][slot] = b_frag(nst, 0, slot);
+            } else if (slot < Q3_FIRST) af[0][slot - NT] = a_frag(nst, 0, slot - NT);
             else if ((slot - Q3_FIRST) % Q3_EVERY == 0 && (slot - Q3_FIRST) / Q3_EVERY < INST)
               issue_half(st, k2, 0, (slot - Q3_FIRST) / Q3_EVERY);
           }
@@ -1393,14 +1442,14 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   }
 }
 
-template <int WAVES, int KB>
+template <int WAVES, int KB, bool B_KN = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
                                                          const bf16_t* __restrict__ B,
                                                          bf16_t* __restrict__ C, int M, int N, int K,
                                                          const int* __restrict__ valid, int tiles_m,
                                                          int tiles_n, int patched, int run_above,
                                                          int run_upto) {
-  gemm_nt256_body<WAVES, KB>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto);
+  gemm_nt256_body<WAVES, KB, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto);
 }
 
 // A row bound read on the device decides which tile size fills the chip best (512 valid rows of
@@ -1459,6 +1508,7 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   IRON_LAUNCH_CHECK();
 }
 
+template <bool B_KN = false>
 static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                              const int* valid, hipStream_t s, int run_above = -1, int run_upto = INT_MAX) {
   const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
@@ -1466,13 +1516,13 @@ static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M,
   const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
+  hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
                      tiles_m, tiles_n, patched, run_above, run_upto);
   IRON_LAUNCH_CHECK();
 }
@@ -1522,7 +1572,11 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
       if (rc != 0) return rc;
       return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, QkvTail{}, -1, few);
     }
-    // (K,N) B is read in whole 128-column tiles straight into LDS: N must be whole tiles.
+    // (K,N) B is read in whole tiles straight into LDS: N must be whole tiles.  Enough whole
+    // 256x256 tiles to fill the chip, and a matrix a 32-bit byte offset spans: the large-tile kernel.
+    if (valid == nullptr && M % BIG_BM == 0 && N % BIG_BN == 0 && (long)(M / BIG_BM) * (N / BIG_BN) >= 192 &&
+        (long)K * N * 2 < (1L << 31))
+      return launch_gemm_nt256<true>(A, B, C, M, N, K, valid, s);
     if (N % 128 == 0) return launch_gemm_nt<true>(A, B, C, M, N, K, valid, s);
   }
   // 128x128 tiles fill the 256 CUs once at 2048x2048; narrower problems take 64-wide tiles.

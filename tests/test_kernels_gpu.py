@@ -100,19 +100,33 @@ def test_gemm_layouts(cuda, b_col_maj, c_col_maj):
     assert np.all(np.abs(from_torch(C) - want) <= bound)
 
 
+@pytest.mark.parametrize("b_col_maj", [True, False])
 @pytest.mark.parametrize("n", [4096, 8192])
-def test_gemm_large_squares_on_sampled_rows(cuda, n):
-    """The 256 x 256-tile kernel at the benchmark's large squares: a sample of rows (tile edges and
-    random ones) of the product against float64 dot products, and nothing left unwritten."""
+def test_gemm_large_squares_on_sampled_rows(cuda, n, b_col_maj):
+    """The 256 x 256-tile kernel at the benchmark's large squares, B as (N, K) and as (K, N): a sample
+    of rows (tile edges and random ones) of the product against float64 dot products, and nothing
+    left unwritten."""
     rng = np.random.default_rng(n)
-    A, B = bf(rng, n, n, scale=0.02), bf(rng, n, n, scale=0.02)   # B is (N, K)
+    A, B = bf(rng, n, n, scale=0.02), bf(rng, n, n, scale=0.02)   # B is (N, K) or (K, N) as the flag says
     C = out_like((n, n), cuda, fill=float("nan"))
-    K.gemm(dev(A, cuda), dev(B, cuda), C, M=n, N=n, K=n, b_col_maj=True)
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=n, N=n, K=n, b_col_maj=b_col_maj)
     got = from_torch(C)
     assert not np.isnan(got).any()
     rows = sorted({0, 1, 127, 128, 255, 256, 257, n // 2 - 1, n // 2, n - 256, n - 1, *rng.integers(0, n, 21).tolist()})
-    want = round_bf16((A[rows].astype(np.float64) @ B.astype(np.float64).T).astype(np.float32))
+    Bd = B.astype(np.float64)
+    want = round_bf16((A[rows].astype(np.float64) @ (Bd.T if b_col_maj else Bd)).astype(np.float32))
     close(got[rows], want, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("M,Kdim,N", [(2048, 192, 6144), (4096, 64, 3072), (3072, 1152, 4096)])
+def test_gemm_large_tiles_with_b_as_stored_by_default(cuda, M, Kdim, N):
+    """B (K, N) through the 256 x 256 tiles (192 whole tiles or more): one stage, three, and
+    eighteen of them, every element against the oracle."""
+    rng = np.random.default_rng(M + N + Kdim)
+    A, B = bf(rng, M, Kdim), bf(rng, Kdim, N)
+    C = out_like((M, N), cuda, fill=float("nan"))
+    K.gemm(dev(A, cuda), dev(B, cuda), C, M=M, N=N, K=Kdim)
+    close(C, ops.gemm(A, B))
 
 
 def test_gemm_headline_shape(cuda):
