@@ -644,6 +644,7 @@ def main():
     # The prefill projections of the decoder (2048 tokens; weights (N,K)) and two larger squares.
     gemm += [bench_gemm(torch, K, dev, max(20, n // 4), rng, True, M=m, N=nn, Kd=k)
              for m, nn, k in ((2048, 8192, 2048), (2048, 2048, 8192), (4096, 4096, 4096), (8192, 8192, 8192))]
+    gemm.append(bench_gemm(torch, K, dev, max(20, n // 4), rng, False, M=4096, N=4096, Kd=4096))   # B (K,N) on the large tiles
     attention = bench_attention(torch, K, dev, n, rng)
     pre_attention = bench_pre_attention(torch, K, dev, n)
     sample = bench_sample(torch, K, dev, n, rng)
