@@ -606,7 +606,7 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
 // through LDS so that it leaves as whole 128-byte row segments (16 bytes a lane) instead of 8-byte
 // pieces of 16 rows an instruction -- the epilogue of the direct form took 3.3 us of a 2048^3
 // product's 20.  Same operands, bounds, fused-projection tail and residual epilogue as gemm_nt_body.
-template <bool QKV>
+template <bool QKV, bool B_KN = false>
 __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
                                                bf16_t* __restrict__ C_, int M, int N_, int K,
                                                const int* __restrict__ valid, int tiles_m, int tiles_n,
@@ -616,6 +616,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int LOADS = 2 * INST;
   static_assert(BK == 64 && INST == 4, "two 32-wide k-steps a stage, eight loads a wave");
+  static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
   extern __shared__ __align__(16) char smem_nt[];
   const int Mv = bound_or(valid, M);
   if (Mv <= run_above || Mv > run_upto) return;
@@ -655,6 +656,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane >> 3, pch = lane & 7;
+  auto kn_swizzle = [](int k) { return ((k & 3) << 1) | (((k >> 3) & 1) << 3); };
   int a_voff[INST], b_voff[INST];
 #pragma unroll
   for (int i = 0; i < INST; ++i) {
@@ -662,10 +664,17 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
     const int lch = pch ^ ((r >> 1) & 7);
     // Rows past the end re-read the last row; what they produce is never stored.
     a_voff[i] = (int)(((size_t)(min(m0 + r, M - 1) - m0) * K + lch * 8) * 2);
-    b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
+    if constexpr (!B_KN) {
+      b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
+    } else {
+      // B (K,N) lands as stored: 64 k-rows of 128 columns (256 bytes a row, four rows an
+      // instruction), a row's 16 chunks XORed with kn_swizzle(row) for the transposing reads below.
+      const int kr = (wave * INST + i) * 4 + (lane >> 4);
+      b_voff[i] = (int)(((size_t)kr * N + ((lane & 15) ^ kn_swizzle(kr)) * 8) * 2);
+    }
   }
   const bf16_t* a_tile = A + (size_t)m0 * K;
-  const bf16_t* b_tile = B + (size_t)n0 * K;
+  const bf16_t* b_tile = B_KN ? B + n0 : B + (size_t)n0 * K;
   auto issue_one = [&](char* st, int kt, int idx) {
     const int k0 = kt * BK;
     if (idx < INST) {
@@ -673,7 +682,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16,
                                                (int)a_voff[idx], 0, 0, 0);
     } else {
-      const __amdgpu_buffer_rsrc_t rows = stage_rows(b_tile + k0);
+      const __amdgpu_buffer_rsrc_t rows = stage_rows(b_tile + (B_KN ? (size_t)k0 * N : (size_t)k0));
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024),
                                                16, (int)b_voff[idx - INST], 0, 0, 0);
     }
@@ -721,11 +730,40 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
     return *reinterpret_cast<const bf16x8*>(st + b_row + j * 16 * 128 + (((ks * 4 + kq) ^ swz) << 4));
   };
 
+  // (K,N): the B operand of tile j wants, for column n = 16 j + fr, the k-step's k = 8 kq .. + 7; a
+  // transposing read hands a 16-lane group the 4 k-rows x 16 columns its lanes point at, turned
+  // round (a lane gets 4 k of one column): rows 8 kq .. + 3, then 8 kq + 4 .. + 7.
+  const int tr_k = 8 * kq + ((lane & 15) >> 2), tr_n = wn * 64 + 4 * (lane & 3);
+  const unsigned kn_base = (unsigned)(size_t)IRON_LDS_PTR(smem_nt) + NT_A_BYTES;
+  auto b_frag_kn = [&](int stage_bytes, int ks, int j, TrFrag& t) {
+    const int k = ks * 32 + tr_k, n = tr_n + j * 16;   // kn_swizzle(k + 4) = kn_swizzle(k): k % 8 < 4
+    const unsigned at = kn_base + stage_bytes + (((n >> 3) ^ kn_swizzle(k)) << 4) + ((n & 4) << 1);
+    t.lo = lds_read_tr16(at + k * 256);
+    t.hi = lds_read_tr16(at + (k + 4) * 256);
+  };
+  TrFrag tfb[2][4];
+  // The compiler does not count the transposing reads: a k-step's B fragments pass through this
+  // wait before they are joined into operands.  LDS reads return in order and the only reads
+  // issued after a k-step's B fragments are its four A fragments, so "at most four outstanding"
+  // is "B has arrived".
+  auto join_b = [&](int ks, bf16x8 (&b)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(tfb[ks][0].lo), "+v"(tfb[ks][0].hi), "+v"(tfb[ks][1].lo), "+v"(tfb[ks][1].hi),
+                                           "+v"(tfb[ks][2].lo), "+v"(tfb[ks][2].hi), "+v"(tfb[ks][3].lo), "+v"(tfb[ks][3].hi));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[j] = tr_join(tfb[ks][j]);
+  };
+
   wait_vmcnt<(NT_STAGES - 2) * LOADS>();   // stage 0 has landed once only the two younger ones are out
   block_barrier();
   bf16x8 af[2][4], bfr[2][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { bfr[0][i] = b_frag(smem_nt, 0, i); af[0][i] = a_frag(smem_nt, 0, i); }
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (B_KN) b_frag_kn(0, 0, i, tfb[0][i]);
+    else bfr[0][i] = b_frag(smem_nt, 0, i);
+  }
+  __builtin_amdgcn_sched_barrier(0);   // B's reads first, then A's: join_b counts on that order
+#pragma unroll
+  for (int i = 0; i < 4; ++i) af[0][i] = a_frag(smem_nt, 0, i);
   for (int kt = 0; kt < nk; ++kt) {
     // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
     // (into buffers nobody reads any more) rather than branch: every iteration issues the same
@@ -745,7 +783,9 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
         block_barrier();
       }
       const char* from = ks == 0 ? st : st1;
+      const int from_bytes = ((ks == 0 ? kt : kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
       const int nks = ks ^ 1;
+      if constexpr (B_KN) join_b(ks, bfr[ks]);
       // Source order is issue order (nothing crosses a sched_barrier): after an MFMA one fragment
       // read of the next k-step (B's first: its first MFMAs need all of them) or one load goes out.
 #pragma unroll
@@ -755,8 +795,10 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
           mfma_16x16x32_in_place(acc[i][j], bfr[ks][j], af[ks][i]);
           __builtin_amdgcn_sched_barrier(0);
           const int slot = i * 4 + j;
-          if (slot < 4) bfr[nks][slot] = b_frag(from, nks, slot);
-          else if (slot < 8) af[nks][slot - 4] = a_frag(from, nks, slot - 4);
+          if (slot < 4) {
+            if constexpr (B_KN) b_frag_kn(from_bytes, nks, slot, tfb[nks][slot]);
+            else bfr[nks][slot] = b_frag(from, nks, slot);
+          } else if (slot < 8) af[nks][slot - 4] = a_frag(from, nks, slot - 4);
           else if (slot & 1) issue_one(nst, kn, ks * 4 + (slot - 9) / 2);
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -844,8 +886,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       int tiles_n, int patched, int run_above,
                                                       int run_upto, QkvTail qkv) {
   if constexpr (QKV) to_cache_rows(qkv, valid, M);
-  if constexpr (T == 2 && !B_KN)
-    gemm_nt16_body<QKV>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+  if constexpr (T == 2)
+    gemm_nt16_body<QKV, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
   else
     gemm_nt_body<B_KN, QKV, T>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
 }
