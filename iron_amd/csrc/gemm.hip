@@ -323,19 +323,21 @@ __device__ __forceinline__ void to_cache_rows(QkvTail& t, const int* __restrict_
   t.Cv += (size_t)first * t.kv_n;
 }
 
-template <bool B_KN, bool QKV, int T>
-__device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
-                                             bf16_t* __restrict__ C_, int M, int N_, int K,
-                                             const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                             int patched, int run_above, int run_upto, const QkvTail& qkv) {
-  static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
-  static_assert(T == 2 || (T == 1 && !B_KN && !QKV), "64x64 tiles: B (N,K), plain output");
-  // T = 32x32 MFMA tiles a wave owns along each of m and n: 128x128 block tiles (T = 2), or 64x64
-  // (T = 1) for problems -- or row bounds -- whose 128x128 tiles would leave CUs idle.
-  constexpr int NT_BM = 64 * T, NT_BN = 64 * T;
+// 64 x 64 tiles, B as (N,K), for problems -- or row bounds -- whose 128 x 128 tiles would leave CUs
+// idle (k/v projections, short chunks): the direct-to-LDS pipeline of the 128 x 128 kernel below
+// (buffer loads, XOR-swizzled chunks, four stages, one barrier a stage before its last k-step) with
+// a wave owning one 32x32x16 MFMA tile.  A block takes 64 KB of LDS, so a CU holds two.
+// `qkv` carries only the optional residual epilogue here.
+__device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+                                               bf16_t* __restrict__ C, int M, int N, int K,
+                                               const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                               int patched, int run_above, int run_upto, const QkvTail& qkv) {
+  constexpr int NT_BM = 64, NT_BN = 64;
   constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int LOADS = 2 * INST;
+  constexpr int KSTEPS = BK / 16;
+  static_assert(LOADS == KSTEPS, "one load rides each k-step's MFMA");
   extern __shared__ __align__(16) char smem_nt[];
   const int Mv = bound_or(valid, M);
   // Two launches may share one problem, each taking a range of the row bound (see iron_gemm_bf16).
@@ -356,32 +358,14 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
     tm = first + in_band % height;
     tn = in_band / height;
   }
-  const int m0 = tm * NT_BM;
+  const int m0 = tm * NT_BM, n0 = tn * NT_BN;
   if (m0 >= Mv) return;
-  const bf16_t* B = B_;
-  bf16_t* C = C_;
-  int N = N_, which = 0;
-  if constexpr (QKV) {
-    const int q_tiles = N_ / NT_BN, kv_tiles = qkv.kv_n / NT_BN;
-    if (tn >= q_tiles) {
-      which = tn < q_tiles + kv_tiles ? 1 : 2;
-      tn -= q_tiles + (which - 1) * kv_tiles;
-      B = which == 1 ? qkv.Bk : qkv.Bv;
-      C = which == 1 ? qkv.Ck : qkv.Cv;
-      N = qkv.kv_n;
-    }
-  }
-  const int n0 = tn * NT_BN;
 
   // The wave's number is uniform, so what depends on it (LDS destinations, the rows it loads) stays
   // in scalar registers.
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int lrow = lane >> 3, pch = lane & 7;
-  // Loads are buffer loads straight into LDS.  The buffer is the tile's rows from the stage's k on
-  // (rebuilt once a stage with scalar instructions); a lane's place in it never changes, so it is a
-  // constant 32-bit vector offset and a load costs one scalar add (its LDS destination) on top of
-  // itself -- no vector ALU work between two MFMAs.
   int a_voff[INST], b_voff[INST];
 #pragma unroll
   for (int i = 0; i < INST; ++i) {
@@ -389,16 +373,10 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
     const int lch = pch ^ ((r >> 1) & 7);
     // Rows past the end re-read the last row; what they produce is never stored.
     a_voff[i] = (int)(((size_t)(min(m0 + r, M - 1) - m0) * K + lch * 8) * 2);
-    if constexpr (!B_KN) {
-      b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
-    } else {
-      const int kr = (wave * INST + i) * 4 + (lane >> 4);       // k row of the tile
-      const int lc = (lane & 15) ^ ((kr & 7) << 1);               // logical 16-byte chunk (8 n)
-      b_voff[i] = (int)(((size_t)kr * N + lc * 8) * 2);
-    }
+    b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
   }
   const bf16_t* a_tile = A + (size_t)m0 * K;
-  const bf16_t* b_tile = B_KN ? B + n0 : B + (size_t)n0 * K;
+  const bf16_t* b_tile = B + (size_t)n0 * K;
   // One load of the 2*INST a wave issues per stage (A's first, then B's).
   auto issue_one = [&](char* st, int kt, int idx) {
     const int k0 = kt * BK;
@@ -407,95 +385,51 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + (wave * INST + idx) * 1024), 16,
                                                (int)a_voff[idx], 0, 0, 0);
     } else {
-      const __amdgpu_buffer_rsrc_t rows = stage_rows(b_tile + (B_KN ? (size_t)k0 * N : (size_t)k0));
+      const __amdgpu_buffer_rsrc_t rows = stage_rows(b_tile + k0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + NT_A_BYTES + (wave * INST + idx - INST) * 1024),
                                                16, (int)b_voff[idx - INST], 0, 0, 0);
     }
   };
-  auto issue = [&](int kt, int buf) {
-    char* st = smem_nt + buf * NT_STAGE_BYTES;
-#pragma unroll
-    for (int idx = 0; idx < 2 * INST; ++idx) issue_one(st, kt, idx);
-  };
 
-  f32x16 acc[T][T];
+  f32x16 acc;
 #pragma unroll
-  for (int i = 0; i < T; ++i)
-#pragma unroll
-    for (int j = 0; j < T; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
 
+  // acc[e]: row fr of the wave's tile, column 8 (e/4) + 4 kh + e%4.
+  const int fr = lane & 31, kh = lane >> 5;
+  const int m = m0 + wm * 32 + fr, nb = n0 + wn * 32 + 4 * kh;
   // A residual's pieces this lane will add in the epilogue are requested now, so that their
   // latency passes under the whole product instead of at its end (N a multiple of 4: 8-byte pieces).
-  uint2 res[T][T][4];
-  const bool res_ahead = !QKV && qkv.residual != nullptr && (N & 3) == 0;
-  if constexpr (!QKV) {
-    if (res_ahead) {
+  uint2 res[4];
+  const bool res_ahead = qkv.residual != nullptr && (N & 3) == 0;
+  if (res_ahead) {
 #pragma unroll
-      for (int i = 0; i < T; ++i)
-#pragma unroll
-        for (int j = 0; j < T; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int m = min(m0 + wm * 32 * T + i * 32 + (lane & 31), M - 1);
-            const int n = min(n0 + wn * 32 * T + j * 32 + 8 * q + (lane >> 5) * 4, N - 4);
-            res[i][j][q] = *reinterpret_cast<const uint2*>(qkv.residual + (size_t)m * N + n);
-          }
-    }
+    for (int q = 0; q < 4; ++q)
+      res[q] = *reinterpret_cast<const uint2*>(qkv.residual + (size_t)min(m, M - 1) * N + min(nb + 8 * q, N - 4));
   }
 
   const int nk = K / BK;
   // Always three stages in flight before the loop (short K repeats its last stage), so the
   // loop's wait counts hold from the first iteration.
 #pragma unroll
-  for (int s = 0; s < NT_STAGES - 1; ++s) issue(min(s, nk - 1), s);
+  for (int s = 0; s < NT_STAGES - 1; ++s)
+#pragma unroll
+    for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_nt + s * NT_STAGE_BYTES, min(s, nk - 1), idx);
 
-  const int fr = lane & 31, kh = lane >> 5;
-  int a_off[T], a_swz[T], b_off[T], b_swz[T];
-#pragma unroll
-  for (int i = 0; i < T; ++i) {
-    const int ra = wm * 32 * T + i * 32 + fr, rb = wn * 32 * T + i * 32 + fr;
-    a_off[i] = ra * 128; a_swz[i] = (ra >> 1) & 7;
-    b_off[i] = NT_A_BYTES + rb * 128; b_swz[i] = (rb >> 1) & 7;
-  }
-  // (K,N) B: this lane's row within a 16-k step and its 8-byte piece of the row.
-  const int tr_k = (kh << 3) + ((lane & 15) >> 2);
-  int tr_n[T];
-#pragma unroll
-  for (int i = 0; i < T; ++i) tr_n[i] = wn * 64 + i * 32 + (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  const int ra = wm * 32 + fr, rb = wn * 32 + fr;
+  const int a_off = ra * 128, a_swz = (ra >> 1) & 7, b_off = NT_A_BYTES + rb * 128, b_swz = (rb >> 1) & 7;
+  auto a_frag = [&](const char* st, int ks) {
+    return *reinterpret_cast<const bf16x8*>(st + a_off + (((ks * 2 + kh) ^ a_swz) << 4));
+  };
+  auto b_frag = [&](const char* st, int ks) {
+    return *reinterpret_cast<const bf16x8*>(st + b_off + (((ks * 2 + kh) ^ b_swz) << 4));
+  };
 
-  auto read_frag_pair = [&](const char* st, int ks, int i, bf16x8& a, bf16x8& b, TrFrag& t) {
-    const int j = ks * 2 + kh;
-    a = *reinterpret_cast<const bf16x8*>(st + a_off[i] + ((j ^ a_swz[i]) << 4));
-    if constexpr (!B_KN) {
-      b = *reinterpret_cast<const bf16x8*>(st + b_off[i] + ((j ^ b_swz[i]) << 4));
-    } else {
-      const int k = ks * 16 + tr_k;  // rows k and k + 4, each with its own swizzle
-      const int c0 = ((tr_n[i] >> 3) ^ ((k & 7) << 1)) << 4;
-      const int c1 = ((tr_n[i] >> 3) ^ (((k + 4) & 7) << 1)) << 4;
-      const int half = (tr_n[i] & 4) << 1;
-      const unsigned base = (unsigned)(size_t)IRON_LDS_PTR(st + NT_A_BYTES + half);
-      t.lo = lds_read_tr16(base + k * 256 + c0);
-      t.hi = lds_read_tr16(base + (k + 4) * 256 + c1);
-    }
-  };
-  auto read_frags = [&](const char* st, int ks, bf16x8 (&af)[T], bf16x8 (&bfr)[T], TrFrag (&tf)[T]) {
-#pragma unroll
-    for (int i = 0; i < T; ++i) read_frag_pair(st, ks, i, af[i], bfr[i], tf[i]);
-  };
-  // A wave is alone on its SIMD, so nothing overlaps unless its own instruction stream interleaves:
-  // each k-step's four MFMAs are issued with the next step's fragment reads and a quarter of the
-  // stage being prefetched between them.  The one barrier a stage needs sits before its LAST k-step,
-  // whose fragments are in registers by then: after it every wave's share of the next stage has
-  // landed and nobody reads this stage any more, so the next stage's first fragments are read under
-  // the last k-step's MFMAs (no read latency is exposed where a stage begins) and the buffer of the
-  // stage before is free for the prefetch.
   wait_vmcnt<(NT_STAGES - 2) * LOADS>();   // stage 0 has landed once only the two younger ones are out
   block_barrier();
-  bf16x8 af[2][T], bfr[2][T];
-  TrFrag tf[2][T];
-  read_frags(smem_nt, 0, af[0], bfr[0], tf[0]);
+  bf16x8 af[2], bfr[2];
+  af[0] = a_frag(smem_nt, 0);
+  bfr[0] = b_frag(smem_nt, 0);
   for (int kt = 0; kt < nk; ++kt) {
     // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
     // (into buffers nobody reads any more) rather than branch: every iteration issues the same
@@ -505,107 +439,69 @@ __device__ __forceinline__ void gemm_nt_body(const bf16_t* __restrict__ A, const
     const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
     const char* st1 = smem_nt + ((kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
+    for (int ks = 0; ks < KSTEPS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks == BK / 16 - 1) {
+      if (ks == KSTEPS - 1) {
         // This wave has every fragment of stage kt; of the loads in flight the oldest LOADS are
-        // stage kt+1's (then stage kt+2's, and the 3 T issued so far for stage kt+3).
+        // stage kt+1's (then stage kt+2's, and the 3 issued so far for stage kt+3).
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        wait_vmcnt<LOADS + 3 * T>();
+        wait_vmcnt<LOADS + 3>();
         block_barrier();
       }
-      if constexpr (B_KN) {
-        lds_tr_wait(tf[cur][0], tf[cur][T - 1]);
-        bfr[cur][0] = tr_join(tf[cur][0]);
-        bfr[cur][T - 1] = tr_join(tf[cur][T - 1]);
-      }
-      // Source order is issue order (nothing crosses a sched_barrier): while an MFMA runs, half of
-      // the next k-step's fragment reads or one prefetch load goes out.
-#pragma unroll
-      for (int i = 0; i < T; ++i) {
-        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0], af[cur][i], acc[i][0], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (ks + 1 < BK / 16) read_frag_pair(st, ks + 1, i, af[nxt][i], bfr[nxt][i], tf[nxt][i]);
-        else read_frag_pair(st1, 0, i, af[nxt][i], bfr[nxt][i], tf[nxt][i]);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (T == 2) {
-          acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][1], af[cur][i], acc[i][1], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        issue_one(nst, kn, ks * T + i);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      // Source order is issue order (nothing crosses a sched_barrier): while the MFMA runs, the
+      // next k-step's fragment reads (the next stage's first, under the last k-step) and one
+      // prefetch load go out.
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur], af[cur], acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      af[nxt] = a_frag(ks + 1 < KSTEPS ? st : st1, ks + 1 < KSTEPS ? ks + 1 : 0);
+      bfr[nxt] = b_frag(ks + 1 < KSTEPS ? st : st1, ks + 1 < KSTEPS ? ks + 1 : 0);
+      issue_one(nst, kn, ks);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
   wait_vmcnt<0>();  // the idle fetches of the last iterations land before the block's LDS is released
-  if constexpr (QKV) {
-    if (which < 2) {
-      // acc[i][0][e] and acc[i][1][e] are columns c and c + 32 of the wave's head, c = 8 (e/4) + 4 kh + e%4,
-      // of row m = fr of tile i: the pair RoPE turns by the angle row's (cos, sin) number c.
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int m = min(m0 + wm * 64 + i * 32 + fr, M - 1);
-        const bf16_t* ang = qkv.angles + (size_t)m * 64 + 8 * kh;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float cs[8];
-          unpack8(*reinterpret_cast<const uint4*>(ang + 16 * q), cs);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float x1 = round_bf16(acc[i][0][4 * q + e]), x2 = round_bf16(acc[i][1][4 * q + e]);
-            const float c = cs[2 * e], sn = cs[2 * e + 1];
-            acc[i][0][4 * q + e] = x1 * c - x2 * sn;
-            acc[i][1][4 * q + e] = x2 * c + x1 * sn;
-          }
-        }
-      }
-    }
-  }
-  const int hi = kh * 4;
   const bool vec = (N & 3) == 0;
 #pragma unroll
-  for (int i = 0; i < T; ++i)
-#pragma unroll
-    for (int j = 0; j < T; ++j) {
-      const int m = m0 + wm * 32 * T + i * 32 + fr, nb = n0 + wn * 32 * T + j * 32;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = nb + 8 * q + hi;
-        if (m >= Mv || n >= N) continue;
-        bf16_t* p = C + (size_t)m * N + n;
-        if constexpr (!QKV) {
-          if (qkv.residual != nullptr) {   // the product rounded as it would be stored, then scale * it + residual
-            const bf16_t* r = qkv.residual + (size_t)m * N + n;
-            float rf[4] = {0.f, 0.f, 0.f, 0.f};
-            if (vec && n + 4 <= N) {
-              const uint2 rv = res_ahead ? res[i][j][q] : *reinterpret_cast<const uint2*>(r);
-              rf[0] = __uint_as_float(rv.x << 16); rf[1] = __uint_as_float(rv.x & 0xffff0000u);
-              rf[2] = __uint_as_float(rv.y << 16); rf[3] = __uint_as_float(rv.y & 0xffff0000u);
-            } else {
-              for (int e = 0; e < 4 && n + e < N; ++e) rf[e] = bf16_to_f32(r[e]);
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              acc[i][j][4 * q + e] = fmaf(qkv.residual_scale, round_bf16(acc[i][j][4 * q + e]), rf[e]);
-          }
-        }
-        if (vec && n + 4 <= N) {
-          *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
-                                                    pack_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]));
-        } else {
-          for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(acc[i][j][4 * q + e]);
-        }
+  for (int q = 0; q < 4; ++q) {
+    const int n = nb + 8 * q;
+    if (m >= Mv || n >= N) continue;
+    bf16_t* p = C + (size_t)m * N + n;
+    if (qkv.residual != nullptr) {   // the product rounded as it would be stored, then scale * it + residual
+      const bf16_t* r = qkv.residual + (size_t)m * N + n;
+      float rf[4] = {0.f, 0.f, 0.f, 0.f};
+      if (vec && n + 4 <= N) {
+        const uint2 rv = res_ahead ? res[q] : *reinterpret_cast<const uint2*>(r);
+        rf[0] = __uint_as_float(rv.x << 16); rf[1] = __uint_as_float(rv.x & 0xffff0000u);
+        rf[2] = __uint_as_float(rv.y << 16); rf[3] = __uint_as_float(rv.y & 0xffff0000u);
+      } else {
+        for (int e = 0; e < 4 && n + e < N; ++e) rf[e] = bf16_to_f32(r[e]);
       }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[4 * q + e] = fmaf(qkv.residual_scale, round_bf16(acc[4 * q + e]), rf[e]);
     }
+    if (vec && n + 4 <= N) {
+      *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[4 * q], acc[4 * q + 1]), pack_bf16(acc[4 * q + 2], acc[4 * q + 3]));
+    } else {
+      for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(acc[4 * q + e]);
+    }
+  }
 }
 
-// The 128 x 128 tile on 16x16x32 MFMAs, B as (N,K): the loop of gemm_nt_body with a wave's 64 x 64 as
-// 4 x 4 tiles of 16 x 16 (two 32-wide k-steps a stage; the part sustains more of these MFMAs under
-// its power limit than of the 32x32x16 form), accumulators tied in place, and the output staged
-// through LDS so that it leaves as whole 128-byte row segments (16 bytes a lane) instead of 8-byte
-// pieces of 16 rows an instruction -- the epilogue of the direct form took 3.3 us of a 2048^3
-// product's 20.  Same operands, bounds, fused-projection tail and residual epilogue as gemm_nt_body.
+// 128 x 128 x 64 tiles, four stages of 32 KB fed straight from global memory into LDS (buffer loads:
+// the tile's rows from the stage's k on are the buffer, rebuilt per stage with scalar instructions,
+// a lane's place in it a constant 32-bit offset, so a load costs one scalar add for its LDS
+// destination and no vector ALU work between two MFMAs); 16-byte chunks XOR-swizzled by the row so
+// unpadded rows read conflict-free; a bare s_barrier and counted s_waitcnt vmcnt(N).  Four waves, a
+// wave's 64 x 64 as 4 x 4 tiles of 16x16x32 MFMAs (two 32-wide k-steps a stage; the part sustains
+// more of these under its power limit than of the 32x32x16 form), accumulators tied in place.  A
+// wave is alone on its SIMD, so its own instruction stream interleaves: after an MFMA one fragment
+// read of the next k-step or one prefetch load goes out, and the stage's one barrier sits before
+// its second k-step, whose fragments are in registers by then.  B as (N,K), or as (K,N): then the
+// stage lands as stored and the B operands come from transposing reads.  The output is staged
+// through LDS so that it leaves as whole 128-byte row segments (16 bytes a lane).  QKV: the fused
+// projections' per-tile choice of weight and output, RoPE on the accumulators.  Otherwise `qkv`
+// carries the optional residual epilogue.
 template <bool QKV, bool B_KN = false>
 __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
                                                bf16_t* __restrict__ C_, int M, int N_, int K,
@@ -886,10 +782,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       int tiles_n, int patched, int run_above,
                                                       int run_upto, QkvTail qkv) {
   if constexpr (QKV) to_cache_rows(qkv, valid, M);
+  static_assert(T == 2 || (T == 1 && !B_KN && !QKV), "64x64 tiles: B (N,K), plain or residual output");
   if constexpr (T == 2)
     gemm_nt16_body<QKV, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
   else
-    gemm_nt_body<B_KN, QKV, T>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+    gemm_nt64_body(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
 }
 
 template <bool B_KN, bool QKV = false, int T = 2>
@@ -964,7 +861,7 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
     if (g < heads + kv_heads) return qkv.Bk + (size_t)(g - heads) * 64 * K;
     return qkv.Bv + (size_t)(g - heads - kv_heads) * 64 * K;
   };
-  // Buffer loads straight into LDS (see gemm_nt_body): the activations' tile rows are one buffer;
+  // Buffer loads straight into LDS (see gemm_nt16_body): the activations' tile rows are one buffer;
   // the eight weight rows of an instruction lie in one head, so each of a wave's weight
   // instructions has its own buffer, which starts at its first row.  The stage's k is the scalar
   // offset, a lane's place the constant vector offset.
@@ -1517,7 +1414,7 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
                                     QkvTail{});
   } else {
     if (bid < t64.tiles_m * t64.tiles_n)
-      gemm_nt_body<false, false, 1>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX,
+      gemm_nt64_body(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX,
                                     QkvTail{});
   }
 }
