@@ -323,11 +323,45 @@ __device__ __forceinline__ void to_cache_rows(QkvTail& t, const int* __restrict_
   t.Cv += (size_t)first * t.kv_n;
 }
 
+// Which tile a block computes.  Blocks are dispatched in id order and dealt round-robin over the 8
+// XCDs, each with an L2 of its own, so the order is chosen for what an XCD's blocks share:
+// `patched` (whole 8 x 4-tile patches, a multiple of 8 of them): an XCD owns patches, whose A and B
+// panels it re-reads from its own L2.  Few tile rows (under 8, and a multiple of 8 tile columns,
+// e.g. the 512 live rows of a prompt chunk): an XCD owns whole columns of tiles, so the weight tile
+// its blocks share crosses HBM once instead of once an XCD.  Otherwise bands of 8 tile rows.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int patched, int& tm, int& tn) {
+  if (patched) {
+    const int xcd = bid & 7, loc = bid >> 3;
+    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
+    const int patches_n = tiles_n >> 2;
+    tm = (patch / patches_n) * 8 + (within & 7);
+    tn = (patch % patches_n) * 4 + (within >> 3);
+  } else if (tiles_m < 8 && (tiles_n & 7) == 0) {
+    const int xcd = bid & 7, loc = bid >> 3;
+    tm = loc % tiles_m;
+    tn = (loc / tiles_m) * 8 + xcd;
+  } else {
+    constexpr int BAND = 8;
+    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
+    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
+    tm = first + in_band % height;
+    tn = in_band / height;
+  }
+}
+
 // 64 x 64 tiles, B as (N,K), for problems -- or row bounds -- whose 128 x 128 tiles would leave CUs
 // idle (k/v projections, short chunks): the direct-to-LDS pipeline of the 128 x 128 kernel below
-// (buffer loads, XOR-swizzled chunks, four stages, one barrier a stage before its last k-step) with
-// a wave owning one 32x32x16 MFMA tile.  A block takes 64 KB of LDS, so a CU holds two.
+// (buffer loads, XOR-swizzled chunks) with a wave owning one 32x32x16 MFMA tile.  A stage is four
+// MFMAs of a wave, far less than an LDS read takes to return, so the fragments of a WHOLE stage
+// are read one stage ahead into a second register set: at the top of stage kt the stage's one
+// barrier (stage kt+1 has landed in every wave, and nobody reads stage kt-1 any more), then the
+// eight fragment reads of stage kt+1, the loads of stage kt+STAGES-1 into stage kt-1's buffer, and
+// stage kt's four MFMAs out of registers on two accumulators (even and odd k-steps, so that no MFMA
+// waits for the one before it).  Reading a k-step ahead, as the larger tiles do, left every MFMA
+// waiting for its operands: 600 cycles a stage.  STAGES = 4 (64 KB: a CU holds two blocks) where
+// the tiles outnumber the CUs, 8 (128 KB, more loads in flight) where a CU has one block anyway.
 // `qkv` carries only the optional residual epilogue here.
+template <int STAGES>
 __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                bf16_t* __restrict__ C, int M, int N, int K,
                                                const int* __restrict__ valid, int tiles_m, int tiles_n,
@@ -337,27 +371,14 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
   constexpr int LOADS = 2 * INST;
   constexpr int KSTEPS = BK / 16;
-  static_assert(LOADS == KSTEPS, "one load rides each k-step's MFMA");
+  static_assert(LOADS == KSTEPS && STAGES >= 4, "one load rides each k-step's MFMA");
   extern __shared__ __align__(16) char smem_nt[];
   const int Mv = bound_or(valid, M);
   // Two launches may share one problem, each taking a range of the row bound (see iron_gemm_bf16).
   if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
-  const int bid = blockIdx.x;
-  if (patched) {
-    const int xcd = bid & 7, loc = bid >> 3;
-    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
-    const int patches_n = tiles_n >> 2;
-    tm = (patch / patches_n) * 8 + (within & 7);
-    tn = (patch % patches_n) * 4 + (within >> 3);
-  } else {
-    constexpr int BAND = 8;
-    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
-    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
-    tm = first + in_band % height;
-    tn = in_band / height;
-  }
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
   const int m0 = tm * NT_BM, n0 = tn * NT_BN;
   if (m0 >= Mv) return;
 
@@ -391,9 +412,11 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
     }
   };
 
-  f32x16 acc;
+  f32x16 acc[2];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[h][e] = 0.f;
 
   // acc[e]: row fr of the wave's tile, column 8 (e/4) + 4 kh + e%4.
   const int fr = lane & 31, kh = lane >> 5;
@@ -409,10 +432,10 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
   }
 
   const int nk = K / BK;
-  // Always three stages in flight before the loop (short K repeats its last stage), so the
+  // Always STAGES-1 stages in flight before the loop (short K repeats its last stage), so the
   // loop's wait counts hold from the first iteration.
 #pragma unroll
-  for (int s = 0; s < NT_STAGES - 1; ++s)
+  for (int s = 0; s < STAGES - 1; ++s)
 #pragma unroll
     for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_nt + s * NT_STAGE_BYTES, min(s, nk - 1), idx);
 
@@ -425,42 +448,40 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
     return *reinterpret_cast<const bf16x8*>(st + b_off + (((ks * 2 + kh) ^ b_swz) << 4));
   };
 
-  wait_vmcnt<(NT_STAGES - 2) * LOADS>();   // stage 0 has landed once only the two younger ones are out
+  wait_vmcnt<(STAGES - 2) * LOADS>();   // stage 0 has landed once only the younger ones are out
   block_barrier();
-  bf16x8 af[2], bfr[2];
-  af[0] = a_frag(smem_nt, 0);
-  bfr[0] = b_frag(smem_nt, 0);
-  for (int kt = 0; kt < nk; ++kt) {
-    // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
-    // (into buffers nobody reads any more) rather than branch: every iteration issues the same
-    // loads, which keeps the wait counts exact and the scheduling region whole.
-    const int kn = min(kt + NT_STAGES - 1, nk - 1);
-    char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
-    const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
-    const char* st1 = smem_nt + ((kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
+  bf16x8 af[2][KSTEPS], bfr[2][KSTEPS];   // [stage parity][k-step]
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) { af[0][ks] = a_frag(smem_nt, ks); bfr[0][ks] = b_frag(smem_nt, ks); }
+  // Two stages an iteration, so that the register sets are named at compile time.
+  auto stage = [&](int kt, auto parity) {
+    constexpr int P = decltype(parity)::value;
+    // Of this wave's loads in flight the oldest LOADS are stage kt+1's; the STAGES-3 stages after it may stay out.
+    wait_vmcnt<(STAGES - 3) * LOADS>();
+    block_barrier();
+    const char* st1 = smem_nt + ((kt + 1) % STAGES) * NT_STAGE_BYTES;     // past the end: a stage nobody needs
+    char* nst = smem_nt + ((kt + STAGES - 1) % STAGES) * NT_STAGE_BYTES;  // stage kt-1's buffer
+    const int kn = min(kt + STAGES - 1, nk - 1);   // past the end the last stage again: the wait counts stay exact
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks == KSTEPS - 1) {
-        // This wave has every fragment of stage kt; of the loads in flight the oldest LOADS are
-        // stage kt+1's (then stage kt+2's, and the 3 issued so far for stage kt+3).
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        wait_vmcnt<LOADS + 3>();
-        block_barrier();
-      }
-      // Source order is issue order (nothing crosses a sched_barrier): while the MFMA runs, the
-      // next k-step's fragment reads (the next stage's first, under the last k-step) and one
-      // prefetch load go out.
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur], af[cur], acc, 0, 0, 0);
+      acc[ks & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[P][ks], af[P][ks], acc[ks & 1], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      af[nxt] = a_frag(ks + 1 < KSTEPS ? st : st1, ks + 1 < KSTEPS ? ks + 1 : 0);
-      bfr[nxt] = b_frag(ks + 1 < KSTEPS ? st : st1, ks + 1 < KSTEPS ? ks + 1 : 0);
+      af[P ^ 1][ks] = a_frag(st1, ks);
+      bfr[P ^ 1][ks] = b_frag(st1, ks);
       issue_one(nst, kn, ks);
       __builtin_amdgcn_sched_barrier(0);
     }
+  };
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    stage(kt, std::integral_constant<int, 0>{});
+    stage(kt + 1, std::integral_constant<int, 1>{});
   }
+  if (kt < nk) stage(kt, std::integral_constant<int, 0>{});
 
   wait_vmcnt<0>();  // the idle fetches of the last iterations land before the block's LDS is released
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[0][e] += acc[1][e];
   const bool vec = (N & 3) == 0;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -478,12 +499,13 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
         for (int e = 0; e < 4 && n + e < N; ++e) rf[e] = bf16_to_f32(r[e]);
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[4 * q + e] = fmaf(qkv.residual_scale, round_bf16(acc[4 * q + e]), rf[e]);
+      for (int e = 0; e < 4; ++e) acc[0][4 * q + e] = fmaf(qkv.residual_scale, round_bf16(acc[0][4 * q + e]), rf[e]);
     }
     if (vec && n + 4 <= N) {
-      *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[4 * q], acc[4 * q + 1]), pack_bf16(acc[4 * q + 2], acc[4 * q + 3]));
+      *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[0][4 * q], acc[0][4 * q + 1]),
+                                                pack_bf16(acc[0][4 * q + 2], acc[0][4 * q + 3]));
     } else {
-      for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(acc[4 * q + e]);
+      for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(acc[0][4 * q + e]);
     }
   }
 }
@@ -518,20 +540,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
   if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
-  const int bid = blockIdx.x;
-  if (patched) {
-    const int xcd = bid & 7, loc = bid >> 3;
-    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
-    const int patches_n = tiles_n >> 2;
-    tm = (patch / patches_n) * 8 + (within & 7);
-    tn = (patch % patches_n) * 4 + (within >> 3);
-  } else {
-    constexpr int BAND = 8;
-    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
-    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
-    tm = first + in_band % height;
-    tn = in_band / height;
-  }
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
   const int m0 = tm * NT_BM;
   if (m0 >= Mv) return;
   const bf16_t* B = B_;
@@ -774,7 +783,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
 }
 
 
-template <bool B_KN, bool QKV, int T>
+template <bool B_KN, bool QKV, int T, int STAGES64 = 4>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__ A,
                                                       const bf16_t* __restrict__ B,
                                                       bf16_t* __restrict__ C, int M, int N, int K,
@@ -786,26 +795,31 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
   if constexpr (T == 2)
     gemm_nt16_body<QKV, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
   else
-    gemm_nt64_body(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+    gemm_nt64_body<STAGES64>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
 }
 
-template <bool B_KN, bool QKV = false, int T = 2>
+template <bool B_KN, bool QKV = false, int T = 2, int STAGES64 = 4>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                           const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}, int run_above = -1,
                           int run_upto = INT_MAX) {
   constexpr int BM = 64 * T, BN = 64 * T;
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / BN : (N + BN - 1) / BN;
-  const size_t lds = (size_t)NT_STAGES * (BM + BN) * BK * 2;
+  if constexpr (T == 1 && STAGES64 == 4) {
+    // No more 64 x 64 tiles than CUs: a CU has one block whatever its LDS, so the deeper pipeline.
+    if ((long)tiles_m * tiles_n <= 256)
+      return launch_gemm_nt<B_KN, QKV, 1, 8>(A, B, C, M, N, K, valid, s, qkv, run_above, run_upto);
+  }
+  const size_t lds = (size_t)(T == 1 ? STAGES64 : NT_STAGES) * (BM + BN) * BK * 2;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV, T>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV, T, STAGES64>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV, T>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
+  hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV, T, STAGES64>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
                      valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
   IRON_LAUNCH_CHECK();
 }
@@ -836,20 +850,7 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
   if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
-  const int bid = blockIdx.x;
-  if (patched) {
-    const int xcd = bid & 7, loc = bid >> 3;
-    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
-    const int patches_n = tiles_n >> 2;
-    tm = (patch / patches_n) * 8 + (within & 7);
-    tn = (patch % patches_n) * 4 + (within >> 3);
-  } else {
-    constexpr int BAND = 8;
-    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
-    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
-    tm = first + in_band % height;
-    tn = in_band / height;
-  }
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
   const int m0 = tm * Q3_BM;
   if (m0 >= Mv) return;
 
@@ -1163,20 +1164,7 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
-  const int bid = blockIdx.x;
-  if (patched) {
-    const int xcd = bid & 7, loc = bid >> 3;
-    const int patch = (loc >> 5) * 8 + xcd, within = loc & 31;
-    const int patches_n = tiles_n >> 2;
-    tm = (patch / patches_n) * 8 + (within & 7);
-    tn = (patch % patches_n) * 4 + (within >> 3);
-  } else {
-    constexpr int BAND = 8;
-    const int per_band = BAND * tiles_n, band = bid / per_band, first = band * BAND;
-    const int height = min(BAND, tiles_m - first), in_band = bid - band * per_band;
-    tm = first + in_band % height;
-    tn = in_band / height;
-  }
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
   const int m0 = tm * BIG_BM, n0 = tn * BIG_BN;
   if (m0 >= Mv) return;
 
@@ -1414,7 +1402,7 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
                                     QkvTail{});
   } else {
     if (bid < t64.tiles_m * t64.tiles_n)
-      gemm_nt64_body(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX,
+      gemm_nt64_body<8>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX,
                                     QkvTail{});
   }
 }

@@ -404,8 +404,17 @@ def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
         a, b = fused.logits(tokens), plain.logits(tokens)
         assert np.abs(a - b).max() <= 0.02 * np.abs(b).max(), step
         assert_close(a, golden.logits(tokens), f"fused step {step}")
+    # Greedy decoding through the fused step, judged by the step-by-step model on the same context:
+    # the two sum in different orders (tile sizes, MFMA shapes), so where the best two logits are
+    # closer than that they may pick either; every fused token must be one of the plain model's best.
     prompt = np.random.default_rng(8).integers(0, SCALED.vocab_size, 40)
-    assert fused.generate(prompt, 24) == plain.generate(prompt, 24)
+    drawn = fused.generate(prompt, 24)
+    assert len(drawn) == 24
+    context = [int(t) for t in prompt]
+    for step, token in enumerate(drawn):
+        row = plain.logits(np.asarray(context))
+        assert row[token] >= row.max() - 0.02 * np.abs(row).max(), (step, token, int(row.argmax()))
+        context.append(int(token))
     fused.release()
     plain.release()
 
