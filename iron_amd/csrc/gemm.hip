@@ -807,7 +807,9 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
   const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / BN : (N + BN - 1) / BN;
   if constexpr (T == 1 && STAGES64 == 4) {
     // No more 64 x 64 tiles than CUs: a CU has one block whatever its LDS, so the deeper pipeline.
-    if ((long)tiles_m * tiles_n <= 256)
+    // The same where the launch runs only for few rows of a row bound (the rest of its blocks
+    // leave at once): 512 live rows of a 2048-row prompt chunk are 256 tiles at 2048 columns.
+    if ((long)tiles_m * tiles_n <= 256 || run_upto != INT_MAX)
       return launch_gemm_nt<B_KN, QKV, 1, 8>(A, B, C, M, N, K, valid, s, qkv, run_above, run_upto);
   }
   const size_t lds = (size_t)(T == 1 ? STAGES64 : NT_STAGES) * (BM + BN) * BK * 2;
