@@ -1392,7 +1392,7 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
                                                           const bf16_t* __restrict__ B, bf16_t* __restrict__ C,
                                                           int M, int N, int K, const int* __restrict__ valid,
                                                           Tiling t256, Tiling t128, Tiling t64, int few256,
-                                                          int few128) {
+                                                          int few128, QkvTail tail) {
   // The blocks of this launch are four waves whatever the stand-alone large-tile launch uses.
   const int Mv = bound_or(valid, M), bid = blockIdx.x;
   if (BIG && Mv > few256) {
@@ -1400,24 +1400,28 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
       gemm_nt256_body<4, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched, -1, INT_MAX);
   } else if (Mv > few128) {
     if (bid < t128.tiles_m * t128.tiles_n)
-      gemm_nt16_body<false>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX,
-                                    QkvTail{});
+      gemm_nt16_body<false>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX, tail);
   } else {
     if (bid < t64.tiles_m * t64.tiles_n)
-      gemm_nt64_body<8>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX,
-                                    QkvTail{});
+      gemm_nt64_body<8>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX, tail);
   }
 }
 
 template <bool BIG>
 static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K, const int* valid,
-                              hipStream_t s, int few256, int few128) {
+                              hipStream_t s, int few256, int few128, QkvTail tail = QkvTail{}) {
   // Rows a tiling can be chosen for: the large one all of them, the others up to the next one's bound.
   const int rows128 = BIG ? (few256 < M ? few256 : M) : M, rows64 = few128 < M ? few128 : M;
   const int n128 = (N + 127) / 128, n64 = (N + 63) / 64;
   const Tiling t256{BIG ? M / BIG_BM : 0, BIG ? N / BIG_BN : 0, BIG ? patched_order(M / BIG_BM, N / BIG_BN) : 0};
-  const Tiling t128{(rows128 + 127) / 128, n128, patched_order((rows128 + 127) / 128, n128)};
-  const Tiling t64{(rows64 + 63) / 64, n64, patched_order((rows64 + 63) / 64, n64)};
+  // Tile rows rounded up to whole patches where that lets the XCD-aware order apply: the added
+  // tiles lie past the bound any block of that tiling runs for, and leave at once.
+  auto tiling = [](int tile_rows, int tile_cols) {
+    const int whole = (tile_rows + 7) & ~7;
+    if (tile_rows >= 8 && !patched_order(tile_rows, tile_cols) && patched_order(whole, tile_cols)) tile_rows = whole;
+    return Tiling{tile_rows, tile_cols, patched_order(tile_rows, tile_cols)};
+  };
+  const Tiling t128 = tiling((rows128 + 127) / 128, n128), t64 = tiling((rows64 + 63) / 64, n64);
   constexpr size_t out_bytes = (size_t)4 * 128 * BIG_OUT_ROW_BYTES(4);   // this launch's large tiles are four waves'
   constexpr size_t lds256 = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
   constexpr size_t lds128 = (size_t)NT_STAGES * 256 * BK * 2;
@@ -1433,7 +1437,7 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   if (t256.tiles_m * t256.tiles_n > blocks) blocks = t256.tiles_m * t256.tiles_n;
   if (t64.tiles_m * t64.tiles_n > blocks) blocks = t64.tiles_m * t64.tiles_n;
   hipLaunchKernelGGL((gemm_either_kernel<BIG>), dim3(blocks), dim3(256), lds, s, A, B, C, M, N, K, valid, t256, t128, t64,
-                     few256, few128);
+                     few256, few128, tail);
   IRON_LAUNCH_CHECK();
 }
 
@@ -1488,18 +1492,15 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
     }
     if (b_col_maj) {
       // 128x128 tiles that would occupy under half the CUs give way to 64x64 ones: always, where
-      // the shape says so; under a row bound, by a second launch for the low range of the bound
-      // (two launches, not one whose blocks choose: on their own the 64x64 tiles' 64 KB of LDS let
-      // a CU hold two blocks, worth more than the empty launch costs -- 35 against 40 us at
-      // 512 rows of 2048 x 2048 x 8192).
+      // the shape says so; under a row bound, the blocks of one launch choose where the bound is
+      // known (the few-row 64x64 tiles run the eight-stage pipeline, a block a CU, so nothing is
+      // lost to the launch's 128 KB of LDS and the second, empty launch is saved).
       const int tiles_n128 = (N + 127) / 128;
       const long tiles128 = (long)((M + 127) / 128) * tiles_n128;
       if (tiles128 < 128) return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s);
       const int few = tiles_n128 >= 128 ? 0 : 128 * (127 / tiles_n128);   // rows up to which 64x64 tiles win
       if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s);
-      const int rc = launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, QkvTail{}, few, INT_MAX);
-      if (rc != 0) return rc;
-      return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, QkvTail{}, -1, few);
+      return launch_gemm_either<false>(A, B, C, M, N, K, valid, s, 0, few);
     }
     // (K,N) B is read in whole tiles straight into LDS: N must be whole tiles.  Enough whole
     // 256x256 tiles to fill the chip, and a matrix a 32-bit byte offset spans: the large-tile kernel.
@@ -1534,9 +1535,7 @@ extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, con
   if (tiles128 < 128) return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, tail);
   const int few = tiles_n128 >= 128 ? 0 : 128 * (127 / tiles_n128);
   if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, tail);
-  const int rc = launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, tail, few, INT_MAX);
-  if (rc != 0) return rc;
-  return launch_gemm_nt<false, false, 1>(A, B, C, M, N, K, valid, s, tail, -1, few);
+  return launch_gemm_either<false>(A, B, C, M, N, K, valid, s, 0, few, tail);
 }
 
 static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,
