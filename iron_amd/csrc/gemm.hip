@@ -18,7 +18,6 @@
 #include "../../include/iron_hip.h"
 #include "common.h"
 
-#include <climits>
 
 namespace iron {
 
@@ -365,7 +364,7 @@ template <int STAGES>
 __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                bf16_t* __restrict__ C, int M, int N, int K,
                                                const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                               int patched, int run_above, int run_upto, const QkvTail& qkv) {
+                                               int patched, const QkvTail& qkv) {
   constexpr int NT_BM = 64, NT_BN = 64;
   constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
@@ -374,8 +373,6 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
   static_assert(LOADS == KSTEPS && STAGES >= 4, "one load rides each k-step's MFMA");
   extern __shared__ __align__(16) char smem_nt[];
   const int Mv = bound_or(valid, M);
-  // Two launches may share one problem, each taking a range of the row bound (see iron_gemm_bf16).
-  if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
   tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
@@ -528,7 +525,7 @@ template <bool QKV, bool B_KN = false>
 __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B_,
                                                bf16_t* __restrict__ C_, int M, int N_, int K,
                                                const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                               int patched, int run_above, int run_upto, const QkvTail& qkv) {
+                                               int patched, const QkvTail& qkv) {
   constexpr int NT_BM = 128, NT_BN = 128;
   constexpr int NT_A_BYTES = NT_BM * BK * 2, NT_STAGE_BYTES = (NT_BM + NT_BN) * BK * 2;
   constexpr int INST = NT_BM / 8 / 4;  // 1 KB loads of A (and of B) a wave issues per stage
@@ -537,7 +534,6 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
   static_assert(!(B_KN && QKV), "the fused projections read weights as stored, (N,K)");
   extern __shared__ __align__(16) char smem_nt[];
   const int Mv = bound_or(valid, M);
-  if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
   tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
@@ -788,29 +784,25 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const bf16_t* __restrict__
                                                       const bf16_t* __restrict__ B,
                                                       bf16_t* __restrict__ C, int M, int N, int K,
                                                       const int* __restrict__ valid, int tiles_m,
-                                                      int tiles_n, int patched, int run_above,
-                                                      int run_upto, QkvTail qkv) {
+                                                      int tiles_n, int patched, QkvTail qkv) {
   if constexpr (QKV) to_cache_rows(qkv, valid, M);
   static_assert(T == 2 || (T == 1 && !B_KN && !QKV), "64x64 tiles: B (N,K), plain or residual output");
   if constexpr (T == 2)
-    gemm_nt16_body<QKV, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+    gemm_nt16_body<QKV, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, qkv);
   else
-    gemm_nt64_body<STAGES64>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+    gemm_nt64_body<STAGES64>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, qkv);
 }
 
 template <bool B_KN, bool QKV = false, int T = 2, int STAGES64 = 4>
 static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
-                          const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}, int run_above = -1,
-                          int run_upto = INT_MAX) {
+                          const int* valid, hipStream_t s, QkvTail qkv = QkvTail{}) {
   constexpr int BM = 64 * T, BN = 64 * T;
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = QKV ? (N + 2 * qkv.kv_n) / BN : (N + BN - 1) / BN;
   if constexpr (T == 1 && STAGES64 == 4) {
     // No more 64 x 64 tiles than CUs: a CU has one block whatever its LDS, so the deeper pipeline.
-    // The same where the launch runs only for few rows of a row bound (the rest of its blocks
-    // leave at once): 512 live rows of a 2048-row prompt chunk are 256 tiles at 2048 columns.
-    if ((long)tiles_m * tiles_n <= 256 || run_upto != INT_MAX)
-      return launch_gemm_nt<B_KN, QKV, 1, 8>(A, B, C, M, N, K, valid, s, qkv, run_above, run_upto);
+    if ((long)tiles_m * tiles_n <= 256)
+      return launch_gemm_nt<B_KN, QKV, 1, 8>(A, B, C, M, N, K, valid, s, qkv);
   }
   const size_t lds = (size_t)(T == 1 ? STAGES64 : NT_STAGES) * (BM + BN) * BK * 2;
   static bool once = false;
@@ -822,7 +814,7 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV, T, STAGES64>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
-                     valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+                     valid, tiles_m, tiles_n, patched, qkv);
   IRON_LAUNCH_CHECK();
 }
 
@@ -842,14 +834,13 @@ template <int HPT>
 __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
                                                bf16_t* __restrict__ Cq, int M, int heads, int kv_heads, int K,
                                                const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                               int patched, int run_above, int run_upto, const QkvTail& qkv) {
+                                               int patched, const QkvTail& qkv) {
   constexpr int Q3_BN = 64 * HPT, Q3_STAGE_BYTES = (Q3_BM + Q3_BN) * BK * 2, NACC = 2 * HPT;
   constexpr int A_INST = Q3_BM / 8 / 4, B_INST = Q3_BN / 8 / 4, LOADS = A_INST + B_INST;   // 4 + 6 (or 2) a wave
   constexpr int PER = LOADS / 3, REST = LOADS - 3 * PER;   // loads issued under each of a stage's first three k-steps, and its last
   static_assert(PER <= NACC && REST <= NACC, "a load rides an MFMA");
   extern __shared__ __align__(16) char smem_q3[];
   const int Mv = bound_or(valid, M);
-  if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
   tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
@@ -995,9 +986,9 @@ __global__ __launch_bounds__(256) void qkv192_kernel(const bf16_t* __restrict__ 
                                                      const bf16_t* __restrict__ Bq, bf16_t* __restrict__ Cq,
                                                      int M, int heads, int kv_heads, int K,
                                                      const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                                     int patched, int run_above, int run_upto, QkvTail qkv) {
+                                                     int patched, QkvTail qkv) {
   to_cache_rows(qkv, valid, M);
-  qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, run_above, run_upto, qkv);
+  qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, qkv);
 }
 
 __global__ __launch_bounds__(256) void qkv64_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
@@ -1005,7 +996,7 @@ __global__ __launch_bounds__(256) void qkv64_kernel(const bf16_t* __restrict__ A
                                                     const int* __restrict__ valid, int tiles_m, int tiles_n,
                                                     int patched, QkvTail qkv) {
   to_cache_rows(qkv, valid, M);
-  qkv_heads_body<1>(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, -1, INT_MAX, qkv);
+  qkv_heads_body<1>(A, Bq, Cq, M, heads, kv_heads, K, valid, tiles_m, tiles_n, patched, qkv);
 }
 
 // Both tilings in one launch: the row bound is read on the device, and which tiling makes fewer
@@ -1026,14 +1017,13 @@ __global__ __launch_bounds__(256) void qkv_either_kernel(const bf16_t* __restric
   to_cache_rows(qkv, valid, M);
   if (Mv <= thin_upto) {   // so few rows that one-head tiles still fit one round over the chip
     if ((int)blockIdx.x < thin.tiles_m * thin.tiles_n)
-      qkv_heads_body<1>(A, Bq, Cq, M, heads, kv_heads, K, valid, thin.tiles_m, thin.tiles_n, thin.patched, -1, INT_MAX, qkv);
+      qkv_heads_body<1>(A, Bq, Cq, M, heads, kv_heads, K, valid, thin.tiles_m, thin.tiles_n, thin.patched, qkv);
   } else if (wide.tiles_n > 0 && past == (wide_top != 0)) {
     if ((int)blockIdx.x < wide.tiles_m * wide.tiles_n)
-      qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, -1, INT_MAX, qkv);
+      qkv_heads_body<3>(A, Bq, Cq, M, heads, kv_heads, K, valid, wide.tiles_m, wide.tiles_n, wide.patched, qkv);
   } else {
     if ((int)blockIdx.x < narrow.tiles_m * narrow.tiles_n)
-      gemm_nt16_body<true>(A, Bq, Cq, M, heads * 64, K, valid, narrow.tiles_m, narrow.tiles_n, narrow.patched,
-                                   -1, INT_MAX, qkv);
+      gemm_nt16_body<true>(A, Bq, Cq, M, heads * 64, K, valid, narrow.tiles_m, narrow.tiles_n, narrow.patched, qkv);
   }
 }
 
@@ -1084,7 +1074,7 @@ static int launch_qkv64(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, in
 }
 
 static int launch_qkv192(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, int heads, int kv_heads, int K,
-                         const int* valid, hipStream_t s, QkvTail qkv, int run_above, int run_upto) {
+                         const int* valid, hipStream_t s, QkvTail qkv) {
   const int tiles_m = (M + Q3_BM - 1) / Q3_BM, tiles_n = (heads + 2 * kv_heads) / 3;
   const size_t lds = (size_t)Q3_STAGES * Q3_STAGE_BYTES;
   static bool once = false;
@@ -1095,7 +1085,7 @@ static int launch_qkv192(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, i
     once = true;
   }
   hipLaunchKernelGGL(qkv192_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid,
-                     tiles_m, tiles_n, patched_order(tiles_m, tiles_n), run_above, run_upto, qkv);
+                     tiles_m, tiles_n, patched_order(tiles_m, tiles_n), qkv);
   IRON_LAUNCH_CHECK();
 }
 
@@ -1152,7 +1142,7 @@ template <int WAVES, int KB, bool B_KN = false>
 __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                 bf16_t* __restrict__ C, int M, int N, int K,
                                                 const int* __restrict__ valid, int tiles_m, int tiles_n,
-                                                int patched, int run_above, int run_upto) {
+                                                int patched) {
   static_assert(KB == 64, "k per stage: 64 (32 with four stages of half-line rows measured 13 % slower)");
   constexpr int ROWB = KB * 2;               // bytes of a tile row in LDS
   constexpr int CPR = KB / 8;                // its 16-byte chunks
@@ -1163,7 +1153,6 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   constexpr int TN = 8 / WAVES * 2;          // 32-column MFMA tiles a wave owns along n (4 or 2)
   extern __shared__ __align__(16) char smem_big[];
   const int Mv = bound_or(valid, M);
-  if (Mv <= run_above || Mv > run_upto) return;
 
   int tm, tn;
   tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
@@ -1376,9 +1365,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __
                                                          const bf16_t* __restrict__ B,
                                                          bf16_t* __restrict__ C, int M, int N, int K,
                                                          const int* __restrict__ valid, int tiles_m,
-                                                         int tiles_n, int patched, int run_above,
-                                                         int run_upto) {
-  gemm_nt256_body<WAVES, KB, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched, run_above, run_upto);
+                                                         int tiles_n, int patched) {
+  gemm_nt256_body<WAVES, KB, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched);
 }
 
 // A row bound read on the device decides which tile size fills the chip best (512 valid rows of
@@ -1397,13 +1385,13 @@ __global__ __launch_bounds__(256) void gemm_either_kernel(const bf16_t* __restri
   const int Mv = bound_or(valid, M), bid = blockIdx.x;
   if (BIG && Mv > few256) {
     if (bid < t256.tiles_m * t256.tiles_n)
-      gemm_nt256_body<4, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched, -1, INT_MAX);
+      gemm_nt256_body<4, BIG_KB>(A, B, C, M, N, K, valid, t256.tiles_m, t256.tiles_n, t256.patched);
   } else if (Mv > few128) {
     if (bid < t128.tiles_m * t128.tiles_n)
-      gemm_nt16_body<false>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, -1, INT_MAX, tail);
+      gemm_nt16_body<false>(A, B, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, tail);
   } else {
     if (bid < t64.tiles_m * t64.tiles_n)
-      gemm_nt64_body<8>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, -1, INT_MAX, tail);
+      gemm_nt64_body<8>(A, B, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, tail);
   }
 }
 
@@ -1443,7 +1431,7 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
 
 template <bool B_KN = false>
 static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
-                             const int* valid, hipStream_t s, int run_above = -1, int run_upto = INT_MAX) {
+                             const int* valid, hipStream_t s) {
   const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
   constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
   const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
@@ -1456,7 +1444,7 @@ static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M,
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
-                     tiles_m, tiles_n, patched, run_above, run_upto);
+                     tiles_m, tiles_n, patched);
   IRON_LAUNCH_CHECK();
 }
 
@@ -1585,7 +1573,7 @@ static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk
       if (wide_wins(live) != wide_wins(rows)) above = live;
   if (valid == nullptr) thin_upto = 0;
   if (above < 0 && thin_upto == 0) {
-    if (wide_wins(rows)) return launch_qkv192(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, -1, INT_MAX);
+    if (wide_wins(rows)) return launch_qkv192(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail);
     return launch_gemm_nt<false, true>(x, Wq, q_out, rows, heads * d, hidden, valid, s, tail);
   }
   return launch_qkv_either(x, Wq, q_out, rows, heads, kv_heads, hidden, valid, s, tail, above, wide_wins(rows), wide_ok,
