@@ -828,7 +828,7 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
 // tiles leave most CUs idle (512 rows of that layer: 192 tiles of one head against 64 of three).
 constexpr int Q3_BM = 128, Q3_BN = 192, Q3_STAGES = 3;
 constexpr int Q3_A_BYTES = Q3_BM * BK * 2, Q3_STAGE_BYTES = (Q3_BM + Q3_BN) * BK * 2;
-constexpr int Q1_STAGE_BYTES = (Q3_BM + 64) * BK * 2;
+constexpr int Q1_STAGE_BYTES = (Q3_BM + 64) * BK * 2, Q1_STAGES = 5;   // one head a tile: five 24 KB stages
 
 template <int HPT>
 __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bq,
@@ -892,17 +892,67 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
     for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
 
   const int nk = K / BK;
-#pragma unroll
-  for (int s = 0; s < Q3_STAGES - 1; ++s)
-#pragma unroll
-    for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_q3 + s * Q3_STAGE_BYTES, min(s, nk - 1), idx);
-
   const int fr = lane & 31, kh = lane >> 5;
   const int swz = (fr >> 1) & 7;   // tile rows are multiples of 32 apart: one swizzle for all
   const int a_off = (wave * 32 + fr) * 128, b_off = Q3_A_BYTES + fr * 128;
   auto frag = [&](const char* st, int off, int ks) {
     return *reinterpret_cast<const bf16x8*>(st + off + (((ks * 2 + kh) ^ swz) << 4));
   };
+  if constexpr (HPT == 1) {
+    // One head a tile: a k-step is two MFMAs of a wave, far less than an LDS read takes to return,
+    // so -- as in gemm_nt64_body -- the fragments of a whole stage are read one stage ahead into a
+    // second register set.  At the top of stage kt the one barrier (stage kt+1 has landed in every
+    // wave, nobody reads stage kt-1 any more), then stage kt's eight MFMAs out of registers with
+    // the twelve fragment reads of stage kt+1 and the six loads of stage kt+STAGES-1 between them.
+    constexpr int STAGES = Q1_STAGES, KSTEPS = BK / 16;
+    static_assert(LOADS == 6 && KSTEPS == 4, "six loads and twelve reads ride eight MFMAs");
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+#pragma unroll
+      for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_q3 + s * Q3_STAGE_BYTES, min(s, nk - 1), idx);
+    wait_vmcnt<(STAGES - 2) * LOADS>();   // stage 0 has landed once only the younger ones are out
+    block_barrier();
+    bf16x8 af[2][KSTEPS], bfr[2][KSTEPS][2];   // [stage parity][k-step]([column half])
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      af[0][ks] = frag(smem_q3, a_off, ks);
+      bfr[0][ks][0] = frag(smem_q3, b_off, ks);
+      bfr[0][ks][1] = frag(smem_q3, b_off + 32 * 128, ks);
+    }
+    auto stage = [&](int kt, auto parity) {
+      constexpr int P = decltype(parity)::value;
+      // Of this wave's loads in flight the oldest LOADS are stage kt+1's; the STAGES-3 stages after it may stay out.
+      wait_vmcnt<(STAGES - 3) * LOADS>();
+      block_barrier();
+      const char* st1 = smem_q3 + ((kt + 1) % STAGES) * Q3_STAGE_BYTES;     // past the end: a stage nobody needs
+      char* nst = smem_q3 + ((kt + STAGES - 1) % STAGES) * Q3_STAGE_BYTES;  // stage kt-1's buffer
+      const int kn = min(kt + STAGES - 1, nk - 1);   // past the end the last stage again: the wait counts stay exact
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[P][ks][0], af[P][ks], acc[0], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        af[P ^ 1][ks] = frag(st1, a_off, ks);
+        bfr[P ^ 1][ks][0] = frag(st1, b_off, ks);
+        if (ks < 2) issue_one(nst, kn, ks);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[P][ks][1], af[P][ks], acc[1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        bfr[P ^ 1][ks][1] = frag(st1, b_off + 32 * 128, ks);
+        issue_one(nst, kn, 2 + ks);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+      stage(kt, std::integral_constant<int, 0>{});
+      stage(kt + 1, std::integral_constant<int, 1>{});
+    }
+    if (kt < nk) stage(kt, std::integral_constant<int, 0>{});
+  } else {
+#pragma unroll
+  for (int s = 0; s < Q3_STAGES - 1; ++s)
+#pragma unroll
+    for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_q3 + s * Q3_STAGE_BYTES, min(s, nk - 1), idx);
 
   wait_vmcnt<LOADS>();   // stage 0 has landed once only stage 1's loads are out
   block_barrier();
@@ -940,6 +990,7 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  }
   }
   wait_vmcnt<0>();   // the idle fetches of the last iterations land before the block's LDS is released
 
@@ -1060,7 +1111,7 @@ static int launch_qkv_either(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int 
 static int launch_qkv64(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, int heads, int kv_heads, int K,
                         const int* valid, hipStream_t s, QkvTail qkv) {
   const int tiles_m = (M + Q3_BM - 1) / Q3_BM, tiles_n = heads + 2 * kv_heads;
-  const size_t lds = (size_t)Q3_STAGES * Q1_STAGE_BYTES;
+  const size_t lds = (size_t)Q1_STAGES * Q1_STAGE_BYTES;
   static bool once = false;
   if (!once) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv64_kernel),
