@@ -169,6 +169,36 @@ def test_gemm_weight_layout_fast_paths(cuda, M, Kdim, N, rows):
     assert np.all(got[lim:] == 5.0)
 
 
+@pytest.mark.parametrize("M,Kdim,N,rows", [
+    # 64 x 64 tiles, eight stages (no more tiles than CUs): fewer k-stages than the pipeline is deep, an odd count, many
+    (512, 64, 2048, None), (512, 192, 2048, None), (512, 576, 2048, None), (448, 1024, 1024, None),
+    # 64 x 64 tiles, four stages (more tiles than CUs, too few for 128 x 128 ones): one stage, odd, even
+    (1024, 64, 1536, None), (1024, 320, 1536, None), (1024, 512, 1536, 1000),
+    # a row bound under which the blocks of one launch pick 64 x 64 tiles, short and odd in k
+    (2048, 64, 2048, 512), (2048, 192, 2048, 300), (2048, 576, 2048, 896), (2048, 576, 2048, 897)])
+@pytest.mark.parametrize("residual", [False, True])
+def test_gemm_small_tiles_at_every_depth(cuda, M, Kdim, N, rows, residual):
+    """The whole-stage-ahead pipelines of the 64 x 64 tiles where they start and end: K of one stage,
+    fewer stages than are in flight, odd and even counts, with and without the residual epilogue."""
+    rng = np.random.default_rng(M + Kdim + N)
+    A, B, R = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.1), bf(rng, M, N)
+    want = ops.gemm(A, B, b_col_maj=True)
+    if residual:
+        want = round_bf16(np.float32(0.5) * want + R)
+    lim = M if rows is None else rows
+    if rows is not None:
+        A[rows:] = np.nan
+    C = out_like((M, N), cuda, fill=5.0)
+    bound = None if rows is None else word(rows, cuda)
+    if residual:
+        K.gemm_residual(dev(A, cuda), dev(B, cuda), dev(R, cuda), C, M=M, N=N, K=Kdim, residual_scale=0.5, valid=bound)
+    else:
+        K.gemm(dev(A, cuda), dev(B, cuda), C, M=M, N=N, K=Kdim, b_col_maj=True, valid=bound)
+    got = from_torch(C)
+    close(got[:lim], want[:lim], rtol=1e-2, atol=2e-2)
+    assert np.all(got[lim:] == 5.0)
+
+
 @pytest.mark.parametrize("rows,bound,H,G", [(2048, None, 32, 8), (256, 150, 16, 4), (128, None, 2, 2),
                                             # bounds on either side of where the 192-wide tiles take over
                                             (2048, 1280, 32, 8), (2048, 1281, 32, 8), (2048, 1999, 32, 8),
@@ -182,6 +212,31 @@ def test_prefill_qkv_equals_three_projections_then_rope(cuda, rows, bound, H, G)
     x = bf(rng, rows, E)
     Wq, Wk, Wv = bf(rng, H * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05)
     table = round_bf16(ops.rope_angles(D, rows + 5, 500000.0))[5:]
+    lim = rows if bound is None else bound
+    q, k, v = (ops.gemm(x, W, b_col_maj=True) for W in (Wq, Wk, Wv))
+    want_q = ops.rope(q.reshape(rows * H, D), table).reshape(rows, H * D)
+    want_k = ops.rope(k.reshape(rows * G, D), table).reshape(rows, G * D)
+    if bound is not None:
+        x[bound:] = np.nan
+    outs = [out_like((rows, n), cuda, fill=7.0) for n in (H * D, G * D, G * D)]
+    K.prefill_qkv(dev(x, cuda), dev(Wq, cuda), dev(Wk, cuda), dev(Wv, cuda), dev(table, cuda), *outs, rows=rows,
+                  hidden=E, heads=H, kv_heads=G, d=D, valid=None if bound is None else word(bound, cuda))
+    for got, want in zip(outs, (want_q, want_k, v)):
+        got = from_torch(got)
+        close(got[:lim], want[:lim], rtol=1e-2, atol=1e-2)
+        assert np.all(got[lim:] == 7.0)
+
+
+@pytest.mark.parametrize("E", [64, 192, 320])
+@pytest.mark.parametrize("rows,bound", [(512, None), (2048, 600)])
+def test_prefill_qkv_one_head_tiles_at_short_hidden(cuda, E, rows, bound):
+    """The one-head tiles a short chunk takes (whole-stage-ahead pipeline, five stages) with fewer
+    k-stages than are in flight and an odd count of them."""
+    rng = np.random.default_rng(E + rows)
+    H, G, D = 32, 8, 64
+    x = bf(rng, rows, E)
+    Wq, Wk, Wv = bf(rng, H * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05), bf(rng, G * D, E, scale=0.05)
+    table = round_bf16(ops.rope_angles(D, rows, 500000.0))
     lim = rows if bound is None else bound
     q, k, v = (ops.gemm(x, W, b_col_maj=True) for W in (Wq, Wk, Wv))
     want_q = ops.rope(q.reshape(rows * H, D), table).reshape(rows, H * D)
