@@ -234,13 +234,14 @@ class CausalLM(iron.Graph):
         return [{}, {"ids": ((self.config.prefill_chunk,), np.int32)}]
 
     def load_versions(self, *, capture: bool = True, check: bool = False, fuse: bool = True) -> None:
-        """Compile both versions into the shared arena, upload the weights, capture the decode step.
-        ``fuse=False`` launches every recorded step on its own (what ``check=True`` implies);
-        ``capture=False`` keeps the decode step eager."""
+        """Compile both versions into the shared arena, upload the weights, capture each as a HIP
+        graph (the prompt chunk's ids are copied into its arena slot and its per-call words
+        rewritten before every replay).  ``fuse=False`` launches every recorded step on its own
+        (what ``check=True`` implies); ``capture=False`` keeps both versions eager."""
         for_decode, for_prompt = self.shapes()
         try:
             decode = self.compile(capture=capture, check=check, fuse=fuse, **for_decode)
-            prompt = self.compile(capture=False, check=check, fuse=fuse, **for_prompt)
+            prompt = self.compile(capture=capture, check=check, fuse=fuse, **for_prompt)
             for version in (decode, prompt):
                 version.load()
         except Exception:
