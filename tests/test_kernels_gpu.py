@@ -169,6 +169,23 @@ def test_gemm_weight_layout_fast_paths(cuda, M, Kdim, N, rows):
     assert np.all(got[lim:] == 5.0)
 
 
+@pytest.mark.parametrize("M,Kdim,N", [(130, 128, 264), (200, 192, 136), (1000, 256, 1000), (65, 64, 65), (2047, 320, 2050), (333, 128, 384)])
+@pytest.mark.parametrize("b_col_maj", [False, True])
+def test_gemm_direct_to_lds_tiles_at_ragged_edges(cuda, M, Kdim, N, b_col_maj):
+    """K a multiple of 64 takes the direct-to-LDS tiles whatever M and N are: rows and columns past
+    the edge are clamped on the way in and never stored, and nothing beyond C is touched."""
+    if not b_col_maj:
+        N = (N + 7) // 8 * 8   # B as (K,N) is loaded 16 bytes along N
+    rng = np.random.default_rng(M * 7 + N)
+    A, B = bf(rng, M, Kdim), bf(rng, (N if b_col_maj else Kdim), (Kdim if b_col_maj else N), scale=0.1)
+    guard = 64
+    C = out_like((M * N + guard,), cuda, fill=3.0)
+    K.gemm(dev(A, cuda), dev(B, cuda), C[: M * N].view(M, N), M=M, N=N, K=Kdim, b_col_maj=b_col_maj)
+    got = from_torch(C)
+    close(got[: M * N].reshape(M, N), ops.gemm(A, B, b_col_maj=b_col_maj), rtol=1e-2, atol=2e-2)
+    assert np.all(got[M * N:] == 3.0)
+
+
 @pytest.mark.parametrize("M,Kdim,N,rows", [
     # 64 x 64 tiles, eight stages (no more tiles than CUs): fewer k-stages than the pipeline is deep, an odd count, many
     (512, 64, 2048, None), (512, 192, 2048, None), (512, 576, 2048, None), (448, 1024, 1024, None),
