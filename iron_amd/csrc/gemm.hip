@@ -1,20 +1,17 @@
 // GEMM: C = A @ B in bf16 on the MFMA matrix cores, f32 accumulation, one rounding.
 //
-// A block of 4 waves computes a BM x BN tile of C.  Per 64-wide K step the block
-// stages a BM x 64 tile of A and a BN x 64 tile of B in LDS (both K-contiguous,
-// rows padded to 72 elements so the 16-byte fragment reads of 32 consecutive rows
-// fall in distinct banks), double-buffered: the global loads of step k+1 are in
-// flight while the MFMAs of step k run.  A wave owns a (BM/WM) x (BN/WN) sub-tile
-// as 32x32 MFMA tiles (v_mfma_f32_32x32x16_bf16: a lane supplies 8 consecutive k of
-// one row of each operand).
+// Two families of kernels.  The general one (gemm_kernel, first below) takes every shape and
+// option: a block of 4 waves computes a BM x BN tile of C; per 64-wide K step it stages a BM x 64
+// tile of A and a BN x 64 tile of B in LDS through registers (both K-contiguous, rows padded to
+// 72 elements so the 16-byte fragment reads of 32 consecutive rows fall in distinct banks),
+// double-buffered; a wave owns a (BM/WM) x (BN/WN) sub-tile as 32x32x16 MFMA tiles; B as (K,N) is
+// transposed on its way into LDS (a thread loads a 4(k) x 8(n) patch and writes eight 8-byte
+// k-runs).  The fast ones (K a multiple of 64, row-major C) feed LDS straight from global memory
+// and come in four tile sizes: 64 x 64, 128 x 128, 128 x 192 / 128 x 64 for the fused projections,
+// and 256 x 256; each is described where it stands.
 //
-// B as stored by a checkpoint, (N,K), is already K-contiguous.  B as (K,N) is
-// transposed on its way into LDS: a thread loads a 4(k) x 8(n) patch and writes
-// eight 8-byte k-runs.
-//
-// For a row-major C the MFMA is issued with the operands swapped (B tile as the
-// "A" operand), so a lane ends up holding 4 consecutive columns of one row of C
-// and stores them as 8 bytes.
+// For a row-major C the MFMA is issued with the operands swapped (B tile as the "A" operand), so a
+// lane ends up holding 4 consecutive columns of one row of C and stores them as 8 bytes.
 #include "../../include/iron_hip.h"
 #include "common.h"
 
@@ -272,23 +269,22 @@ __global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A,
 
 
 // ---------------------------------------------------------------------------
-// Fast path: A (M,K) and B (N,K) both K-contiguous, K a multiple of 64, row-major C.
+// Fast paths: A (M,K) K-contiguous, K a multiple of 64, row-major C.
 //
-// Tiles stream global -> LDS directly (global_load_lds_dwordx4: no VGPR staging, and the
-// L2 -> CU path delivers more per clock to LDS than to registers), four 32 KB stages deep.
-// A wave instruction moves 8 rows x 128 B; the 16-byte chunk a lane fetches is XOR-swizzled
-// by its row ((row >> 1) & 7) so the fragment reads of 16 consecutive rows fall in distinct
-// bank groups although LDS rows are unpadded.  The stage barrier is a bare s_barrier: the
-// fence __syncthreads() carries would wait for every outstanding load (vmcnt(0)) and drain
-// the prefetch; each wave instead waits until only the two youngest stages are in flight.
-// Blocks are ordered so each XCD (block id mod 8) owns 8x4-tile patches and re-reads its
-// A/B panels from its own L2.
+// Tiles stream global -> LDS directly (buffer loads with the LDS bit: no VGPR staging, and the
+// L2 -> CU path delivers more per clock to LDS than to registers), several stages deep.  A wave
+// instruction moves 8 rows x 128 B; the 16-byte chunk a lane fetches is XOR-swizzled by its row
+// ((row >> 1) & 7) so the fragment reads of 16 consecutive rows fall in distinct bank groups
+// although LDS rows are unpadded.  The stage barrier is a bare s_barrier: the fence
+// __syncthreads() carries would wait for every outstanding load (vmcnt(0)) and drain the
+// prefetch; each wave instead waits until only the younger stages are in flight.
 constexpr int NT_STAGES = 4;
 
-// B_KN: B is (K,N) row-major.  Its tile lands in LDS as stored, [64 k][128 n] (a wave
-// instruction moves 4 k-rows x 256 B, chunks swizzled by 2*(k & 7)), and the fragments are
-// fetched with the transposing LDS read (ds_read_b64_tr_b16): within 16 lanes, lane i points
-// at 4 consecutive n of row k0 + i/4 and receives k0..k0+3 of column n0 + i%16.
+// B_KN (128 x 128 and 256 x 256 tiles): B is (K,N) row-major.  Its tile lands in LDS as stored, a
+// row a k (a wave instruction moves 4 k-rows x 256 B, or 2 x 512 B; chunks swizzled by the row so
+// that the four rows of a 16-lane group, and the groups of a pass, lie in different banks), and
+// the fragments are fetched with the transposing LDS read (ds_read_b64_tr_b16): within 16 lanes,
+// lane i points at 4 consecutive n of row k0 + i/4 and receives k0..k0+3 of column n0 + i%16.
 // QKV: one launch for a prompt chunk's three projections and the rotation of two of them.  B, C and
 // N then stand for q's weight (N,K), output and width; `qkv` brings k's and v's (each kv_n wide,
 // widths multiples of the 128-column tile) and the chunk's angle rows (M, 64; cos and sin

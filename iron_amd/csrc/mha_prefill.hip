@@ -21,7 +21,7 @@ constexpr int BQ = 128;   // query rows per block
 constexpr int BKV = 64;   // key rows per tile
 constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks split each block's tiles over two halves
 
-// K and V tiles go straight from global memory into LDS (global_load_lds, no register staging), as
+// K and V tiles go straight from global memory into LDS (buffer loads with the LDS bit, no register staging), as
 // stored: [64 keys][D], STAGES tiles deep.  16-byte chunks of a row are XOR-swizzled so unpadded
 // rows read without bank conflicts: K by (key >> 1) & 7 for its 16-byte fragment reads, V by
 // 2 * (key & 3) for the transposing reads (ds_read_b64_tr_b16) that deliver V^T fragments.  A bare
