@@ -16,7 +16,8 @@ in a prompt chunk's version (several rows, 64-wide heads),
 
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
   ... and Copy k/v -> the chunk's cache rows             => iron_prefill_qkv_cache_bf16
-  SiLU, ElementwiseMul (the gated feed-forward)          => iron_silu_mul_bf16
+  GEMM (up), SiLU (of the gate), ElementwiseMul          => iron_gemm_gated_bf16
+  SiLU, ElementwiseMul (no such product before them)     => iron_silu_mul_bf16
   GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
 
 and in either,
@@ -258,6 +259,29 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), R=tensor(other), C=tensor(ad.outputs["y"]))
                 kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, residual_scale=scale, valid=word(gv))
                 got = Fused("gemm_add", i, 2, lambda a=args, kw=kw: kernels.gemm_residual(**a, **kw))
+        elif (_name(s) == "GEMM" and i + 2 < len(steps) and _name(steps[i + 1]) == "SiLU"
+              and _name(steps[i + 2]) == "ElementwiseMul"
+              and s.op.b_col_maj and not s.op.c_col_maj and "valid_k" not in s.values
+              and s.op.M >= 64 and s.op.N >= 64 and s.op.K % 64 == 0):
+            # a gated feed-forward's second projection over many rows: the activated gate rides its epilogue
+            sl, ml = steps[i + 1], steps[i + 2]
+            up, gate, act = s.outputs["C"], sl.inputs["x"], sl.outputs["y"]
+            a, b = ml.inputs["a"], ml.inputs["b"]
+            paired = (_same_view(a, act) and _same_view(b, up)) or (_same_view(a, up) and _same_view(b, act))
+            gv, sv, mv = s.values.get("valid"), sl.values.get("valid"), ml.values.get("valid")
+            # the elementwise bounds count elements, the product's rows
+            bounds_agree = sv == mv and ((gv is None and sv is None) or (
+                gv is not None and sv is not None and gv.value == sv.value and gv.linear and sv.linear
+                and sv.scale == gv.scale * s.op.N and sv.bias == gv.bias * s.op.N))
+            flat = all(h.index is None and h.ids is None
+                       for h in (*s.inputs.values(), up, gate, act, a, b, ml.outputs["y"]))
+            if (paired and flat and once(up) and once(act) and bounds_agree and gate.buffer is not up.buffer
+                    and gate.elements == up.elements and sl.op.size == up.elements and ml.op.size == up.elements
+                    and ml.outputs["y"].elements == up.elements
+                    and set(sl.values) <= {"valid"} and set(ml.values) <= {"valid"}):
+                args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), G=tensor(gate), C=tensor(ml.outputs["y"]))
+                kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, valid=word(gv))
+                got = Fused("gemm_gated", i, 3, lambda a=args, kw=kw: kernels.gemm_gated(**a, **kw))
         elif _name(s) == "SiLU" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseMul":
             # a gated feed-forward's activation and gate over many rows: one pass instead of two
             m = steps[i + 1]

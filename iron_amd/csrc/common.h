@@ -71,6 +71,9 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
   return v;
 }
 
+// SiLU as every kernel here computes it, so that fused and separate launches round alike.
+__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
+
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // 16-byte streaming load that does not displace reusable lines in the caches.
 __device__ __forceinline__ uint4 load_stream(const uint4* p) {

@@ -302,6 +302,9 @@ struct QkvTail {
   // (one fused multiply-add; residual (M, N) like C), when residual is not NULL.
   const bf16_t* residual;
   float residual_scale;
+  // ... or, with gated set, C = bf16(bf16(SiLU(residual)) * bf16(A B)): `residual` then holds a gated
+  // feed-forward's other product, and this one leaves as the activated gate times it.
+  int gated;
   // Of the fused projections again: Ck and Cv are KV caches of kv_rows rows (a row kv_n wide, as the
   // projections write one), and the chunk's rows go to rows *kv_row0 on, when kv_row0 is not NULL.
   const int* kv_row0;
@@ -492,7 +495,10 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
         for (int e = 0; e < 4 && n + e < N; ++e) rf[e] = bf16_to_f32(r[e]);
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[0][4 * q + e] = fmaf(qkv.residual_scale, round_bf16(acc[0][4 * q + e]), rf[e]);
+      for (int e = 0; e < 4; ++e) {
+        const float prod = round_bf16(acc[0][4 * q + e]);
+        acc[0][4 * q + e] = qkv.gated ? round_bf16(silu_f32(rf[e])) * prod : fmaf(qkv.residual_scale, prod, rf[e]);
+      }
     }
     if (vec && n + 4 <= N) {
       *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[0][4 * q], acc[0][4 * q + 1]),
@@ -761,7 +767,8 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
           for (int e = 0; e < 8 && out_n + e < N; ++e) rf[e] = bf16_to_f32(qkv.residual[(size_t)m * N + out_n + e]);
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = fmaf(qkv.residual_scale, x[e], rf[e]);
+        for (int e = 0; e < 8; ++e)
+          x[e] = qkv.gated ? round_bf16(silu_f32(rf[e])) * x[e] : fmaf(qkv.residual_scale, x[e], rf[e]);
         v = pack8(x);
       }
     }
@@ -1551,19 +1558,17 @@ extern "C" int iron_gemm_bf16(const uint16_t* A, const uint16_t* B, uint16_t* C,
   return launch_gemm<64, 64, 2, 2>(A, B, C, M, N, K, b_col_maj, c_col_maj, valid, valid_k, s);
 }
 
-extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
-                                       int N, int K, float residual_scale, const int* valid, void* stream) {
-  IRON_REQUIRE(A && B && R && C, "gemm_residual: null operand");
+// A product over many rows whose epilogue reads a second (M, N) operand: the residual sum or the gate.
+static int gemm_with_tail(const char* what, const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C,
+                          int M, int N, int K, const QkvTail& tail, const int* valid, void* stream) {
+  IRON_REQUIRE(A && B && R && C, "%s: null operand", what);
   IRON_REQUIRE(K <= (1 << 22) && N <= (1 << 22),
-               "gemm_residual: K (%d) and N (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", K, N);
+               "%s: K (%d) and N (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", what, K, N);
   IRON_REQUIRE(M >= 64 && N >= 64 && K > 0 && K % BK == 0,
-               "gemm_residual: M (%d) and N (%d) at least 64, K (%d) a positive multiple of %d", M, N, K, BK);
+               "%s: M (%d) and N (%d) at least 64, K (%d) a positive multiple of %d", what, M, N, K, BK);
   IRON_REQUIRE((((uintptr_t)A | (uintptr_t)B | (uintptr_t)R | (uintptr_t)C) & 15) == 0,
-               "gemm_residual: operands must be 16-byte aligned");
+               "%s: operands must be 16-byte aligned", what);
   hipStream_t s = (hipStream_t)stream;
-  QkvTail tail{};
-  tail.residual = R;
-  tail.residual_scale = residual_scale;
   // The tile sizes of iron_gemm_bf16's (N,K) path below the 256-wide ones.
   const int tiles_n128 = (N + 127) / 128;
   const long tiles128 = (long)((M + 127) / 128) * tiles_n128;
@@ -1571,6 +1576,22 @@ extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, con
   const int few = tiles_n128 >= 128 ? 0 : 128 * (127 / tiles_n128);
   if (valid == nullptr || few == 0 || few >= M) return launch_gemm_nt<false>(A, B, C, M, N, K, valid, s, tail);
   return launch_gemm_either<false>(A, B, C, M, N, K, valid, s, 0, few, tail);
+}
+
+extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
+                                       int N, int K, float residual_scale, const int* valid, void* stream) {
+  QkvTail tail{};
+  tail.residual = R;
+  tail.residual_scale = residual_scale;
+  return gemm_with_tail("gemm_residual", A, B, R, C, M, N, K, tail, valid, stream);
+}
+
+extern "C" int iron_gemm_gated_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* G, uint16_t* C, int M,
+                                    int N, int K, const int* valid, void* stream) {
+  QkvTail tail{};
+  tail.residual = G;
+  tail.gated = 1;
+  return gemm_with_tail("gemm_gated", A, B, G, C, M, N, K, tail, valid, stream);
 }
 
 static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,

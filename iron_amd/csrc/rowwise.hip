@@ -140,7 +140,6 @@ __global__ __launch_bounds__(256) void rope_kernel(const bf16_t* __restrict__ x,
 // ------------------------------------------------------------ elementwise
 enum class Ew { kSilu, kMul, kAdd, kSiluMul };
 
-__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
 
 template <Ew OP>
 __device__ __forceinline__ float ew_apply(float a, float b) {

@@ -79,6 +79,16 @@ def gemm_residual(A, B, R, C, *, M, N, K, residual_scale=1.0, valid=None):
                                         ptr(_word(valid, "valid")), current_stream()), "iron_gemm_residual_bf16")
 
 
+def gemm_gated(A, B, G, C, *, M, N, K, valid=None):
+    """``C = SiLU(G) * (A @ B.T)`` over many rows, B stored ``(N, K)``."""
+    _numel(_dev(A, "A"), M * K, "A")
+    _numel(_dev(B, "B"), N * K, "B")
+    _numel(_dev(G, "G"), M * N, "G")
+    _numel(_dev(C, "C"), M * N, "C")
+    check(lib().iron_gemm_gated_bf16(ptr(A), ptr(B), ptr(G), ptr(C), M, N, K, ptr(_word(valid, "valid")),
+                                     current_stream()), "iron_gemm_gated_bf16")
+
+
 def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, residual_scale=1.0, epilogue=0):
     """One-row fusion: ``[RMSNorm ->] GEMV [-> + residual | gate/up -> SiLU -> Mul]``."""
     _numel(_dev(W, "W"), M * K, "W")
