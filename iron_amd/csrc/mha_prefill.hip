@@ -17,6 +17,15 @@
 
 namespace iron {
 
+// max(x, x of the lane 32 away) without a trip through LDS: the two halves of the wave swapped
+// between two copies (v_permlane32_swap), then one maximum.  The wait states a vector write needs
+// before the swap reads it are in the statement, since the compiler does not look inside it.
+__device__ __forceinline__ float max_with_other_half(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+
 constexpr int BQ = 128;   // query rows per block
 constexpr int BKV = 64;   // key rows per tile
 constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks split each block's tiles over two halves
@@ -145,20 +154,24 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
       k_voff[i] = r * row_bytes + (l_pch ^ ((r >> 1) & 7)) * 16;
       v_voff[i] = r * row_bytes + (l_pch ^ ((r & 3) << 1)) * 16;
     }
+    // The keys (and values) of the head that this block can see, from row kv_lo's start to the
+    // last key's row end, are one buffer for the whole loop; a tile's place in it goes into the
+    // lanes' offsets, the part of the address the bounds check sees.
+    const int reach = (kv_tokens - kv_lo - 1) * row_bytes + ROWB;
+    const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(Kh + (long)kv_lo * kv_row_stride), 0, reach, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(Vh + (long)kv_lo * kv_row_stride), 0, reach, 0x00020000);
+    const int tile_bytes = BKV * row_bytes;
     auto issue = [&](int tile, int buf) {
       char* st = smem + buf * STAGE;
-      const int first = kv_lo + tile * BKV;
-      const int reach = (min(BKV, kv_tokens - first) - 1) * row_bytes + ROWB;   // bytes up to the last key's row end
-      const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<bf16_t*>(Kh + (long)first * kv_row_stride), 0, reach, 0x00020000);
-      const __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<bf16_t*>(Vh + (long)first * kv_row_stride), 0, reach, 0x00020000);
+      const int at = tile * tile_bytes;
 #pragma unroll
       for (int i = 0; i < INST; ++i) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rows, IRON_LDS_PTR(st + (wave * INST + i) * 1024), 16,
-                                                 (int)k_voff[i], 0, 0, 0);
+                                                 (int)k_voff[i] + at, 0, 0, 0);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rows, IRON_LDS_PTR(st + TILE + (wave * INST + i) * 1024), 16,
-                                                 (int)v_voff[i], 0, 0, 0);
+                                                 (int)v_voff[i] + at, 0, 0, 0);
       }
     };
     // Always STAGES-1 tiles in flight before the loop and one more each iteration (past the end
@@ -180,6 +193,14 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
       v_frag[dt] = v_key * ROWB + ((chunk ^ v_swz) << 4) + ((lane & 1) << 3);
     }
     const unsigned lds_base = (unsigned)(size_t)IRON_LDS_PTR(smem);
+    // The keys this lane's query may see are one range of positions for the whole loop: key kpos
+    // is masked out iff (unsigned)(kpos - see_lo) > see_span (an empty range lets nothing pass).
+    int see_hi = kv_tokens - 1, see_lo = 0;
+    if (causal) see_hi = min(see_hi, qpos);
+    else if (window >= 0) see_hi = min(see_hi, qpos + window);
+    if (window >= 0) see_lo = max(0, qpos - window);
+    const unsigned see_span = see_hi >= see_lo ? (unsigned)(see_hi - see_lo) : 0u;
+    if (see_hi < see_lo) see_lo = 1 << 30;
 
     for (int step = 0; step < steps; ++step) {
       const int tile = step * SPLIT + half;
@@ -227,24 +248,19 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
         else if (window >= 0) edge |= kv0 + BKV - 1 > wq_lo + window;
         if (window >= 0) edge |= kv0 < wq_hi - window;
         if (edge) {
+          const int rel = kv0 + 4 * g - see_lo;
 #pragma unroll
           for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-              const int kpos = kv0 + 32 * t + 8 * (e >> 2) + 4 * g + (e & 3);
-              bool dead = kpos >= kv_tokens;
-              if (causal) dead |= kpos > qpos;
-              else if (window >= 0) dead |= kpos > qpos + window;
-              if (window >= 0) dead |= kpos < qpos - window;
-              sacc[t][e] = dead ? -INFINITY : sacc[t][e];
-            }
+            for (int e = 0; e < 16; ++e)
+              sacc[t][e] = (unsigned)(rel + 32 * t + 8 * (e >> 2) + (e & 3)) > see_span ? -INFINITY : sacc[t][e];
         }
         float rmax = sacc[0][0];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 32, 64));
+        rmax = max_with_other_half(rmax);
         const float m_new = fmaxf(m_run, rmax);
         const float mc = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
         const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc));  // exp2(-inf) = 0 at the start
@@ -409,6 +425,9 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
   const long kv_row = kv_interleaved ? (long)kv_heads * d : d;
   const long kv_head = kv_interleaved ? d : (long)kv_len * d;
   IRON_REQUIRE(kv_row <= (1L << 20), "mha_prefill: a key row spans %ld values, more than the 2^20 a tile's 32-bit offsets reach", kv_row);
+  IRON_REQUIRE((long)kv_len * kv_row * 2 < (1L << 31),
+               "mha_prefill: the keys of a head span %ld bytes, more than the 2^31 its loads' 32-bit offsets reach",
+               (long)kv_len * kv_row * 2);
   const float scale_log2 = scale * 1.4426950408889634f;
   if (d == 512) {
     IRON_REQUIRE(seq <= 65535, "mha_prefill: at d = 512 seq (%d) is a grid dimension, at most 65535", seq);
