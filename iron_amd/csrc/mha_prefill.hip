@@ -18,11 +18,12 @@
 namespace iron {
 
 // max(x, x of the lane 32 away) without a trip through LDS: the two halves of the wave swapped
-// between two copies (v_permlane32_swap), then one maximum.  The wait states a vector write needs
-// before the swap reads it are in the statement, since the compiler does not look inside it.
+// between two copies (v_permlane32_swap), then one maximum.  The wait states between a vector
+// write and the swap that reads it, and between the swap and what reads its results, are in the
+// statement, since the compiler does not look inside it.
 __device__ __forceinline__ float max_with_other_half(float x) {
   float a = x, b = x;
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
   return fmaxf(a, b);
 }
 
