@@ -40,6 +40,18 @@ def test_argument_refusals_need_no_gpu():
     assert b"multiple of kv_heads" in lib.iron_last_error()
 
 
+def test_every_entry_point_refuses_null_operands():
+    """Each entry point that takes pointers returns 1 with a reason, before any launch, when they
+    are all null and every size is zero: nothing is dereferenced or launched on bad arguments."""
+    lib = _lib.lib()
+    for name, (_, args) in sorted(_lib.SIGNATURES.items()):
+        if not any(a is _lib._P for a in args):
+            continue
+        call = [None if a is _lib._P else (0.0 if a is ctypes.c_float else 0) for a in args]
+        assert getattr(lib, name)(*call) == 1, name
+        assert lib.iron_last_error(), name
+
+
 def test_bench_refuses_more_than_one_gpu():
     """``bench.py --gpus N`` with N above 1 exits with a message: this build is the one-GPU path."""
     import subprocess
