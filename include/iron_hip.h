@@ -56,13 +56,13 @@ int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16_t* y, int 
 int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
                             int N, int K, float residual_scale, const int* valid, void* stream);
 
-/* C = bf16(bf16(SiLU(G)) * bf16(A B^T)) for the rows under *valid (or M): a gated feed-forward's second
- * projection with the activated gate in its epilogue.  A (M,K), B (N,K), G and C (M,N); K % 64 == 0,
- * M, N >= 64.  C may be G.
- * Replaces GEMM (up_proj), SiLU (of gate_proj's product G) and ElementwiseMul
- * (iron/lm/blocks.py:697-699), rounding where they round. */
+/* C = bf16(bf16(act(G)) * bf16(A B^T)) for the rows under *valid (or M): a gated feed-forward's second
+ * projection with the activated gate in its epilogue; activation 1: SiLU, 2: GELU by its tanh form.
+ * A (M,K), B (N,K), G and C (M,N); K % 64 == 0, M, N >= 64.  C may be G.
+ * Replaces GEMM (up_proj), SiLU or GELU (of gate_proj's product G) and ElementwiseMul
+ * (iron/lm/blocks.py:688,697-699), rounding where they round. */
 int iron_gemm_gated_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* G, uint16_t* C, int M,
-                         int N, int K, const int* valid, void* stream);
+                         int N, int K, int activation, const int* valid, void* stream);
 
 /* One-row fusions of a decoder layer (no single counterpart in the reference: each replaces a run
  * of its steps, iron/lm/blocks.py:627-648,697-699,723-733, and rounds where those steps round).

@@ -16,7 +16,7 @@ in a prompt chunk's version (several rows, 64-wide heads),
 
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
   ... and Copy k/v -> the chunk's cache rows             => iron_prefill_qkv_cache_bf16
-  GEMM (up), SiLU (of the gate), ElementwiseMul          => iron_gemm_gated_bf16
+  GEMM (up), SiLU or GELU (tanh) of the gate, Mul        => iron_gemm_gated_bf16
   SiLU, ElementwiseMul (no such product before them)     => iron_silu_mul_bf16
   GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
 
@@ -259,7 +259,9 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), R=tensor(other), C=tensor(ad.outputs["y"]))
                 kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, residual_scale=scale, valid=word(gv))
                 got = Fused("gemm_add", i, 2, lambda a=args, kw=kw: kernels.gemm_residual(**a, **kw))
-        elif (_name(s) == "GEMM" and i + 2 < len(steps) and _name(steps[i + 1]) == "SiLU"
+        elif (_name(s) == "GEMM" and i + 2 < len(steps)
+              and (_name(steps[i + 1]) == "SiLU"
+                   or (_name(steps[i + 1]) == "GELU" and steps[i + 1].op.approximate == "tanh"))
               and _name(steps[i + 2]) == "ElementwiseMul"
               and s.op.b_col_maj and not s.op.c_col_maj and "valid_k" not in s.values
               and s.op.M >= 64 and s.op.N >= 64 and s.op.K % 64 == 0):
@@ -280,7 +282,8 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                     and ml.outputs["y"].elements == up.elements
                     and set(sl.values) <= {"valid"} and set(ml.values) <= {"valid"}):
                 args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), G=tensor(gate), C=tensor(ml.outputs["y"]))
-                kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, valid=word(gv))
+                kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, valid=word(gv),
+                          activation="silu" if _name(sl) == "SiLU" else "gelu_tanh")
                 got = Fused("gemm_gated", i, 3, lambda a=args, kw=kw: kernels.gemm_gated(**a, **kw))
         elif _name(s) == "SiLU" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseMul":
             # a gated feed-forward's activation and gate over many rows: one pass instead of two

@@ -10,10 +10,7 @@ namespace iron {
 // ------------------------------------------------------------------ unary
 template <int KIND>
 __device__ __forceinline__ float unary_apply(float v, float p0, float p1) {
-  if (KIND == IRON_UNARY_GELU_TANH) {
-    const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-    return 0.5f * v * (1.0f + tanhf(inner));
-  }
+  if (KIND == IRON_UNARY_GELU_TANH) return gelu_tanh_f32(v);
   if (KIND == IRON_UNARY_GELU_ERF) return 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
   if (KIND == IRON_UNARY_RELU) return v > 0.f ? v : 0.f;
   if (KIND == IRON_UNARY_SIGMOID) return 1.0f / (1.0f + __expf(-v));

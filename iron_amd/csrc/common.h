@@ -71,8 +71,13 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
   return v;
 }
 
-// SiLU as every kernel here computes it, so that fused and separate launches round alike.
+// SiLU, and GELU by its tanh form, as every kernel here computes them, so that fused and separate
+// launches round alike.
 __device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
+__device__ __forceinline__ float gelu_tanh_f32(float v) {
+  const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+  return 0.5f * v * (1.0f + tanhf(inner));
+}
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // 16-byte streaming load that does not displace reusable lines in the caches.

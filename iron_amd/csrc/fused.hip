@@ -11,12 +11,6 @@
 
 namespace iron {
 
-__device__ __forceinline__ float silu_ref(float v) { return v / (1.0f + __expf(-v)); }
-// GELU by its tanh form, as the catalog's unary kernel computes it.
-__device__ __forceinline__ float gelu_tanh_ref(float v) {
-  const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-  return 0.5f * v * (1.0f + tanhf(inner));
-}
 
 // All fused kernels share one shape: a block of 4 waves owns a few rows and its 256 threads
 // split K in 16-byte chunks (thread t takes chunks t, t+256, ...), so the weight loads of a row
@@ -142,7 +136,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
       if (EPI == EPI_SILU_MUL || EPI == EPI_GELU_MUL) {
         const float u = round_bf16(part[0][MATS - 1][r] + part[1][MATS - 1][r] + part[2][MATS - 1][r] +
                                    part[3][MATS - 1][r]);
-        v = round_bf16(EPI == EPI_SILU_MUL ? silu_ref(v) : gelu_tanh_ref(v)) * u;
+        v = round_bf16(EPI == EPI_SILU_MUL ? silu_f32(v) : gelu_tanh_f32(v)) * u;
       }
       y[row] = f32_to_bf16(v);
     }

@@ -302,14 +302,17 @@ struct QkvTail {
   // (one fused multiply-add; residual (M, N) like C), when residual is not NULL.
   const bf16_t* residual;
   float residual_scale;
-  // ... or, with gated set, C = bf16(bf16(SiLU(residual)) * bf16(A B)): `residual` then holds a gated
-  // feed-forward's other product, and this one leaves as the activated gate times it.
+  // ... or, with gated set, C = bf16(bf16(act(residual)) * bf16(A B)): `residual` then holds a gated
+  // feed-forward's other product, and this one leaves as the activated gate times it (1: SiLU,
+  // 2: GELU by its tanh form).
   int gated;
   // Of the fused projections again: Ck and Cv are KV caches of kv_rows rows (a row kv_n wide, as the
   // projections write one), and the chunk's rows go to rows *kv_row0 on, when kv_row0 is not NULL.
   const int* kv_row0;
   int kv_rows;
 };
+
+__device__ __forceinline__ float gate_of(int kind, float g) { return kind == 2 ? gelu_tanh_f32(g) : silu_f32(g); }
 
 // The k and v outputs moved to the chunk's rows of their caches.  The first row is held where the
 // rows under the bound still end inside the cache, whatever the word holds.
@@ -497,7 +500,7 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float prod = round_bf16(acc[0][4 * q + e]);
-        acc[0][4 * q + e] = qkv.gated ? round_bf16(silu_f32(rf[e])) * prod : fmaf(qkv.residual_scale, prod, rf[e]);
+        acc[0][4 * q + e] = qkv.gated ? round_bf16(gate_of(qkv.gated, rf[e])) * prod : fmaf(qkv.residual_scale, prod, rf[e]);
       }
     }
     if (vec && n + 4 <= N) {
@@ -768,7 +771,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          x[e] = qkv.gated ? round_bf16(silu_f32(rf[e])) * x[e] : fmaf(qkv.residual_scale, x[e], rf[e]);
+          x[e] = qkv.gated ? round_bf16(gate_of(qkv.gated, rf[e])) * x[e] : fmaf(qkv.residual_scale, x[e], rf[e]);
         v = pack8(x);
       }
     }
@@ -1587,10 +1590,12 @@ extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, con
 }
 
 extern "C" int iron_gemm_gated_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* G, uint16_t* C, int M,
-                                    int N, int K, const int* valid, void* stream) {
+                                    int N, int K, int activation, const int* valid, void* stream) {
+  IRON_REQUIRE(activation == 1 || activation == 2, "gemm_gated: activation (%d) is 1 (SiLU) or 2 (GELU, tanh form)",
+               activation);
   QkvTail tail{};
   tail.residual = G;
-  tail.gated = 1;
+  tail.gated = activation;
   return gemm_with_tail("gemm_gated", A, B, G, C, M, N, K, tail, valid, stream);
 }
 

@@ -79,14 +79,18 @@ def gemm_residual(A, B, R, C, *, M, N, K, residual_scale=1.0, valid=None):
                                         ptr(_word(valid, "valid")), current_stream()), "iron_gemm_residual_bf16")
 
 
-def gemm_gated(A, B, G, C, *, M, N, K, valid=None):
-    """``C = SiLU(G) * (A @ B.T)`` over many rows, B stored ``(N, K)``."""
+def gemm_gated(A, B, G, C, *, M, N, K, activation="silu", valid=None):
+    """``C = act(G) * (A @ B.T)`` over many rows, B stored ``(N, K)``; ``activation`` "silu" or
+    "gelu_tanh"."""
+    kinds = {"silu": 1, "gelu_tanh": 2}
+    if activation not in kinds:
+        raise ValueError(f"gemm_gated: activation {activation!r} is neither 'silu' nor 'gelu_tanh'")
     _numel(_dev(A, "A"), M * K, "A")
     _numel(_dev(B, "B"), N * K, "B")
     _numel(_dev(G, "G"), M * N, "G")
     _numel(_dev(C, "C"), M * N, "C")
-    check(lib().iron_gemm_gated_bf16(ptr(A), ptr(B), ptr(G), ptr(C), M, N, K, ptr(_word(valid, "valid")),
-                                     current_stream()), "iron_gemm_gated_bf16")
+    check(lib().iron_gemm_gated_bf16(ptr(A), ptr(B), ptr(G), ptr(C), M, N, K, kinds[activation],
+                                     ptr(_word(valid, "valid")), current_stream()), "iron_gemm_gated_bf16")
 
 
 def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, residual_scale=1.0, epilogue=0):

@@ -328,15 +328,17 @@ def test_gemm_residual_epilogue(cuda, M, Kdim, N, rows, scale):
     close(from_torch(Rd)[:lim], want[:lim], rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("M,Kdim,N,rows", [(2048, 2048, 8192, 512), (2048, 256, 8192, None), (2048, 256, 2048, 1500),
-                                           (256, 128, 512, 100), (128, 64, 64, None), (4096, 192, 1024, 3000),
-                                           (200, 128, 136, None)])
-def test_gemm_gated_epilogue(cuda, M, Kdim, N, rows):
-    """A gated feed-forward's second projection over many rows with the activated gate in its
-    epilogue.  The chain rounds twice (the product, then the gated product), so it is checked link
-    by link: the product of the separate launch against the oracle's GEMM, the fused launch against
-    the oracle's SiLU and ElementwiseMul of that product, and bit for bit against this library's
-    own separate launches.  The first case is Llama-3.2-1B's prompt chunk."""
+@pytest.mark.parametrize("M,Kdim,N,rows,activation", [
+    (2048, 2048, 8192, 512, "silu"), (2048, 256, 8192, None, "silu"), (2048, 256, 2048, 1500, "silu"),
+    (256, 128, 512, 100, "silu"), (128, 64, 64, None, "silu"), (4096, 192, 1024, 3000, "silu"), (200, 128, 136, None, "silu"),
+    (2048, 256, 8192, 512, "gelu_tanh"), (256, 128, 512, 100, "gelu_tanh"), (200, 128, 136, None, "gelu_tanh")])
+def test_gemm_gated_epilogue(cuda, M, Kdim, N, rows, activation):
+    """A gated feed-forward's second projection over many rows with the activated gate (SiLU, or
+    GELU by its tanh form) in its epilogue.  The chain rounds twice (the product, then the gated
+    product), so it is checked link by link: the product of the separate launch against the oracle's
+    GEMM, the fused launch against the oracle's activation and ElementwiseMul of that product, and
+    bit for bit against this library's own separate launches.  The first case is Llama-3.2-1B's
+    prompt chunk."""
     rng = np.random.default_rng(M + N + 1)
     A, B, G = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.05), bf(rng, M, N, scale=2.0)
     lim = M if rows is None else rows
@@ -344,21 +346,28 @@ def test_gemm_gated_epilogue(cuda, M, Kdim, N, rows):
     if rows is not None:
         A[rows:] = np.nan
     bound = None if rows is None else word(rows, cuda)
-    # the separate launches: the product, then SiLU and the multiplication in one pass
+    flat_bound = None if rows is None else word(rows * N, cuda)
+    # the separate launches: the product, then the activation and the multiplication
     U, Y = out_like((M, N), cuda, fill=7.0), out_like((M, N), cuda, fill=7.0)
     K.gemm(dev(A, cuda), dev(B, cuda), U, M=M, N=N, K=Kdim, b_col_maj=True, valid=bound)
-    K.silu_mul(dev(G, cuda).reshape(-1), U.reshape(-1), Y.reshape(-1), n=M * N,
-               valid=None if rows is None else word(rows * N, cuda))
+    if activation == "silu":
+        K.silu_mul(dev(G, cuda).reshape(-1), U.reshape(-1), Y.reshape(-1), n=M * N, valid=flat_bound)
+        activated = ops.silu(G[:lim])
+    else:
+        act = out_like((M, N), cuda, fill=7.0)
+        K.unary(dev(G, cuda).reshape(-1), act.reshape(-1), "gelu_tanh", n=M * N, valid=flat_bound)
+        K.mul(act.reshape(-1), U.reshape(-1), Y.reshape(-1), n=M * N, valid=flat_bound)
+        activated = ops.gelu(G[:lim], approximate="tanh")
     close(U[:lim], product, rtol=1e-2, atol=1e-2)
     C = out_like((M, N), cuda, fill=7.0)
-    K.gemm_gated(dev(A, cuda), dev(B, cuda), dev(G, cuda), C, M=M, N=N, K=Kdim, valid=bound)
+    K.gemm_gated(dev(A, cuda), dev(B, cuda), dev(G, cuda), C, M=M, N=N, K=Kdim, activation=activation, valid=bound)
     got = from_torch(C)
-    close(got[:lim], ops.mul(ops.silu(G[:lim]), from_torch(U)[:lim]), rtol=1e-2, atol=1e-2)
+    close(got[:lim], ops.mul(activated, from_torch(U)[:lim]), rtol=1e-2, atol=1e-2)
     assert np.all(got[lim:] == 7.0)
     assert torch.equal(Y[:lim], C[:lim])
     # in place: the gate's product is its own output
     Gd = dev(G, cuda)
-    K.gemm_gated(dev(np.nan_to_num(A), cuda), dev(B, cuda), Gd, Gd, M=M, N=N, K=Kdim, valid=bound)
+    K.gemm_gated(dev(np.nan_to_num(A), cuda), dev(B, cuda), Gd, Gd, M=M, N=N, K=Kdim, activation=activation, valid=bound)
     assert torch.equal(Gd[:lim], C[:lim])
 
 
