@@ -27,8 +27,9 @@ __device__ __forceinline__ float max_with_other_half(float x) {
   return fmaxf(a, b);
 }
 
-constexpr int BQ = 128;   // query rows per block
+constexpr int BQ = 128;   // query rows per block (four waves of 32; 64 where a block is two)
 constexpr int BKV = 64;   // key rows per tile
+constexpr int kFewBlocks = 256;          // launches of fewer blocks than this halve their blocks' queries
 constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks split each block's tiles over two halves
 
 // K and V tiles go straight from global memory into LDS (buffer loads with the LDS bit, no register staging), as
@@ -45,8 +46,11 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 // the odd key tiles (their own loads, their own stage buffers), and the two halves' (max, sum, O)
 // are merged through LDS at the end.  A query block's chain of tiles is half as long, which is what
 // bounds a short sequence: its blocks are few and the one that sees every key finishes last.
-template <int D, int SPLIT>
-__global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1))) void mha_prefill_kernel(
+//
+// W: the waves that share a tile's loads, each with 32 of the block's 32 W queries.  Four; two
+// where four would leave CUs without a block (a short prompt), so that twice as many blocks go out.
+template <int D, int SPLIT, int W = 4>
+__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(D <= 128 && W == 4 ? 2 : 1))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -59,7 +63,8 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   constexpr int STAGES = D == 64 ? 3 : 2;
   constexpr int TILE = BKV * ROWB;       // bytes of a K (or V) tile
   constexpr int STAGE = 2 * TILE;
-  constexpr int INST = TILE / 1024 / 4;  // 1 KB loads of K (and of V) a wave issues per tile
+  constexpr int BQW = 32 * W;            // query rows of this block
+  constexpr int INST = TILE / 1024 / W;  // 1 KB loads of K (and of V) a wave issues per tile
   constexpr int RPI = 1024 / ROWB;       // rows one load covers
   extern __shared__ __align__(1024) char smem_all[];   // SPLIT * STAGES * STAGE bytes
 
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   // Which tiles, and which 32 queries -- uniform over the wave, so what depends on them (LDS
   // destinations, the rows a wave loads) stays in scalar registers.
   const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int half = wave_id >> 2, wave = wave_id & 3;
+  const int half = wave_id / W, wave = wave_id % W;
   char* smem = smem_all + half * (STAGES * STAGE);            // this half's stage buffers
   const int col = lane & 31, g = lane >> 5;
   // Blocks are dispatched in id order, so the id runs over the query blocks from the last (under a
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   const int head = (heads % 8 == 0) ? (j % 8) * (heads / 8) + j / 8 : j;
   const int kvh = head / group;
   const int qb = (int)(gridDim.x / heads) - 1 - (int)(blockIdx.x / heads);
-  const int q0 = qb * BQ;
+  const int q0 = qb * BQW;
 
   const int q_tokens = valid ? bound_or(valid, seq) : seq_len;
   const int kv_tokens = kv_valid ? bound_or(kv_valid, kv_len) : (kv_len - seq + q_tokens);
@@ -95,7 +100,7 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   bf16_t* Oh = O + (size_t)head * q_head_stride;
   // Rows of this block past the bound: zeros.  A block wholly past it does only that.
   if (q0 >= q_tokens || offset < 0) {
-    for (int i = tid; i < BQ * CPR; i += 256 * SPLIT) {
+    for (int i = tid; i < BQW * CPR; i += 64 * W * SPLIT) {
       const int r = q0 + i / CPR, c = (i % CPR) * 8;
       if (r < seq) *reinterpret_cast<uint4*>(Oh + (size_t)r * q_row_stride + c) = make_uint4(0, 0, 0, 0);
     }
@@ -122,7 +127,7 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
   float m_run = -INFINITY, l_run = 0.f;   // the running max is of the raw (unscaled) scores
 
   // Keys this block's live queries can see.
-  const int q_last = min(q0 + BQ, q_tokens) - 1;
+  const int q_last = min(q0 + BQW, q_tokens) - 1;
   int kv_hi = kv_tokens;
   if (causal) kv_hi = min(kv_hi, offset + q_last + 1);
   else if (window >= 0) kv_hi = min(kv_hi, offset + q_last + window + 1);
@@ -339,7 +344,7 @@ __global__ __launch_bounds__(256 * SPLIT) __attribute__((amdgpu_waves_per_eu(D <
     // The odd tiles' half hands its (max, sum, O) over through LDS, a value a lane a row (no bank
     // conflicts); the even tiles' half folds it in by the usual rule and stores.
     constexpr int FIELDS = 2 + 16 * DT;
-    static_assert(4 * FIELDS * 64 * 4 <= SPLIT * STAGES * STAGE, "the hand-over fits the stage buffers");
+    static_assert(W * FIELDS * 64 * 4 <= SPLIT * STAGES * STAGE, "the hand-over fits the stage buffers");
     float* hand = reinterpret_cast<float*>(smem_all) + wave * FIELDS * 64 + lane;
     block_barrier();   // every wave is out of the tile loop: the stage buffers are free
     if (half == 1) {
@@ -394,18 +399,18 @@ struct PrefillArgs {
 };
 
 // The stage buffers are dynamic LDS (more than the 64 KB a kernel may declare statically).
-template <int D, int SPLIT>
+template <int D, int SPLIT, int W = 4>
 static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
   constexpr int STAGES = D == 64 ? 3 : 2;
   constexpr size_t lds = (size_t)SPLIT * STAGES * 2 * BKV * D * 2;
   static bool once = false;
   if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT, W>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("mha_prefill: %s", hipGetErrorString(e)); return (int)e; }
     once = true;
   }
-  hipLaunchKernelGGL((mha_prefill_kernel<D, SPLIT>), dim3(blocks), dim3(256 * SPLIT), lds, (hipStream_t)stream, a.Q,
+  hipLaunchKernelGGL((mha_prefill_kernel<D, SPLIT, W>), dim3(blocks), dim3(64 * W * SPLIT), lds, (hipStream_t)stream, a.Q,
                      a.K, a.V, a.O, a.heads, a.group, a.seq, a.seq_len, a.kv_len, a.scale_log2, a.causal, a.window,
                      a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid, a.kv_first, a.kv_rows);
   return 0;
@@ -463,7 +468,9 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
   PrefillArgs a{Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window,
                 q_row, q_head, kv_row, kv_head, valid, kv_valid, kv_first, kv_rows};
   int rc;
-  if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
+  // Fewer blocks of 128 queries than CUs (a short prompt): blocks of 64, two waves a part.
+  if (d == 64 && blocks < kFewBlocks) rc = launch_prefill<64, 2, 2>(a, ((seq + 63) / 64) * heads, stream);
+  else if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
   else if (d == 128) rc = split ? launch_prefill<128, 2>(a, blocks, stream) : launch_prefill<128, 1>(a, blocks, stream);
   else rc = launch_prefill<256, 1>(a, blocks, stream);
   if (rc != 0) return rc;
