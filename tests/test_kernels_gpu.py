@@ -629,6 +629,29 @@ def test_mha_prefill_longest_shape_on_sampled_queries(cuda):
         close(got[r : r + 1], want)
 
 
+@pytest.mark.parametrize("rows", [512, 1500])
+def test_mha_prefill_bounded_chunk_at_the_decoder_s_width(cuda, rows):
+    """A 2048-row prompt chunk of 32 heads under row and key bounds read on the device (512 rows
+    as the benchmark's prompt leaves, and 1500): every head of a sample of rows against the oracle's
+    one-query attention over the keys before it; the rows past the bound are zero, and NaN there
+    reaches nothing."""
+    rng = np.random.default_rng(rows)
+    S, H, G, d = 2048, 32, 8, 64
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    Q[rows:], Kc[rows:], Vc[rows:] = np.nan, np.nan, np.nan
+    O = out_like(Q.shape, cuda, fill=float("nan"))
+    K.mha_prefill(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, seq=S, seq_len=S,
+                  kv_len=S, scale=0.125, causal=True, q_interleaved=True, kv_interleaved=True,
+                  valid=word(rows, cuda), kv_valid=word(rows, cuda))
+    got = from_torch(O)
+    assert np.all(got[rows:] == 0)
+    assert not np.isnan(got[:rows]).any()
+    for r in sorted({0, 1, 31, 32, 63, 64, 65, 127, 128, 129, rows - 65, rows - 64, rows - 1, *rng.integers(0, rows, 10).tolist()}):
+        want = ops.mha(Q[r : r + 1], Kc[: r + 1], Vc[: r + 1], num_heads=H, num_KV_heads=G, seq_len=1, kv_len=r + 1,
+                       d=d, causal=True, scale=0.125, heads_interleaved=True, kv_interleaved=True)
+        close(got[r : r + 1], want)
+
+
 @pytest.mark.parametrize("S", [512, 2048])
 def test_mha_prefill_llama_shape(cuda, S):
     rng = np.random.default_rng(11)
