@@ -585,6 +585,30 @@ def counter_probe(torch, K, dev, rng):
                       "attention_prefill": [{"S": 2048, "launches": 2}, {"S": 8192, "launches": 2}]}))
 
 
+def attention_probe(torch, K, dev):
+    """One query over caches of 1024, 4096 and 16384 keys (32 q / 8 kv heads, d 64), 4 launches each over
+    distinct caches, then a plain copy of known size: what a counter or kernel-trace run of decode
+    attention alone needs."""
+    H, G, D = 32, 8, 64
+    ws = K.mha_decode_workspace(H, D, dev)
+    shapes = []
+    for L in (1024, 4096, 16384):
+        Q = torch.randn((1, H, D), device=dev).to(torch.bfloat16)
+        O = torch.empty_like(Q)
+        for _ in range(4):
+            Kc, Vc = (torch.randn((L, G, D), device=dev).to(torch.bfloat16) for _ in range(2))
+            K.mha_decode(Q, Kc, Vc, O, heads=H, kv_heads=G, d=D, kv_len=L, scale=0.125, kv_interleaved=True, workspace=ws)
+        shapes.append({"L": L, "launches": 4, "algorithmic_bytes": 2 * L * G * D * 2 + 2 * H * D * 2})
+    rows = PROBE_COPY_BYTES // 4096
+    src = torch.zeros(PROBE_COPY_BYTES // 4, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        K.copy_rows(src, dst, rows=rows, row_elems=1024, src_rows=rows, dst_rows=rows)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "attention", "decode": shapes,
+                      "copy": {"launches": 2, "bytes_read": PROBE_COPY_BYTES, "bytes_written": PROBE_COPY_BYTES}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -600,6 +624,9 @@ def main():
                     help="prefill the 512-token prompt once, replay N decode steps and exit (for a rocprofv3 --kernel-trace or --pmc run)")
     ap.add_argument("--prompt-probe", action="store_true",
                     help="run only the decoder's 512-token prompt chunk, 20 times (for a rocprofv3 --kernel-trace run) and exit")
+    ap.add_argument("--attention-probe", action="store_true",
+                    help="launch only decode attention at 1024 / 4096 / 16384 keys and a plain copy of known size "
+                         "(for a rocprofv3 --pmc or --kernel-trace run) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is a one-GPU hot path; --gpus must be 1 "
@@ -632,6 +659,9 @@ def main():
         return 0
     if args.prompt_probe:
         prompt_probe(torch, dev)
+        return 0
+    if args.attention_probe:
+        attention_probe(torch, K, dev)
         return 0
     if args.decode_probe:
         bench_decoder(torch, dev, args.steps, args.warmup, False, probe_steps=args.decode_probe)

@@ -218,12 +218,24 @@ int iron_mha_prefill_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_
 /* Attention, one query (decode; the reference's "packed" MHA, seq_len == 1).
  * Q,O: (heads, d).  K,V as above.  kv_tokens = *kv_valid (or kv_len); the query sits at
  * kv_tokens - 1.  workspace: iron_mha_decode_workspace_bytes(heads, d) bytes of device memory.
- * d in {64, 128, 256} with 1, 2, 3, 4, 5, 6 or 8 query heads a KV head, or d = 512 with any.
+ * d in {64, 128} with up to 16 query heads a KV head, d = 256 with 1, 2, 3, 4, 5, 6 or 8, or d = 512
+ * with any.  The launches depend on (heads, kv_heads, d) and on whether kv_len can pass 1024 rows;
+ * what they read, and how the keys are dealt over the chip, follow *kv_valid (a cache's length only
+ * sizes the buffers: the reference's "attention over a cache costs the context, not the cache",
+ * iron/operators/mha.py:275-278).
  * Replaces the packed single-query MHA: iron/operators/mha.py:476-477,1073-1116. */
 int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
                          int heads, int kv_heads, int d, int kv_len, float scale, int window,
                          int kv_interleaved, const int* kv_valid, void* workspace, void* stream);
 int64_t iron_mha_decode_workspace_bytes(int heads, int d);
+/* The same with the kernel form forced, for tests and measurements (as iron_gemv_bf16_tuned):
+ * form 0 the default choice, 1 the lane-per-column scans, 2 the matrix-core scan (d = 64 or 128);
+ * short_keys > 0: the live-key count up to which the matrix-core scan's one block a KV head writes
+ * the output itself (beyond it the keys are dealt over every CU and a second launch merges). */
+int iron_mha_decode_tuned_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
+                               int heads, int kv_heads, int d, int kv_len, float scale, int window,
+                               int kv_interleaved, const int* kv_valid, void* workspace, int form,
+                               int short_keys, void* stream);
 /* iron_mha_decode_bf16 for callers that cannot allocate (code under HIP-graph capture, tight
  * serving loops, harnesses that forbid hipMalloc): the same kernels, their split-KV partial results
  * in a scratch array the library holds in device memory itself (iron_mha_decode_static_max_bytes()

@@ -49,6 +49,10 @@ SIGNATURES = {
         [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, _P, _P],
     ),
     "iron_mha_decode_workspace_bytes": (c_int64, [c_int, c_int]),
+    "iron_mha_decode_tuned_bf16": (
+        c_int,
+        [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, _P, c_int, c_int, _P],
+    ),
     "iron_mha_decode_static_bf16": (
         c_int,
         [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, _P],

@@ -243,6 +243,10 @@ class Built:
 
     kernel: str
     launch: Callable[[Mapping[str, Any], Mapping[str, Any]], None]
+    # ``(per-call value, limit)``: while that value stays within the limit, ``launch`` has a cheaper
+    # form, which it takes when ``words["__context__"]["bounded"]`` is true.  The caller vouches for
+    # the limit only as far as speed goes: the bounded form is correct for any value.
+    bounded: tuple[str, int] | None = None
 
 
 class Operator:

@@ -1150,6 +1150,11 @@ class CompiledGraph:
         arena.reserve_transients(pool.size)
         self._loaded_generation = None
         self._graph = None
+        self._graph_bounded = None
+        # What a step's launch may read of the call's context: ``bounded`` while every step that has a
+        # cheaper form within a limit (``Built.bounded``) is being launched, or captured, in that form.
+        self._context: dict[str, Any] = {"bounded": False}
+        self._bounds: list[tuple[Affine, int]] = []   # (per-call expression, limit) of those steps
         self._launches: list = []
 
     def _slot(self, expr: Affine) -> int:
@@ -1228,6 +1233,7 @@ class CompiledGraph:
         # ... and where the draw is the captured step's last launch and nothing else is carried from a
         # buffer, it evaluates the tail's expressions too: the step ends without a launch for them.
         self._tail_in_draw = bool(self.capture and self._carry_by_draw and self.n_tail and not self.carry_copies)
+        self._bounds = []
         self._launches = [self._bind(step) for step in self.recording.steps]
         self._fused = {}
         if self.fuse:
@@ -1237,7 +1243,7 @@ class CompiledGraph:
         self.input_tensors = [self._tensor(h) for h in self.recording.inputs]
         self.output_tensors = [self._tensor(h) for h in self.recording.outputs]
         self._loaded_generation = self.arena.generation
-        self._graph = None
+        self._graph = self._graph_bounded = None
         if self.capture:
             self._capture()
         return self
@@ -1256,6 +1262,9 @@ class CompiledGraph:
                 )
         if views:
             words = {**words, "__views__": views}
+        if built.bounded is not None and built.bounded[0] in step.values:
+            self._bounds.append((step.values[built.bounded[0]], int(built.bounded[1])))
+            words = {**words, "__context__": self._context}
         slot = self._carry_by_draw.get(self.recording.steps.index(step)) if self._carry_by_draw else None
         if slot is not None:
             words = {**words, "__carry_token__": self.words[slot : slot + 1]}
@@ -1320,19 +1329,26 @@ class CompiledGraph:
         self._write_words(self.recording.check_values(safe))
         stream = torch.cuda.Stream()
         stream.wait_stream(torch.cuda.current_stream())
+        graphs = {}
         with torch.cuda.stream(stream):
-            self._derive()
-            self._run_steps()
-            stream.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                # The host wrote every word, derived ones included, before the first replay; each
-                # replay re-derives them for the next as it carries.
+            # Steps with a cheaper form within a limit are captured both ways; a call or a replay
+            # takes the bounded graph while the values the host follows stay within every limit.
+            for bounded in ((False, True) if self._bounds else (False,)):
+                self._context["bounded"] = bounded
+                self._derive()
                 self._run_steps()
-                self._carry_on_device()
-            stream.synchronize()
+                stream.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    # The host wrote every word, derived ones included, before the first replay; each
+                    # replay re-derives them for the next as it carries.
+                    self._run_steps()
+                    self._carry_on_device()
+                stream.synchronize()
+                graphs[bounded] = graph
+            self._context["bounded"] = False
         torch.cuda.current_stream().wait_stream(stream)
-        self._graph = graph
+        self._graph, self._graph_bounded = graphs[False], graphs.get(True)
         self._host_values = None   # the warm-up's values start no run of replays
 
     # -- calling -------------------------------------------------------------
@@ -1353,6 +1369,19 @@ class CompiledGraph:
         self.words.copy_(self.host_words, non_blocking=True)
         self._words_copied = torch.cuda.Event()
         self._words_copied.record()
+
+    def _within_bounds(self, values: Mapping[str, int]) -> bool:
+        """Whether every step with a bounded form stays within its limit at these per-call values."""
+        at = {**values, "__const__": 0}
+        return all(expr.evaluate(at) <= limit for expr, limit in self._bounds)
+
+    def _replay_at(self, values: Mapping[str, int]) -> None:
+        """One replay of the captured step from ``values`` (already on the device): the bounded
+        graph where one was captured and the values allow it."""
+        if self._graph_bounded is not None and self._within_bounds(values):
+            self._graph_bounded.replay()
+        else:
+            self._graph.replay()
 
     def _after(self, values: Mapping[str, int], steps: int) -> dict[str, int]:
         """The per-call values ``steps`` runs after ``values``, as far as the host can follow them:
@@ -1429,7 +1458,7 @@ class CompiledGraph:
             dst.copy_(src.reshape(dst.shape), non_blocking=True)
         self._write_words(full)
         if self._graph is not None:
-            self._graph.replay()
+            self._replay_at(full)
         else:
             if self.check:
                 self._run_checked(full)
@@ -1467,7 +1496,7 @@ class CompiledGraph:
         self._write_words(full)
         if self._graph is None:
             raise RuntimeError(f"{rec.name}: this version is not captured in a HIP graph")
-        self._graph.replay()
+        self._replay_at(full)
 
     def replay(self, n: int = 1) -> None:
         """Replay the captured step ``n`` more times, each starting from the values the last one carried."""
@@ -1488,8 +1517,14 @@ class CompiledGraph:
             self.recording.check_values(last)
         except IndexError as e:
             raise IndexError(f"{e}; {n} replay(s) from {known} leave the limits") from None
-        for _ in range(n):
-            self._graph.replay()
+        if self._graph_bounded is None:
+            for _ in range(n):
+                self._graph.replay()
+        else:
+            at = known
+            for _ in range(n):
+                at = self._after(at, 1)
+                self._replay_at(at)
         self._host_values = last
 
     def _run_checked(self, full) -> None:
@@ -1519,7 +1554,7 @@ class CompiledGraph:
                 raise AssertionError(f"{self.recording.name}: step {op.name}: {bad}")
 
     def release(self) -> None:
-        self._graph = None
+        self._graph = self._graph_bounded = None
         self._launches = []
         self._loaded_generation = None
 

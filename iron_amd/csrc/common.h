@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #define IRON_OK 0
 #define IRON_EINVAL 1
 
@@ -31,6 +33,23 @@ void set_error(const char* fmt, ...);
     }                                                \
     return IRON_OK;                                  \
   } while (0)
+
+// A kernel's opt-in to more dynamic LDS than a launch gets by default.  The attribute belongs to a
+// device's copy of the function, so it is set once per device (that device current), from whichever
+// host thread gets there first; two that race both set it, which is harmless.
+struct LdsOptIn {
+  std::atomic<uint64_t> done{0};
+  hipError_t ensure(const void* kernel, size_t bytes) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (device & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+  }
+};
 
 typedef uint16_t bf16_t;  // storage
 

@@ -811,12 +811,10 @@ static int launch_gemm_nt(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, in
       return launch_gemm_nt<B_KN, QKV, 1, 8>(A, B, C, M, N, K, valid, s, qkv);
   }
   const size_t lds = (size_t)(T == 1 ? STAGES64 : NT_STAGES) * (BM + BN) * BK * 2;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV, T, STAGES64>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_nt_kernel<B_KN, QKV, T, STAGES64>), lds); e != hipSuccess) {
+    set_error("gemm: %s", hipGetErrorString(e));
+    return (int)e;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt_kernel<B_KN, QKV, T, STAGES64>), dim3(tiles_m * tiles_n), dim3(256), lds, s, A, B, C, M, N, K,
@@ -1100,12 +1098,10 @@ static int launch_qkv_either(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int 
   const Tiling thin{thin_m, total, patched_order(thin_m, total)};
   const size_t lds_narrow = (size_t)NT_STAGES * 256 * BK * 2, lds_wide = (size_t)Q3_STAGES * Q3_STAGE_BYTES;
   const size_t lds = lds_narrow > lds_wide ? lds_narrow : lds_wide;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv_either_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&qkv_either_kernel), lds); e != hipSuccess) {
+    set_error("prefill_qkv: %s", hipGetErrorString(e));
+    return (int)e;
   }
   int blocks = tiles_m * (narrow.tiles_n > wide.tiles_n ? narrow.tiles_n : wide.tiles_n);
   if (thin.tiles_m * thin.tiles_n > blocks) blocks = thin.tiles_m * thin.tiles_n;
@@ -1118,12 +1114,10 @@ static int launch_qkv64(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, in
                         const int* valid, hipStream_t s, QkvTail qkv) {
   const int tiles_m = (M + Q3_BM - 1) / Q3_BM, tiles_n = heads + 2 * kv_heads;
   const size_t lds = (size_t)Q1_STAGES * Q1_STAGE_BYTES;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv64_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&qkv64_kernel), lds); e != hipSuccess) {
+    set_error("prefill_qkv: %s", hipGetErrorString(e));
+    return (int)e;
   }
   hipLaunchKernelGGL(qkv64_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid,
                      tiles_m, tiles_n, patched_order(tiles_m, tiles_n), qkv);
@@ -1134,12 +1128,10 @@ static int launch_qkv192(const bf16_t* A, const bf16_t* Bq, bf16_t* Cq, int M, i
                          const int* valid, hipStream_t s, QkvTail qkv) {
   const int tiles_m = (M + Q3_BM - 1) / Q3_BM, tiles_n = (heads + 2 * kv_heads) / 3;
   const size_t lds = (size_t)Q3_STAGES * Q3_STAGE_BYTES;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv192_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("prefill_qkv: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&qkv192_kernel), lds); e != hipSuccess) {
+    set_error("prefill_qkv: %s", hipGetErrorString(e));
+    return (int)e;
   }
   hipLaunchKernelGGL(qkv192_kernel, dim3(tiles_m * tiles_n), dim3(256), lds, s, A, Bq, Cq, M, heads, kv_heads, K, valid,
                      tiles_m, tiles_n, patched_order(tiles_m, tiles_n), qkv);
@@ -1155,12 +1147,10 @@ static int launch_gemm(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N
 #define IRON_GEMM_LAUNCH(BNK, CNM)                                                          \
   do {                                                                                      \
     auto kern = gemm_kernel<BM, BN, WM, WN, BNK, CNM>;                                      \
-    static bool once = false;                                                               \
-    if (!once) {                                                                            \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),               \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-      if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }  \
-      once = true;                                                                          \
+    static LdsOptIn opt_in;                                                               \
+    if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(kern), lds); e != hipSuccess) { \
+      set_error("gemm: %s", hipGetErrorString(e));                                        \
+      return (int)e;                                                                      \
     }                                                                                       \
     hipLaunchKernelGGL(kern, grid, block, lds, s, A, B, C, M, N, K, valid, valid_k, tiles_m, \
                        tiles_n);                                                            \
@@ -1471,12 +1461,10 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   constexpr size_t lds256 = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
   constexpr size_t lds128 = (size_t)NT_STAGES * 256 * BK * 2;
   constexpr size_t lds = BIG ? (lds256 > lds128 ? lds256 : lds128) : lds128;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_either_kernel<BIG>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_either_kernel<BIG>), lds); e != hipSuccess) {
+    set_error("gemm: %s", hipGetErrorString(e));
+    return (int)e;
   }
   int blocks = t128.tiles_m * t128.tiles_n;
   if (t256.tiles_m * t256.tiles_n > blocks) blocks = t256.tiles_m * t256.tiles_n;
@@ -1492,12 +1480,10 @@ static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M,
   const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
   constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
   const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("gemm: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>), lds); e != hipSuccess) {
+    set_error("gemm: %s", hipGetErrorString(e));
+    return (int)e;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
   hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,

@@ -12,11 +12,15 @@
 #include "common.h"
 
 #include <mutex>
+#include <type_traits>
 
 namespace iron {
 
-constexpr int kMaxSplits = 128;
-constexpr int kSingleMaxKeys = 2048;  // caches up to this many rows take the one-launch kernel
+constexpr int kMaxSplits = 128;      // what the workspace holds per head
+constexpr int kScanMaxSplits = 128;  // the lane-scan kernels' own limit
+constexpr int kSingleMaxKeys = 2048;  // lane-scan kernels: caches up to this many rows take the one-launch kernel
+constexpr int kShortKeys = 2048;      // one-shape launch: up to this many live keys one block a query head writes O itself
+constexpr int kComputeUnits = 256;    // MI355X: what the split count is sized for
 
 // 2^x for x <= 0 by the hardware's own instruction: a softmax weight small enough to be a denormal
 // counts as 0, which saves the library routine's rescaling around every call.
@@ -217,7 +221,7 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
 template <int D>
 __global__ void mha_decode_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ O,
                                         int nsplit) {
-  __shared__ float wgt[kMaxSplits];
+  __shared__ float wgt[kScanMaxSplits];
   __shared__ float red[2][4];
   const int head = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const float* p = part + (size_t)head * nsplit * (D + 2);
@@ -301,6 +305,407 @@ __global__ __launch_bounds__(1024) void mha_decode_single_kernel(
     }
     O[(size_t)head * D + dd] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
   }
+}
+
+// The run of keys a block of the split scan takes: an equal share of the live keys, in whole
+// 16-key tiles for each of the 2^share_log2 waves that work on one KV head.  The scan and the merge
+// both derive it from the same words.
+__device__ __forceinline__ int decode_chunk(int live, int nsplit, int share_log2) {
+  const int unit = 16 << share_log2;
+  return ((live + nsplit - 1) / nsplit + unit - 1) & ~(unit - 1);
+}
+
+// ---- one query, one launch shape whatever the cache's length
+//
+// grid = (sets, nsplit) blocks of WAVES waves, as many as the chip has CUs; the blocks choose what to
+// do by the live keys n = *kv_valid (less what a window drops), so the work and its spread over the
+// chip follow the context and the cache only sizes the buffers.
+//
+// n <= short_keys: the first `heads` blocks each scan all keys for one query head with the
+// lane-per-column scan above (16 waves a head: the launch is latency-bound, and this is the shortest
+// chain) and write the output row; the others leave at once, and so does the merge launch behind.
+//
+// Otherwise the keys are dealt over the nsplit blocks of a set of KV heads in equal runs sized by n,
+// and a block leaves (max, sum, O) per head for the merge.  Here the G query heads that share a KV
+// head are the columns of a 16-wide MFMA tile (G <= 16; the rest are zero columns), so a key row is
+// multiplied with all of them by one instruction stream whatever G is.  A wave works through its own
+// run of keys 32 at a time.  S^T = K Q^T (M = keys, N = heads): the K rows are the A operand exactly
+// as they lie in memory (lane -> key row lane % 16, 16-byte piece lane / 16 of a 32-wide k-step), so
+// they go from global memory straight into registers.  A lane then owns one head column: the softmax
+// is in-lane but for the maximum over the four lanes of a column, which is only exchanged on the
+// (rare) steps where some lane's own maximum passes the column's reference.  The probabilities,
+// rounded to bf16, are already the B operand of O^T = V^T P^T; V^T comes from the transposing LDS read
+// of the wave's own 32-row V tile, which buffer loads put there as stored (16-byte chunks
+// XOR-swizzled by 2 (row & 3), as the prompt kernel's).  Rows past the last live key lie outside the
+// buffers and read as zeros.
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void mha_decode_either_kernel(
+    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
+    bf16_t* __restrict__ O, float* __restrict__ part, int kv_heads, int group, int hpb_log2, int kv_len,
+    float scale_log2, int window, long row_stride, long head_stride, const int* __restrict__ kv_valid,
+    const int* __restrict__ kv_first, int kv_rows, int short_keys) {
+  constexpr int ROWB = D * 2;            // bytes of a V row in LDS
+  constexpr int KS = D / 32;             // 32-wide k-steps of S^T
+  constexpr int DT = D / 16;             // 16-row tiles of O^T
+  constexpr int CPR = D / 8;             // 16-byte chunks of a row
+  constexpr int TK = 32;                 // keys a step
+  constexpr int TILE = TK * ROWB;        // bytes of a V tile
+  constexpr int VINST = TILE / 1024;     // 1 KB loads into LDS a tile
+  constexpr int RPI = 1024 / ROWB;       // rows one of them covers
+  constexpr int WAVES_LOG2 = WAVES == 16 ? 4 : 3;
+  static_assert(WAVES == 16 || WAVES == 8, "waves a block");
+  extern __shared__ __align__(1024) char smem_dec[];   // WAVES x 2 x TILE bytes
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nsplit = gridDim.y;
+
+  const int kv_tokens = bound_or(kv_valid, kv_len);
+  const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
+  const int live = kv_tokens - first;
+  const long first_row = kv_first ? max(0, min(*kv_first, kv_rows - kv_len)) : 0;
+
+  if (live <= short_keys) {
+    // ---- few keys: block b is one query head, as mha_decode_single_kernel
+    constexpr int LPR = D / 8, RW = 64 / LPR, U = 8;
+    const int b = blockIdx.y * gridDim.x + blockIdx.x;
+    if (b >= kv_heads * group) return;
+    const int kvh = b % kv_heads, head = kvh * group + b / kv_heads;
+    const int sub = lane % LPR, rg = lane / LPR;
+    const bf16_t* Kh = K + (size_t)kvh * head_stride + first_row * row_stride;
+    const bf16_t* Vh = V + (size_t)kvh * head_stride + first_row * row_stride;
+    float m[1], l[1], acc[1][8];
+    decode_scan<D, 1, U, false>(Q, Kh, Vh, head, first + wave * U * RW, kv_tokens, WAVES * U * RW, row_stride,
+                                scale_log2, m, l, acc);
+    float* sm = reinterpret_cast<float*>(smem_dec);   // [WAVES] maxima, [WAVES] sums, [WAVES][D] columns
+    float* sl = sm + WAVES;
+    float* sacc = sl + WAVES;
+    if (rg == 0) {
+      if (sub == 0) {
+        sm[wave] = m[0];
+        sl[wave] = l[0];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sacc[wave * D + sub * 8 + i] = acc[0][i];
+    }
+    __syncthreads();
+    if (tid < D) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, sm[w]);
+      const float ref = (mx == -INFINITY) ? 0.f : mx;
+      float lt = 0.f, at = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        const float e = exp2f(sm[w] - ref);
+        lt += sl[w] * e;
+        at += sacc[w * D + tid] * e;
+      }
+      O[(size_t)head * D + tid] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
+    }
+    return;
+  }
+
+  // ---- many keys: the block takes one run of them for 2^hpb_log2 KV heads at once, wave w on head
+  // w % hpb (with the heads interleaved in a cache row, the block's loads then cover longer pieces of it).
+  const int n = lane & 15, q = lane >> 4;   // head column, quarter of the k slots
+  const int hpb = 1 << hpb_log2, share_log2 = WAVES_LOG2 - hpb_log2;
+  const int split = blockIdx.y;
+  const int kvh = (blockIdx.x << hpb_log2) + (wave & (hpb - 1));
+  const int sub = wave >> hpb_log2;          // this wave's place among the 2^share_log2 on its head
+  const int chunk = decode_chunk(live, nsplit, share_log2);
+  const int blo = first + split * chunk, bhi = min(blo + chunk, kv_tokens);
+  if (blo >= kv_tokens) return;   // the merge reads the splits that hold keys, no more
+  // The wave's run of keys, in whole 16-key MFMA tiles.
+  const int per = ((((bhi - blo) + (1 << share_log2) - 1) >> share_log2) + 15) & ~15;
+  const int wlo = blo + sub * per, whi = min(wlo + per, bhi);
+  const int steps = wlo < whi ? (whi - wlo + TK - 1) / TK : 0;
+
+  const bf16_t* Kh = K + (size_t)kvh * head_stride + first_row * row_stride;
+  const bf16_t* Vh = V + (size_t)kvh * head_stride + first_row * row_stride;
+  const int row_bytes = (int)row_stride * 2;
+  // The head's keys (values) up to the last live one are one buffer: rows past it read as zeros.
+  const int reach = (kv_tokens - 1) * row_bytes + ROWB;
+  const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(Kh), 0, reach, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(Vh), 0, reach, 0x00020000);
+
+  // K fragments: tile t of the step, k-step s -> key 16 t + n, bytes 64 s + 16 q of its row.
+  const int k_lane = n * row_bytes + 16 * q;
+  // V into LDS: load i covers tile rows i RPI + lane / CPR; a lane fetches the logical chunk that the
+  // row's swizzle maps to its physical one.
+  int v_lane[VINST];
+#pragma unroll
+  for (int i = 0; i < VINST; ++i) {
+    const int r = i * RPI + lane / CPR;
+    v_lane[i] = r * row_bytes + (((lane % CPR) ^ ((r & 3) << 1)) << 4);
+  }
+  char* stage = smem_dec + wave * (2 * TILE);
+
+  bf16x8 kf[2][2][KS];   // [register set][tile][k-step]
+  auto issue_v = [&](int step, int set) {
+    const int at = (wlo + step * TK) * row_bytes;
+#pragma unroll
+    for (int i = 0; i < VINST; ++i)
+      // (the cast keeps the offset's type from depending on the template: as a dependent expression
+      // the host pass drops the kernel's stub without a word)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rows, IRON_LDS_PTR(stage + set * TILE + i * 1024), 16,
+                                               (int)v_lane[i] + at, 0, 0, 0);
+  };
+  auto issue = [&](int step, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
+    const int at = (wlo + step * TK) * row_bytes;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        kf[set][t][s] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(
+            k_rows, at + k_lane + t * 16 * row_bytes + 64 * s, 0, 0));
+  };
+  // Steps go in pairs: both steps' loads are out before either is waited for, and the next pair's go
+  // out as each of this pair's register set and stage buffer falls free.  The wait is for everything
+  // in flight, so it needs no count of what the compiler may have moved.
+  using set0 = std::integral_constant<int, 0>;
+  using set1 = std::integral_constant<int, 1>;
+  if (steps > 0) {
+    issue_v(0, 0);
+    issue(0, set0{});
+  }
+  if (steps > 1) {
+    issue_v(1, 1);
+    issue(1, set1{});
+  }
+
+  // Q^T fragments (B operand): lane holds head column n, d = 32 s + 8 q .. + 7; zero columns past G.
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (n < group) v = *reinterpret_cast<const uint4*>(Q + (size_t)(kvh * group + n) * D + 32 * s + 8 * q);
+    qf[s] = __builtin_bit_cast(bf16x8, v);
+  }
+  // V^T fragments (A operand of O^T): the lanes of quarter q point at rows 4 q + 0..3 (k slots 8 q + 0..3;
+  // the same 16 rows on for slots 8 q + 4..7, as S^T's second tile lies in P), 4 columns each of the 16.
+  const int v_swz = ((lane >> 2) & 3) << 1;
+  unsigned v_frag[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    v_frag[dt] = (unsigned)(size_t)IRON_LDS_PTR(stage) + (4 * q + ((lane & 15) >> 2)) * ROWB +
+                 (((2 * dt + ((lane & 3) >> 1)) ^ v_swz) << 4) + ((lane & 1) << 3);
+
+  f32x4 oacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_ref = -INFINITY, l_run = 0.f;   // the column's reference maximum (raw scores), this lane's sum
+
+  auto compute = [&](int step, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
+    TrFrag vf[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      vf[dt].lo = lds_read_tr16_at<set * TILE>(v_frag[dt]);
+      vf[dt].hi = lds_read_tr16_at<set * TILE + 16 * ROWB>(v_frag[dt]);
+    }
+    f32x4 sacc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      sacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s) sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[set][t][s], qf[s], sacc[t], 0, 0, 0);
+    }
+    // Element i of tile t is key k0 + 16 t + 4 q + i; the wave's last step may reach past its run.
+    const int k0 = wlo + step * TK;
+    const int left = whi - k0 - 4 * q;   // keys of this lane's tile-0 quarter inside the run (may be <= 0)
+    const bool edge = k0 + TK > whi;
+    if (edge) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (16 * t + i >= left) sacc[t][i] = -INFINITY;
+    }
+    float lm = sacc[0][0];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lm = fmaxf(lm, sacc[t][i]);
+    if (__builtin_amdgcn_ballot_w64(lm > m_ref) != 0) {
+      float mx = fmaxf(lm, __shfl_xor(lm, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_ref, mx);
+      // A column that had seen no key has zero sums to rescale; one that still has none keeps -inf.
+      const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_ref - m_new) * scale_log2);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
+      m_ref = m_new;
+    }
+    const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * scale_log2;
+    float p[8];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float e = __builtin_amdgcn_exp2f(fmaf(sacc[t][i], scale_log2, -mc));
+        if (edge && 16 * t + i >= left) e = 0.f;   // also where the scale is 0 and -inf * 0 is no number
+        p[4 * t + i] = e;
+        l_run += e;
+      }
+    const bf16x8 pf = __builtin_bit_cast(bf16x8, pack8(p));
+#pragma unroll
+    for (int dt = 0; dt < DT; dt += 2) {
+      lds_tr_wait(vf[dt], vf[dt + 1]);
+      oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tr_join(vf[dt]), pf, oacc[dt], 0, 0, 0);
+      oacc[dt + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tr_join(vf[dt + 1]), pf, oacc[dt + 1], 0, 0, 0);
+    }
+  };
+
+  for (int step = 0; step < steps; step += 2) {
+    wait_vmcnt<0>();
+    compute(step, set0{});
+    if (step + 2 < steps) {
+      issue_v(step + 2, 0);
+      issue(step + 2, set0{});
+    }
+    if (step + 1 < steps) {
+      compute(step + 1, set1{});
+      if (step + 3 < steps) {
+        issue_v(step + 3, 1);
+        issue(step + 3, set1{});
+      }
+    }
+  }
+  wait_vmcnt<0>();
+
+  // The lane's sum over its own keys -> the column's.
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+
+  // Waves hand (max, sum, O^T column) per head over through LDS (the stage buffers, once every wave
+  // is out of its loop); thread (head, d) folds the waves of its KV head, every read issued before
+  // the first is used.
+  __syncthreads();
+  float* hand = reinterpret_cast<float*>(smem_dec);   // [WAVES][group][D + 2]
+  static_assert(16 * (D + 2) * 4 <= 2 * TILE, "a wave's hand-over fits its own stage buffers");
+  if (n < group) {
+    float* mine = hand + ((size_t)wave * group + n) * (D + 2);
+    if (q == 0) {
+      mine[0] = m_ref;
+      mine[1] = l_run;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[2 + 16 * dt + 4 * q + i] = oacc[dt][i];
+  }
+  __syncthreads();
+  // Column hg = (head of the block's, query head of its group) lies in waves hw, hw + hpb, ...: entry
+  // hg + j hpb group of the hand-over for j < share.
+  const int share = 1 << share_log2;
+  const int wave_step = (group << hpb_log2) * (D + 2);
+  for (int idx = tid; idx < (group << hpb_log2) * D; idx += 64 * WAVES) {
+    const int hg = idx / D, dd = idx % D;
+    const float* col = hand + (size_t)hg * (D + 2);
+    float mv[WAVES], lv[WAVES], av[WAVES];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      mv[w] = -INFINITY;
+      lv[w] = av[w] = 0.f;
+      if (w < share) {   // uniform over the block
+        mv[w] = col[w * wave_step];
+        lv[w] = col[w * wave_step + 1];
+        av[w] = col[w * wave_step + 2 + dd];
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, mv[w]);
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float e = (mv[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mv[w] - mx) * scale_log2);
+      lt = fmaf(lv[w], e, lt);
+      at = fmaf(av[w], e, at);
+    }
+    // part layout: [head][split][D + 2] = {max in the exp2 domain, sum, O[D]}.
+    const int head = (blockIdx.x << hpb_log2) * group + hg;
+    float* out = part + ((size_t)head * nsplit + split) * (D + 2);
+    out[2 + dd] = at;
+    if (dd == 0) {
+      out[0] = (mx == -INFINITY) ? -INFINITY : mx * scale_log2;
+      out[1] = lt;
+    }
+  }
+}
+
+// The splits' merge, a block of four waves a head: thread (part, d) sums column d over the splits
+// part, part + 4, ... that hold keys, 32 of them at a time, and the four parts are folded through LDS.
+// A thread's first 32 are requested together with the bound, before it is known how many of them hold
+// anything (the workspace is the caller's own memory, whatever it holds): one trip to memory, not two,
+// for up to 128 splits.  Leaves at once where the scan's blocks wrote the output themselves.
+template <int D>
+__global__ __launch_bounds__(4 * D) void mha_decode_either_merge_kernel(
+    const float* __restrict__ part, bf16_t* __restrict__ O, int nsplit, int share_log2, int kv_len, int window,
+    const int* __restrict__ kv_valid, int short_keys) {
+  const int head = blockIdx.x, t = threadIdx.x % D, quarter = threadIdx.x / D;
+  const float* p = part + (size_t)head * nsplit * (D + 2);
+  float m[32], l[32], a[32];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    const int s = min(quarter + 4 * i, nsplit - 1);
+    m[i] = p[s * (D + 2)];
+    l[i] = p[s * (D + 2) + 1];
+    a[i] = p[s * (D + 2) + 2 + t];
+  }
+  const int kv_tokens = bound_or(kv_valid, kv_len);
+  const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
+  const int live = kv_tokens - first;
+  if (live <= short_keys) return;
+  const int chunk = decode_chunk(live, nsplit, share_log2);
+  const int used = (live + chunk - 1) / chunk;
+  float mx = -INFINITY, lt = 0.f, at = 0.f;
+  for (int s0 = quarter; s0 < used; s0 += 128) {
+    if (s0 >= 128) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        const int s = min(s0 + 4 * i, used - 1);
+        m[i] = p[s * (D + 2)];
+        l[i] = p[s * (D + 2) + 1];
+        a[i] = p[s * (D + 2) + 2 + t];
+      }
+    }
+    float cm = mx;
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+      if (s0 + 4 * i < used) cm = fmaxf(cm, m[i]);
+    const float keep = (mx == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mx - cm);
+    lt *= keep;
+    at *= keep;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const bool in = s0 + 4 * i < used && m[i] != -INFINITY;
+      const float e = in ? __builtin_amdgcn_exp2f(m[i] - cm) : 0.f;
+      lt = fmaf(in ? l[i] : 0.f, e, lt);
+      at = fmaf(in ? a[i] : 0.f, e, at);
+    }
+    mx = cm;
+  }
+  __shared__ float fm[4][D], fl[4][D], fa[4][D];
+  fm[quarter][t] = mx;
+  fl[quarter][t] = lt;
+  fa[quarter][t] = at;
+  __syncthreads();
+  if (quarter != 0) return;
+  float top = fmaxf(fmaxf(fm[0][t], fm[1][t]), fmaxf(fm[2][t], fm[3][t]));
+  float ls = 0.f, as = 0.f;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float e = (fm[k][t] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fm[k][t] - top);
+    ls = fmaf(fl[k][t], e, ls);
+    as = fmaf(fa[k][t], e, as);
+  }
+  O[(size_t)head * D + t] = f32_to_bf16(ls > 0.f ? as / ls : 0.f);
 }
 
 // Many queries, a block a (query row, head): the same scan as above per query, over the keys its
@@ -395,8 +800,38 @@ static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf1
   else
     hipLaunchKernelGGL((mha_decode_kernel<D, G, 4>), dim3(kv_heads, nsplit), dim3(256), 0, s, Q, K, V,
                        part, kv_len, scale_log2, window, row_stride, head_stride, kv_valid, kv_first, kv_rows);
-  hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D > kMaxSplits ? D : kMaxSplits), 0, s,
+  hipLaunchKernelGGL((mha_decode_merge_kernel<D>), dim3(kv_heads * G), dim3(D > kScanMaxSplits ? D : kScanMaxSplits), 0, s,
                      part, O, nsplit);
+}
+
+
+// The one-shape launch and, where the cache can hold more than `short_keys` rows, the merge behind it.
+template <int D, int WAVES>
+static int launch_decode_either(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, float* part, int kv_heads,
+                                int group, int kv_len, float scale_log2, int window, long row_stride, long head_stride,
+                                const int* kv_valid, const int* kv_first, int kv_rows, int short_keys, hipStream_t s) {
+  constexpr size_t lds = (size_t)WAVES * 2 * 32 * D * 2;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_decode_either_kernel<D, WAVES>), lds); e != hipSuccess) {
+    set_error("mha_decode: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  // A block of the split scan serves two KV heads where their number is even (with the heads
+  // interleaved in a cache row its loads then cover 256-byte pieces: measured a tenth faster than one
+  // head a block; four or eight heads a block stream faster still but leave more, smaller partial
+  // results), and there are as many blocks as the chip has CUs -- and no fewer than query heads,
+  // which the few-keys form needs -- whatever the cache's length.
+  const int hpb_log2 = kv_heads % 2 == 0 ? 1 : 0;
+  const int sets = kv_heads >> hpb_log2;
+  int nsplit = kComputeUnits / sets;
+  while (sets * nsplit < kv_heads * group) ++nsplit;
+  nsplit = nsplit < 1 ? 1 : (nsplit > kMaxSplits ? kMaxSplits : nsplit);
+  hipLaunchKernelGGL((mha_decode_either_kernel<D, WAVES>), dim3(sets, nsplit), dim3(64 * WAVES), lds, s, Q, K, V, O,
+                     part, kv_heads, group, hpb_log2, kv_len, scale_log2, window, row_stride, head_stride, kv_valid,
+                     kv_first, kv_rows, short_keys);
+  hipLaunchKernelGGL((mha_decode_either_merge_kernel<D>), dim3(kv_heads * group), dim3(4 * D), 0, s, part, O, nsplit,
+                     (WAVES == 16 ? 4 : 3) - hpb_log2, kv_len, window, kv_valid, short_keys);
+  return 0;
 }
 
 }  // namespace iron
@@ -407,9 +842,11 @@ extern "C" int64_t iron_mha_decode_workspace_bytes(int heads, int d) {
   return (int64_t)heads * kMaxSplits * (d + 2) * sizeof(float);
 }
 
+// form: 0 the default choice, 1 the lane-per-column scans, 2 the matrix-core scan (d = 64 / 128);
+// short_keys: up to how many live keys the matrix-core scan's one block a KV head writes O itself (0: the default).
 static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O, int heads, int kv_heads,
                       int d, int kv_len, float scale, int window, int kv_interleaved, const int* kv_valid,
-                      const int* kv_first, int kv_rows, void* workspace, void* stream) {
+                      const int* kv_first, int kv_rows, void* workspace, void* stream, int form = 0, int short_keys = 0) {
   IRON_REQUIRE(Q && K && V && O && workspace, "mha_decode: null operand");
   IRON_REQUIRE(kv_first == nullptr || (kv_interleaved && kv_rows >= kv_len),
                "mha_decode: a window of the keys takes them row by row (kv_interleaved) out of kv_rows (%d) >= kv_len (%d)",
@@ -427,11 +864,28 @@ static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, u
   // (beyond that the merge of the splits costs more than the extra parallelism gains).
   int nsplit = (kv_len + 127) / 128;
   nsplit = nsplit < 8 ? 8 : (nsplit > 64 ? 64 : nsplit);
-  if (kv_len > 64 * 256) nsplit = (kv_len + 255) / 256 > kMaxSplits ? kMaxSplits : (kv_len + 255) / 256;
+  if (kv_len > 64 * 256) nsplit = (kv_len + 255) / 256 > kScanMaxSplits ? kScanMaxSplits : (kv_len + 255) / 256;
   if (nsplit * 8 > kv_len) nsplit = kv_len >= 8 ? kv_len / 8 : 1;
   const float scale_log2 = scale * 1.4426950408889634f;
   hipStream_t s = (hipStream_t)stream;
   float* part = (float*)workspace;
+  IRON_REQUIRE(form >= 0 && form <= 2 && short_keys >= 0, "mha_decode: form (%d) is 0, 1 or 2 and short_keys (%d) not negative",
+               form, short_keys);
+  // Caches that can hold more rows than a single block scans well: one launch shape, the blocks
+  // choosing by the live keys (d = 64 / 128).  Shorter ones, and the other widths, below.
+  const bool either_fits = (d == 64 || d == 128) && G <= 16 && row_stride <= (1L << 20) &&
+                           (long)kv_len * row_stride * 2 < (1L << 31) && heads <= kMaxSplits * kv_heads;
+  IRON_REQUIRE(form != 2 || either_fits,
+               "mha_decode: the one-shape launch takes d = 64 or 128, up to 16 query heads a KV head and keys within 2^31 bytes");
+  const int upto = short_keys > 0 ? short_keys : kShortKeys;
+  if (form == 2 || (form == 0 && either_fits && kv_len > upto)) {
+    const int rc = d == 64 ? launch_decode_either<64, 16>(Q, K, V, O, part, kv_heads, G, kv_len, scale_log2, window, row_stride,
+                                                          head_stride, kv_valid, kv_first, kv_rows, upto, s)
+                           : launch_decode_either<128, 8>(Q, K, V, O, part, kv_heads, G, kv_len, scale_log2, window, row_stride,
+                                                          head_stride, kv_valid, kv_first, kv_rows, upto, s);
+    if (rc != 0) return rc;
+    IRON_LAUNCH_CHECK();
+  }
   // Caches this short are launch-bound: one launch that needs no merge of splits.
   // ... and 512-wide heads take it at any length (no split kernel is built for them).
   if ((kv_len <= kSingleMaxKeys && (d == 64 || d == 128 || d == 256)) || d == 512) {
@@ -462,7 +916,7 @@ static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, u
 #undef IRON_DEC_D
 #undef IRON_DEC
   IRON_REQUIRE(false, "mha_decode: no kernel for d=%d with %d query heads per KV head "
-               "(d in {64,128,256} with a group in {1,2,3,4,5,6,8}, or d = 512)", d, G);
+               "(d in {64,128} with up to 16, d = 256 with 1, 2, 3, 4, 5, 6 or 8, or d = 512)", d, G);
 }
 
 extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
@@ -471,6 +925,15 @@ extern "C" int iron_mha_decode_bf16(const uint16_t* Q, const uint16_t* K, const 
                                     const int* kv_valid, void* workspace, void* stream) {
   return mha_decode(Q, K, V, O, heads, kv_heads, d, kv_len, scale, window, kv_interleaved, kv_valid, nullptr, 0,
                     workspace, stream);
+}
+
+extern "C" int iron_mha_decode_tuned_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                                          uint16_t* O, int heads, int kv_heads, int d, int kv_len,
+                                          float scale, int window, int kv_interleaved,
+                                          const int* kv_valid, void* workspace, int form, int short_keys,
+                                          void* stream) {
+  return mha_decode(Q, K, V, O, heads, kv_heads, d, kv_len, scale, window, kv_interleaved, kv_valid, nullptr, 0,
+                    workspace, stream, form, short_keys);
 }
 
 // ---- the entry point that allocates nothing

@@ -403,12 +403,10 @@ template <int D, int SPLIT, int W = 4>
 static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
   constexpr int STAGES = D == 64 ? 3 : 2;
   constexpr size_t lds = (size_t)SPLIT * STAGES * 2 * BKV * D * 2;
-  static bool once = false;
-  if (!once) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT, W>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { set_error("mha_prefill: %s", hipGetErrorString(e)); return (int)e; }
-    once = true;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT, W>), lds); e != hipSuccess) {
+    set_error("mha_prefill: %s", hipGetErrorString(e));
+    return (int)e;
   }
   hipLaunchKernelGGL((mha_prefill_kernel<D, SPLIT, W>), dim3(blocks), dim3(64 * W * SPLIT), lds, (hipStream_t)stream, a.Q,
                      a.K, a.V, a.O, a.heads, a.group, a.seq, a.seq_len, a.kv_len, a.scale_log2, a.causal, a.window,

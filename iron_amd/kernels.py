@@ -344,9 +344,10 @@ def mha_decode_workspace(heads, d, device="cuda"):
 
 def mha_decode(
     Q, K, V, O, *, heads, kv_heads, d, kv_len, scale=None, window=None, kv_interleaved=False,
-    kv_valid=None, workspace, kv_first=None, kv_rows=None,
+    kv_valid=None, workspace, kv_first=None, kv_rows=None, form=0, short_keys=0,
 ):
-    """``kv_first`` / ``kv_rows``: the keys are a window of a longer buffer, as ``mha_prefill``'s."""
+    """``kv_first`` / ``kv_rows``: the keys are a window of a longer buffer, as ``mha_prefill``'s.
+    ``form`` / ``short_keys`` force the kernel form (``iron_mha_decode_tuned_bf16``)."""
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     _numel(_dev(Q, "Q"), heads * d, "Q")
     _numel(_dev(O, "O"), heads * d, "O")
@@ -367,6 +368,16 @@ def mha_decode(
         return
     _numel(_dev(K, "K"), kv_len * kv_heads * d, "K")
     _numel(_dev(V, "V"), kv_len * kv_heads * d, "V")
+    if form or short_keys:
+        check(
+            lib().iron_mha_decode_tuned_bf16(
+                ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, kv_len, float(scale),
+                -1 if window is None else int(window), int(kv_interleaved),
+                ptr(_word(kv_valid, "kv_valid")), ptr(workspace), int(form), int(short_keys), current_stream(),
+            ),
+            "iron_mha_decode_tuned_bf16",
+        )
+        return
     check(
         lib().iron_mha_decode_bf16(
             ptr(Q), ptr(K), ptr(V), ptr(O), heads, kv_heads, d, kv_len, float(scale),

@@ -15,6 +15,10 @@ from ..common.declare import Built, In, Operator, Out, Scratch, Select, ceildiv,
 from ..common.testing import Case, Testing
 from ..common.verify import Tolerance
 
+# One query: up to this many live keys one launch does it all (a block a query head); a cache that can
+# hold more takes the launch whose blocks choose by the live keys, and a merge launch behind it.
+SHORT_KEYS = 2048
+
 _CASES = [
     Case(dict(num_heads=1, seq_len=16384), bench=True),
     Case(dict(num_heads=8, num_KV_heads=2, seq_len=16384), extensive=True, bench=True),
@@ -114,9 +118,11 @@ class MHA(Operator):
         if self.kv_len < self.seq_pad:
             raise ValueError(f"MHA: kv_len ({self.kv_len}) must be at least seq_pad ({self.seq_pad}): "
                              "the queries are its last rows")
-        if self.seq_len == 1 and self.num_heads // self.num_KV_heads not in (1, 2, 3, 4, 5, 6, 8):
-            raise ValueError(f"MHA: one query takes 1, 2, 3, 4, 5, 6 or 8 query heads per KV head, "
-                             f"not {self.num_heads // self.num_KV_heads}")
+        group = self.num_heads // self.num_KV_heads
+        if self.seq_len == 1 and group not in (1, 2, 3, 4, 5, 6, 8) and not (
+                group <= 16 and (self.d in (64, 128) or self.kv_len <= SHORT_KEYS)) and self.d != 512:
+            raise ValueError(f"MHA: one query takes up to 16 query heads per KV head at d = 64 or 128 "
+                             f"(1, 2, 3, 4, 5, 6 or 8 at d = 256 over more than {SHORT_KEYS} keys), not {group}")
         if self.seq_len == 1 and not self.causal and self.window is not None:
             raise ValueError("MHA: one query past every key attends backwards: causal")
 
@@ -175,17 +181,26 @@ class MHA(Operator):
             kvi = self.kv_interleaved
             own = {}
 
+            # While the context stays within SHORT_KEYS rows, attention over the cache's first
+            # SHORT_KEYS rows is the same attention, in one launch: a graph that follows its per-call
+            # values on the host captures that form too and replays it for as long as it holds.
+            bounded = ("kv_valid", SHORT_KEYS) if kvi and L > SHORT_KEYS and d != 512 else None
+
             def launch(t, words):
                 ws = t.get("workspace")
                 if ws is None:  # a call outside a graph: allocated once, kept
                     ws = own.get("ws")
                     if ws is None:
                         ws = own["ws"] = kernels.mha_decode_workspace(H, d, t["Q"].device)
-                kernels.mha_decode(t["Q"], t["K"], t["V"], t["O"], heads=H, kv_heads=G, d=d, kv_len=L,
+                keys, values, rows, ring = t["K"], t["V"], L, _key_window(words, G * d)
+                if bounded and not ring and (words.get("__context__") or {}).get("bounded"):
+                    rows = SHORT_KEYS
+                    keys, values = keys.reshape(-1)[: rows * G * d], values.reshape(-1)[: rows * G * d]
+                kernels.mha_decode(t["Q"], keys, values, t["O"], heads=H, kv_heads=G, d=d, kv_len=rows,
                                    scale=scale, window=window, kv_interleaved=kvi,
-                                   kv_valid=words.get("kv_valid"), workspace=ws, **_key_window(words, G * d))
+                                   kv_valid=words.get("kv_valid"), workspace=ws, **ring)
 
-            return Built("iron_mha_decode_bf16", launch)
+            return Built("iron_mha_decode_bf16", launch, bounded)
         seq, seq_len, causal = self.seq_pad, self.seq_len, self.causal
         qi, kvi = self.heads_interleaved, self.kv_interleaved
 

@@ -848,6 +848,54 @@ def test_mha_decode_bounds_windows_groups(cuda, H, G, d, kv_valid, window, L):
         close(O, want)
 
 
+@pytest.mark.parametrize("H,G,d", [(32, 8, 64), (16, 1, 64), (7, 7, 64), (24, 8, 128), (26, 2, 128)])
+@pytest.mark.parametrize("form,short_keys", [(1, 0), (2, 0), (2, 48)])
+def test_mha_decode_every_form_at_every_context(cuda, H, G, d, form, short_keys):
+    """The lane-per-column scans, and the one-shape launch both as a block a query head (few keys) and
+    as runs of keys dealt over the chip with a merge behind (forced onto small contexts by
+    ``short_keys``): contexts that end inside a wave's 16-key tile, at a run's edge and at the cache's
+    last row; windows; rows past the bound and the whole workspace poisoned."""
+    if form == 1 and H // G not in (1, 2, 3, 4, 5, 6, 8):
+        pytest.skip("the lane-scan kernels take 1, 2, 3, 4, 5, 6 or 8 query heads a KV head")
+    rng = np.random.default_rng(161)
+    L = 3000
+    Q, Kc, Vc = bf(rng, 1, H, d), bf(rng, L, G, d), bf(rng, L, G, d)
+    dQ = dev(Q, cuda)
+    ws = K.mha_decode_workspace(H, d, cuda)
+    for kv_valid, window in ((1, None), (17, None), (48, None), (49, None), (777, None), (2049, None), (3000, None),
+                             (2500, 100), (2500, 1500), (3000, 2999)):
+        Kp, Vp = Kc.copy(), Vc.copy()
+        Kp[kv_valid:], Vp[kv_valid:] = np.nan, np.nan
+        ws.fill_(float("nan"))
+        O = out_like((1, H, d), cuda, fill=float("nan"))
+        K.mha_decode(dQ, dev(Kp, cuda), dev(Vp, cuda), O, heads=H, kv_heads=G, d=d, kv_len=L, window=window,
+                     kv_interleaved=True, kv_valid=word(kv_valid, cuda), workspace=ws, form=form, short_keys=short_keys)
+        want = ops.mha(Q, Kp, Vp, num_heads=H, num_KV_heads=G, seq_len=1, kv_len=L, d=d, window=window,
+                       heads_interleaved=True, kv_interleaved=True, kv_valid=kv_valid)
+        close(O, want)
+
+
+def test_mha_decode_cost_follows_the_context_not_the_cache(cuda):
+    """One compile, any context (AGENTS.md:246-255, iron/operators/mha.py:275-278): over a 131072-row
+    cache -- Llama-3.2-1B's own max_seq_len -- a context of 600 keys, one just past what a single block
+    takes, and the whole cache, each against the oracle; and the launches of the first are those of a
+    2048-row cache's (one block a query head does the work), not the cache's."""
+    rng = np.random.default_rng(162)
+    H, G, d, L = 32, 8, 64, 131072
+    Q = bf(rng, 1, H, d)
+    Kc = round_bf16(np.resize(rng.standard_normal((4099, G, d)), (L, G, d)).astype(np.float32))
+    Vc = round_bf16(np.resize(rng.standard_normal((4099, G, d)), (L, G, d)).astype(np.float32))
+    dQ, dK, dV = dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda)
+    ws = K.mha_decode_workspace(H, d, cuda)
+    for kv_valid in (600, 2049, 40000, L):
+        O = out_like((1, H, d), cuda, fill=float("nan"))
+        K.mha_decode(dQ, dK, dV, O, heads=H, kv_heads=G, d=d, kv_len=L, kv_interleaved=True,
+                     kv_valid=word(kv_valid, cuda), workspace=ws)
+        want = ops.mha(Q, Kc[:kv_valid], Vc[:kv_valid], num_heads=H, num_KV_heads=G, seq_len=1, kv_len=kv_valid, d=d,
+                       heads_interleaved=True, kv_interleaved=True)
+        close(O, want)
+
+
 def test_mha_decode_equals_last_row_of_prefill(cuda):
     """A size-independent property: the one-query kernel and the last row of the many-query one agree."""
     rng = np.random.default_rng(17)

@@ -371,6 +371,121 @@ def test_all_sixteen_layers_of_llama_1b_prompt_then_captured_decode(cuda):
         gpu.release()
 
 
+def _fill_caches(gpu, cpu, n: int, upto: int) -> None:
+    """Repeat the caches' first ``n`` rows, a prompt's, up to row ``upto`` -- on the device, and as the
+    host model's state (the device's rows, so that what is compared is the step and not the history):
+    the reference's ``_fill_caches`` (iron/lm/testing.py:367-392) for linear caches."""
+    from iron_amd.common.graph import walk
+
+    version = gpu.decode_step
+    device_states = [x for _, x, parent, _ in walk(gpu) if isinstance(parent, KVCache)]
+    host_states = [x for _, x, parent, _ in walk(cpu) if isinstance(parent, KVCache)]
+    assert device_states and len(device_states) == len(host_states)
+    for on_device, on_host in zip(device_states, host_states):
+        rows = version.read(on_device)
+        for start in range(n, upto, n):
+            rows[start : min(start + n, upto)] = rows[: min(n, upto - start)]
+        version.push(on_device)
+        cpu.decode_step.write(on_host, rows)
+
+
+@pytest.fixture(scope="module")
+def deep(cuda):
+    """Two layers at Llama-3.2-1B's width over caches of 16384 rows in 2048-row chunks, on the GPU and
+    as the graph's host reference, a 300-token prompt run through both."""
+    config = dataclasses.replace(LLAMA_3_2_1B, num_hidden_layers=2, max_seq_len=16384, prefill_chunk=2048)
+    w = weights(config, seed=1)
+    gpu, cpu = Llama(config, w), HostLlama(dataclasses.replace(config, prefill_chunk=512), w)
+    gpu.load_versions()
+    cpu.load_versions()
+    tokens = np.random.default_rng(21).integers(0, config.vocab_size, 300)
+    want, got = cpu.logits(tokens), gpu.logits(tokens)
+    assert_close(got, want, "the prompt")
+    yield gpu, cpu, tokens, int(want.argmax())
+    gpu.release()
+
+
+@pytest.mark.parametrize("position", [600, 2047, 2048, 5000, 16383])
+def test_decode_deep_in_the_cache(deep, position):
+    """The reference's ``check_deep_decode`` (iron/lm/testing.py:314-331, held by
+    tests/applications/long_context/test.py:215-219): a captured decode step at ``position``, every
+    earlier row of the caches filled with the prompt's, against the graph's host reference within
+    the reference's KL bound of 0.1 and its 5 % rule.  600 and 2047 replay the graph captured in the
+    one-launch form of attention, 2048 on the one whose attention deals the keys over the chip."""
+    gpu, cpu, tokens, token = deep
+    assert gpu.decode_step.captured and gpu.decode_step._graph_bounded is not None
+    _fill_caches(gpu, cpu, len(tokens), position)
+    got, _ = gpu(token=token, position=position)
+    got = np.array(got.numpy()).ravel()[: gpu.config.vocab_size]
+    want, _ = cpu(token=token, position=position)
+    want = np.asarray(want.numpy()).ravel()[: gpu.config.vocab_size]
+    assert_close(got, want, f"the step at {position}")
+    assert kl(want, got) <= 0.1
+
+
+def test_replays_cross_from_the_bounded_graph_to_the_full_one(deep):
+    """A run of device-carried replays that starts under the one-launch form's limit and ends past it
+    draws what the same steps draw when each is started from the host."""
+    gpu, cpu, tokens, token = deep
+    decode = gpu.decode_step
+    _fill_caches(gpu, cpu, len(tokens), 2040)
+    held = decode.read(gpu.drawn).copy()
+
+    def run(each: bool) -> list[int]:
+        _fill_caches(gpu, cpu, len(tokens), 2040)   # the steps wrote rows 2040..: start alike
+        decode.start(token=token, position=2040)
+        if each:
+            for i in range(1, 16):
+                drawn = int(decode.read(gpu.drawn)[2040 + i - 1])
+                decode.start(token=drawn, position=2040 + i)
+        else:
+            decode.replay(15)
+        return [int(t) for t in decode.read(gpu.drawn)[2040 : 2040 + 16]]
+
+    assert run(each=False) == run(each=True)
+    assert held.shape == decode.read(gpu.drawn).shape
+
+
+def test_prompt_deep_in_the_cache(deep):
+    """The reference's ``check_deep_prompt`` (iron/lm/testing.py:334-364): the chunk that holds position
+    ``max_seq_len - 1``, 512 rows of it, over caches filled up to the chunk's first row."""
+    gpu, cpu, tokens, _ = deep
+    C, L = gpu.config.prefill_chunk, gpu.config.max_seq_len
+    begin, rows = (L - 1) // C * C, 512
+    chunk = np.resize(tokens, rows)
+    values = dict(token=int(chunk[-1]), position=begin + rows - 1, start=begin, rows=rows, rope_start=begin)
+    _fill_caches(gpu, cpu, len(tokens), begin)
+    got, _ = gpu(gpu.session.prompt_ids(chunk), **values)
+    got = np.array(got.numpy()).ravel()[: gpu.config.vocab_size]
+    want, _ = cpu(cpu.session.prompt_ids(chunk), **values)
+    want = np.asarray(want.numpy()).ravel()[: gpu.config.vocab_size]
+    assert_close(got, want, f"the chunk at {begin}")
+    assert kl(want, got) <= 0.1
+
+
+def test_a_5000_token_prompt_in_three_chunks_then_replayed_steps(cuda):
+    """Toy width, caches of 8192 rows: a prompt of three chunks (attention over a cache longer than
+    the chunk), then eight device-carried decode steps past position 5000 (attention's keys dealt
+    over the chip, merged by the second launch, inside the captured step), teacher-checked against
+    the host model token by token."""
+    config = dataclasses.replace(SCALED, max_seq_len=8192, prefill_chunk=2048)
+    gpu, cpu = Llama(config, weights()), HostLlama(dataclasses.replace(config, prefill_chunk=1024), weights())
+    gpu.load_versions()
+    cpu.load_versions()
+    try:
+        tokens = list(np.random.default_rng(23).integers(0, config.vocab_size, 5000))
+        want, got = cpu.logits(tokens), gpu.logits(tokens)
+        assert_close(got, want, "the prompt")
+        assert kl(want, got) < 1e-2
+        drawn = gpu.generate(tokens, 8)
+        for step, token in enumerate(drawn):
+            want = cpu.logits(tokens)
+            assert want[token] >= want.max() - 0.05 * np.abs(want).max(), f"step {step}"
+            tokens.append(token)
+    finally:
+        gpu.release()
+
+
 def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
     """The fused launches compute what the recorded steps compute: same greedy tokens, logits
     within bf16 rounding, and far fewer launches per decode step."""
