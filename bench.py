@@ -385,6 +385,52 @@ def prompt_probe(torch, dev, repeats=20):
                       "ttft_ms_median": round(1e3 * float(np.median(times)), 3)}))
 
 
+def bench_decoder_contexts(torch, dev, steps, warmup, weights, contexts=(8192, 131072)):
+    """The same 512-token prompt + ``steps`` decode steps with the caches compiled for longer contexts
+    (131072 is Llama-3.2-1B's own max_seq_len): what a token costs is to follow the context, not the
+    cache (the reference's "one compile, any context", AGENTS.md:246-255)."""
+    import dataclasses
+
+    from iron_amd.applications.llama import LLAMA_3_2_1B, Llama
+
+    out = []
+    prompt = np.random.default_rng(512).integers(0, LLAMA_3_2_1B.vocab_size, 512)
+    for rows in contexts:
+        config = dataclasses.replace(LLAMA_3_2_1B, max_seq_len=rows, prefill_chunk=2048)
+        model = Llama(config, weights)
+        model.load_versions()
+        decode = model.decode_step
+
+        def prefill():
+            carry = None
+            for inputs, values in model.session.chunk_calls(prompt, 0):
+                _, carry = model(*inputs, **values)
+            return carry
+
+        decode.start(**prefill())
+        decode.replay(max(warmup, 1))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        carry = prefill()
+        torch.cuda.synchronize()
+        ttft = time.perf_counter() - t0
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        decode.start(**carry)
+        decode.replay(steps - 1)
+        stop.record()
+        stop.synchronize()
+        ms = start.elapsed_time(stop)
+        tokens = decode.read(model.drawn)[512 : 512 + steps]
+        out.append({"max_seq_len": rows, "tok_s": round(steps / (ms / 1e3), 1), "ms_per_token": round(ms / steps, 4),
+                    "ttft_ms": round(ttft * 1e3, 2), "launches_per_step": decode.launches_per_replay,
+                    "first_tokens": [int(t) for t in tokens[:4]]})
+        model.release()
+        del model
+        torch.cuda.empty_cache()
+    return out
+
+
 def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
     """Llama-3.2-1B shape: a 512-token prompt prefill, then ``steps`` greedy decode steps as
     replays of the captured decode step (each starts from the token and position the last one
@@ -467,6 +513,12 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
         drawn = decode.read(model.drawn)[511 : 512 + steps]   # the prompt's draw, then each decode step's
         cpu, out["checked"] = cpu_decoder_baseline(torch, config, weights, prompt, prompt_logits, [int(t) for t in drawn])
     model.release()
+    del model
+    torch.cuda.empty_cache()
+    out["max_seq_len"] = config.max_seq_len
+    out["by_max_seq_len"] = [{"max_seq_len": config.max_seq_len, "tok_s": out["tok_s"], "ms_per_token": out["ms_per_token"],
+                              "ttft_ms": out["ttft_ms"], "launches_per_step": out["launches_per_step"],
+                              "first_tokens": out["first_tokens"]}] + bench_decoder_contexts(torch, dev, steps, warmup, weights)
     return out, cpu
 
 
@@ -511,19 +563,56 @@ def cpu_decoder_baseline(torch, config, weights, prompt, gpu_prompt_logits, gpu_
     host_logits = model.logits(prompt)
     prefill_s = time.perf_counter() - t0
     share = judge(host_logits, gpu_prompt_logits, gpu_tokens[0], "the prompt's logits")
-    history, steps, checked = list(map(int, prompt)), 0, 1
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < budget_s and steps + 1 < len(gpu_tokens):
-        history.append(gpu_tokens[steps])
-        row = model.logits(history)
-        steps += 1
-        judge(row, None, gpu_tokens[steps], f"decode step {steps}")
-        checked += 1
-    dt = time.perf_counter() - t0
-    cpu = {"value": round(steps / dt, 3), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+    # Two timed legs over the same steps' worth of budget.  First as the reference's CPU path runs a
+    # GEMV: the weight is held as bf16 storage and widened to float32 on every call (gemv.py:413) --
+    # the oracle's GEMV is handed the weight's bits and widens them; then with the weights held as
+    # float32 (no widening), which is the faster host program and is reported beside it.
+    from iron_amd.bf16 import from_bits, to_bits
+    from iron_amd.common.declare import REFERENCES
+
+    from iron_amd.common.graph import Param, Weight, walk
+
+    # The host reference keeps each weight as one float32 array (``Resident.host``) and hands the GEMV
+    # a view of it: the view's address names the weight whose bits to widen.
+    bits = {x.host.ctypes.data: to_bits(x.host.reshape(x.shape)) for _, x, _, _ in walk(model)
+            if isinstance(x, (Param, Weight)) and len(x.shape) == 2 and getattr(x, "host", None) is not None}
+    plain_gemv = REFERENCES["GEMV"]
+    widened = [0]
+
+    def widening_gemv(op, A, B):
+        held = bits.get(np.asarray(A).ctypes.data)
+        if held is None:
+            return plain_gemv(op, A, B)
+        widened[0] += 1
+        return plain_gemv(op, from_bits(held), B)
+
+    history, checked, legs = list(map(int, prompt)), 1, {}
+    at = 0
+    for leg, gemv in (("widened", widening_gemv), ("float32", plain_gemv)):
+        REFERENCES["GEMV"] = gemv
+        steps = 0
+        t0 = time.perf_counter()
+        try:
+            while time.perf_counter() - t0 < budget_s / 2 and at + 1 < len(gpu_tokens):
+                history.append(gpu_tokens[at])
+                row = model.logits(history)
+                at += 1
+                steps += 1
+                judge(row, None, gpu_tokens[at], f"decode step {at}")
+                checked += 1
+        finally:
+            REFERENCES["GEMV"] = plain_gemv
+        legs[leg] = (steps, time.perf_counter() - t0)
+    steps, dt = legs["widened"]
+    plain_steps, plain_dt = legs["float32"]
+    assert steps == 0 or widened[0] >= steps * (7 * config.num_hidden_layers + 1), "the widening leg widened nothing"
+    cpu = {"value": round(steps / dt, 3) if steps else None, "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+           "value_float32_weights": round(plain_steps / plain_dt, 3) if plain_steps else None,
            "sample": f"{steps} decode steps after the same 512-token prompt (prefilled on the host in {prefill_s:.1f} s) "
                      f"of the same 16-layer model through the oracle's graph reference, teacher-forced on the GPU's "
-                     f"tokens, {dt:.1f} s wall; weights held as float32 (the reference widens bf16 on every call)"}
+                     f"tokens, {dt:.1f} s wall, every weight widened from bf16 storage on every call as the reference's "
+                     f"GEMV does (gemv.py:413); value_float32_weights: the next {plain_steps} steps with the weights held "
+                     f"as float32, {plain_dt:.1f} s wall"}
     return cpu, {"rule": "within 5 % of the largest logit; same argmax where the top two are apart; each GPU token a best "
                          "one of the host's logits", "prompt_logits_max_diff_share": share, "tokens_checked": checked}
 
@@ -532,6 +621,9 @@ PROBE_COPY_BYTES = 512 << 20
 # HBM bytes one launch moves, by kernel, from hardware counters (FETCH_SIZE and WRITE_SIZE per
 # dispatch, each scaled by what the same counter reads for a plain copy of PROBE_COPY_BYTES): filled
 # from counter runs of `--decode-probe` / `--counter-probe`; a kernel without a reading reports null.
+DOMINANT_TRAFFIC_SOURCE = ("profiles/llama1b_decode_step_hbm_counters.txt (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, over "
+                           "`bench.py --decode-probe 8`; the kernels' template arguments as of that run: a kernel whose "
+                           "arguments have changed since finds no entry and reports null)")
 DOMINANT_TRAFFIC_BYTES: dict[str, int] = {
     "gemv_fused_kernel<2,1,true,2>": 67_358_000,     # norm + gate/up + SiLU*mul: 67.227 MB fetched + 0.131 written
     "gemv_fused_kernel<1,4,false,1>": 33_788_000,    # down projection + residual: 33.755 + 0.033
@@ -714,9 +806,7 @@ def main():
                      "achieved": dominant["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dominant["frac_hbm"],
                      "us": dominant["us"], "algorithmic_bytes": dominant["bytes"],
                      "traffic": DOMINANT_TRAFFIC_BYTES.get(dominant["kernel"]),
-                     "traffic_source": "a separate rocprofv3 --pmc run of `bench.py --decode-probe` (FETCH_SIZE + "
-                                       "WRITE_SIZE per dispatch, scaled by the same counters over a copy of known size); "
-                                       "not measured in this run"},
+                     "traffic_source": DOMINANT_TRAFFIC_SOURCE + "; not measured in this run"},
         "decode_step_kernels": decode_kernels,
         "decoder": decoder,
         "gemv_sweep": {"GBps": round(sweep_bytes / sweep_us / 1e3, 1), "shapes": gemv},

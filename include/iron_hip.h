@@ -242,7 +242,9 @@ int iron_mha_decode_tuned_bf16(const uint16_t* Q, const uint16_t* K, const uint1
  * bytes on each GPU it runs on, until the process ends), so no workspace is passed and nothing is
  * allocated or freed.  Refused (1) when iron_mha_decode_workspace_bytes(heads, d) exceeds that size.
  * Every call on a GPU shares that GPU's array: calls that overlap on one GPU race.  Nothing in it
- * has to start at zero.  No counterpart in the reference. */
+ * has to start at zero.  The first call on a device asks the runtime for the array's address there
+ * (hipGetSymbolAddress, which may load the code object): make one call per device outside any stream
+ * capture before recording calls into a graph.  No counterpart in the reference. */
 int iron_mha_decode_static_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,
                                 int heads, int kv_heads, int d, int kv_len, float scale, int window,
                                 int kv_interleaved, const int* kv_valid, void* stream);

@@ -424,8 +424,9 @@ __global__ __launch_bounds__(64 * WAVES) void mha_decode_either_kernel(
   const bf16_t* Kh = K + (size_t)kvh * head_stride + first_row * row_stride;
   const bf16_t* Vh = V + (size_t)kvh * head_stride + first_row * row_stride;
   const int row_bytes = (int)row_stride * 2;
-  // The head's keys (values) up to the last live one are one buffer: rows past it read as zeros.
-  const int reach = (kv_tokens - 1) * row_bytes + ROWB;
+  // The head's keys (values) up to the last of this wave's run are one buffer: rows past it -- the
+  // next wave's, or past the last live key -- read as zeros and cost no traffic.
+  const int reach = wlo < whi ? (whi - 1) * row_bytes + ROWB : 0;
   const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(Kh), 0, reach, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(Vh), 0, reach, 0x00020000);
 

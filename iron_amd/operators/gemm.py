@@ -41,7 +41,8 @@ def _cases(cls, dev=None):
 
 
 class GEMM(Operator):
-    """``C = A @ B``, tiled 128 x 128 x 64 over the CUs, 32x32x16 MFMA tiles per wave."""
+    """``C = A @ B`` on 16x16x32 bf16 MFMAs, float32 sums, one rounding: 256 x 256, 128 x 128 or 64 x 64
+    tiles by the shape (and, under a per-call row bound, by the bound, chosen on the device)."""
 
     test = Testing(_cases, draw=lambda op: dict(normal=(op.A,)))
 

@@ -50,3 +50,44 @@ def test_decode_attention_from_the_library_s_own_scratch_is_the_workspace_one_bi
     Q, Kc, Vc = bf(1, H, d), bf(64, H, d), bf(64, H, d)
     with pytest.raises(IronHipError, match="scratch holds"):
         K.mha_decode_static(Q, Kc, Vc, torch.empty_like(Q), heads=H, kv_heads=H, d=d, kv_len=64, kv_interleaved=True)
+
+
+def test_static_decode_attention_under_graph_capture_after_one_warm_call(cuda):
+    """What the entry point is for: once a call outside any capture has made the library look its
+    scratch array's address up on this device, the call records into a HIP graph (it allocates
+    nothing and asks the runtime nothing), and every replay is the workspace form bit for bit --
+    replayed several times with eager work and synchronizations in between, new keys each time."""
+    g = torch.Generator(device=cuda)
+    g.manual_seed(6)
+
+    def bf(*shape):
+        return torch.randn(shape, generator=g, device=cuda, dtype=torch.float32).to(torch.bfloat16)
+
+    H, G, d, L = 32, 8, 64, 6000
+    Q, Kc, Vc = bf(1, H, d), bf(L, G, d), bf(L, G, d)
+    kv_valid = torch.tensor([5000], dtype=torch.int32, device=cuda)
+    own = torch.zeros((1, H, d), dtype=torch.bfloat16, device=cuda)
+
+    def launch():
+        K.mha_decode_static(Q, Kc, Vc, own, heads=H, kv_heads=G, d=d, kv_len=L, kv_interleaved=True, kv_valid=kv_valid)
+
+    launch()   # the warm call
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            launch()
+    torch.cuda.current_stream().wait_stream(stream)
+    ws = K.mha_decode_workspace(H, d, cuda)
+    for bound in (5000, 900, 6000, 2049):
+        Kc.copy_(bf(L, G, d))
+        kv_valid.fill_(bound)
+        own.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = torch.empty_like(own)
+        K.mha_decode(Q, Kc, Vc, want, heads=H, kv_heads=G, d=d, kv_len=L, kv_interleaved=True, kv_valid=kv_valid,
+                     workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(own, want), bound
