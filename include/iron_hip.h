@@ -63,6 +63,14 @@ int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t
  * (iron/lm/blocks.py:688,697-699), rounding where they round. */
 int iron_gemm_gated_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* G, uint16_t* C, int M,
                          int N, int K, int activation, const int* valid, void* stream);
+/* Both first projections of a gated feed-forward and the gate in one launch:
+ * G = bf16(A Bg^T), C = bf16(bf16(act(G)) * bf16(A Bu^T)) for the rows under *valid (or M) -- what
+ * iron_gemm_bf16 (gate_proj) followed by iron_gemm_gated_bf16 (up_proj) compute, bit for bit; a block
+ * reads back only the tile of G it wrote itself.  A (M,K); Bg, Bu (N,K); G, C (M,N), distinct.
+ * Replaces GEMM, GEMM, SiLU or GELU, ElementwiseMul (iron/lm/blocks.py:688,697-699). */
+int iron_gemm_gated_pair_bf16(const uint16_t* A, const uint16_t* Bg, const uint16_t* Bu, uint16_t* G,
+                              uint16_t* C, int M, int N, int K, int activation, const int* valid,
+                              void* stream);
 
 /* One-row fusions of a decoder layer (no single counterpart in the reference: each replaces a run
  * of its steps, iron/lm/blocks.py:627-648,697-699,723-733, and rounds where those steps round).

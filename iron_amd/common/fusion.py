@@ -16,6 +16,7 @@ in a prompt chunk's version (several rows, 64-wide heads),
 
   GEMM q/k/v (one input), RoPE q/k                       => iron_prefill_qkv_bf16
   ... and Copy k/v -> the chunk's cache rows             => iron_prefill_qkv_cache_bf16
+  GEMM (gate), GEMM (up), SiLU or GELU (tanh), Mul       => iron_gemm_gated_pair_bf16
   GEMM (up), SiLU or GELU (tanh) of the gate, Mul        => iron_gemm_gated_bf16
   SiLU, ElementwiseMul (no such product before them)     => iron_silu_mul_bf16
   GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
@@ -113,6 +114,48 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
         ok = (_name(s) == "GEMV" and s.op.num_batches is None and not s.values
               and all(_plain(h) for h in (*s.inputs.values(), *s.outputs.values())))
         return ok and (x is None or _same(s.inputs["B"], x))
+
+    def gated_at(j, before=None):
+        """``(args, kw)`` of ``iron_gemm_gated_bf16`` where steps j, j + 1, j + 2 are a many-row product, the
+        activation of an earlier product of the same shape (the gate) and their Mul, or None.  With
+        ``before``, the step right ahead of them must be the product that made the gate, of the same
+        rows by the same bound and read by the activation alone."""
+        if j + 2 >= len(steps):
+            return None
+        s, sl, ml = steps[j], steps[j + 1], steps[j + 2]
+        if not (_name(s) == "GEMM"
+                and (_name(sl) == "SiLU" or (_name(sl) == "GELU" and sl.op.approximate == "tanh"))
+                and _name(ml) == "ElementwiseMul"
+                and s.op.b_col_maj and not s.op.c_col_maj and "valid_k" not in s.values
+                and s.op.M >= 64 and s.op.N >= 64 and s.op.K % 64 == 0):
+            return None
+        up, gate, act = s.outputs["C"], sl.inputs["x"], sl.outputs["y"]
+        a, b = ml.inputs["a"], ml.inputs["b"]
+        paired = (_same_view(a, act) and _same_view(b, up)) or (_same_view(a, up) and _same_view(b, act))
+        gv, sv, mv = s.values.get("valid"), sl.values.get("valid"), ml.values.get("valid")
+        # the elementwise bounds count elements, the product's rows
+        bounds_agree = sv == mv and ((gv is None and sv is None) or (
+            gv is not None and sv is not None and gv.value == sv.value and gv.linear and sv.linear
+            and sv.scale == gv.scale * s.op.N and sv.bias == gv.bias * s.op.N))
+        flat = all(h.index is None and h.ids is None
+                   for h in (*s.inputs.values(), up, gate, act, a, b, ml.outputs["y"]))
+        if not (paired and flat and once(up) and once(act) and bounds_agree and gate.buffer is not up.buffer
+                and gate.elements == up.elements and sl.op.size == up.elements and ml.op.size == up.elements
+                and ml.outputs["y"].elements == up.elements
+                and set(sl.values) <= {"valid"} and set(ml.values) <= {"valid"}):
+            return None
+        if before is not None:
+            g = before
+            if not (_name(g) == "GEMM" and g.op.b_col_maj and not g.op.c_col_maj and "valid_k" not in g.values
+                    and (g.op.M, g.op.N, g.op.K) == (s.op.M, s.op.N, s.op.K) and g.values.get("valid") == gv
+                    and _same_view(g.inputs["A"], s.inputs["A"]) and _same_view(g.outputs["C"], gate) and once(gate)
+                    and gate.buffer is not ml.outputs["y"].buffer
+                    and all(h.index is None and h.ids is None for h in (*g.inputs.values(), g.outputs["C"]))):
+                return None
+        args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), G=tensor(gate), C=tensor(ml.outputs["y"]))
+        kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, valid=word(gv),
+                  activation="silu" if _name(sl) == "SiLU" else "gelu_tanh")
+        return args, kw
 
     fused: list[Fused] = []
     # decode_qkv launches whose RoPE row is a copy of one table row: (producing step, args, kw)
@@ -259,32 +302,16 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), R=tensor(other), C=tensor(ad.outputs["y"]))
                 kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, residual_scale=scale, valid=word(gv))
                 got = Fused("gemm_add", i, 2, lambda a=args, kw=kw: kernels.gemm_residual(**a, **kw))
-        elif (_name(s) == "GEMM" and i + 2 < len(steps)
-              and (_name(steps[i + 1]) == "SiLU"
-                   or (_name(steps[i + 1]) == "GELU" and steps[i + 1].op.approximate == "tanh"))
-              and _name(steps[i + 2]) == "ElementwiseMul"
-              and s.op.b_col_maj and not s.op.c_col_maj and "valid_k" not in s.values
-              and s.op.M >= 64 and s.op.N >= 64 and s.op.K % 64 == 0):
+        elif _name(s) == "GEMM" and (gated := gated_at(i + 1, s)) is not None:
+            # a gated feed-forward's two first projections over many rows: one launch computes both
+            # products tile by tile, the activated gate riding the second one's epilogue
+            args, kw = gated
+            args = dict(A=args["A"], Bg=tensor(s.inputs["B"]), Bu=args["B"], G=args["G"], C=args["C"])
+            got = Fused("gemm_gated_pair", i, 4, lambda a=args, kw=kw: kernels.gemm_gated_pair(**a, **kw))
+        elif _name(s) == "GEMM" and (gated := gated_at(i)) is not None:
             # a gated feed-forward's second projection over many rows: the activated gate rides its epilogue
-            sl, ml = steps[i + 1], steps[i + 2]
-            up, gate, act = s.outputs["C"], sl.inputs["x"], sl.outputs["y"]
-            a, b = ml.inputs["a"], ml.inputs["b"]
-            paired = (_same_view(a, act) and _same_view(b, up)) or (_same_view(a, up) and _same_view(b, act))
-            gv, sv, mv = s.values.get("valid"), sl.values.get("valid"), ml.values.get("valid")
-            # the elementwise bounds count elements, the product's rows
-            bounds_agree = sv == mv and ((gv is None and sv is None) or (
-                gv is not None and sv is not None and gv.value == sv.value and gv.linear and sv.linear
-                and sv.scale == gv.scale * s.op.N and sv.bias == gv.bias * s.op.N))
-            flat = all(h.index is None and h.ids is None
-                       for h in (*s.inputs.values(), up, gate, act, a, b, ml.outputs["y"]))
-            if (paired and flat and once(up) and once(act) and bounds_agree and gate.buffer is not up.buffer
-                    and gate.elements == up.elements and sl.op.size == up.elements and ml.op.size == up.elements
-                    and ml.outputs["y"].elements == up.elements
-                    and set(sl.values) <= {"valid"} and set(ml.values) <= {"valid"}):
-                args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), G=tensor(gate), C=tensor(ml.outputs["y"]))
-                kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, valid=word(gv),
-                          activation="silu" if _name(sl) == "SiLU" else "gelu_tanh")
-                got = Fused("gemm_gated", i, 3, lambda a=args, kw=kw: kernels.gemm_gated(**a, **kw))
+            args, kw = gated
+            got = Fused("gemm_gated", i, 3, lambda a=args, kw=kw: kernels.gemm_gated(**a, **kw))
         elif _name(s) == "SiLU" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseMul":
             # a gated feed-forward's activation and gate over many rows: one pass instead of two
             m = steps[i + 1]

@@ -92,7 +92,9 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 
 // SiLU, and GELU by its tanh form, as every kernel here computes them, so that fused and separate
 // launches round alike.
-__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
+// (the quotient by the hardware's reciprocal, an ulp off the division's: a gated GEMM's epilogue runs
+// this 64 times a thread with nothing left to hide it under)
+__device__ __forceinline__ float silu_f32(float v) { return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
 __device__ __forceinline__ float gelu_tanh_f32(float v) {
   const float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
   return 0.5f * v * (1.0f + tanhf(inner));

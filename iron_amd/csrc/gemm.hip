@@ -1474,6 +1474,60 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   IRON_LAUNCH_CHECK();
 }
 
+// A gated feed-forward's two first projections over many rows as ONE launch: a block computes its
+// tile of the gate's product and stores it (rounded, as the separate product stores it), then
+// computes the same tile of the second product, whose epilogue reads the gate tile back -- the one
+// this very block wrote, so nothing crosses between blocks -- and leaves bf16(bf16(act(g)) * bf16(u)).
+// What goes is a launch boundary: the second launch's start, its first stages' fill and the first
+// one's drain.  The tile size is chosen on the device by the row bound as in gemm_either_kernel.
+__global__ __launch_bounds__(256) void gemm_gated_pair_kernel(const bf16_t* __restrict__ A,
+                                                              const bf16_t* __restrict__ Bg,
+                                                              const bf16_t* __restrict__ Bu, bf16_t* __restrict__ G,
+                                                              bf16_t* __restrict__ C, int M, int N, int K,
+                                                              const int* __restrict__ valid, Tiling t128, Tiling t64,
+                                                              int few128, int activation) {
+  const int Mv = bound_or(valid, M), bid = blockIdx.x;
+  QkvTail none{}, gate{};
+  gate.residual = G;
+  gate.gated = activation;
+  if (Mv > few128) {
+    if (bid >= t128.tiles_m * t128.tiles_n) return;
+    gemm_nt16_body<false>(A, Bg, G, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, none);
+    __syncthreads();   // the gate tile's stores are acknowledged, and every wave is done with the stage buffers
+    gemm_nt16_body<false>(A, Bu, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, gate);
+  } else {
+    if (bid >= t64.tiles_m * t64.tiles_n) return;
+    gemm_nt64_body<8>(A, Bg, G, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, none);
+    __syncthreads();
+    gemm_nt64_body<8>(A, Bu, C, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, gate);
+  }
+}
+
+static int launch_gemm_gated_pair(const bf16_t* A, const bf16_t* Bg, const bf16_t* Bu, bf16_t* G, bf16_t* C, int M,
+                                  int N, int K, const int* valid, int activation, hipStream_t s) {
+  const int n128 = (N + 127) / 128, n64 = (N + 63) / 64;
+  // 64 x 64 tiles up to the rows below which 128 x 128 ones would leave half the CUs idle (as iron_gemm_bf16).
+  int few128 = n128 >= 128 ? 0 : 128 * (127 / n128);
+  if (few128 > M) few128 = M;
+  auto tiling = [](int tile_rows, int tile_cols) {
+    const int whole = (tile_rows + 7) & ~7;
+    if (tile_rows >= 8 && !patched_order(tile_rows, tile_cols) && patched_order(whole, tile_cols)) tile_rows = whole;
+    return Tiling{tile_rows, tile_cols, patched_order(tile_rows, tile_cols)};
+  };
+  const Tiling t128 = tiling((M + 127) / 128, n128), t64 = tiling((few128 + 63) / 64, n64);
+  constexpr size_t lds = (size_t)NT_STAGES * 256 * BK * 2;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_gated_pair_kernel), lds); e != hipSuccess) {
+    set_error("gemm_gated_pair: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  int blocks = t128.tiles_m * t128.tiles_n;
+  if (t64.tiles_m * t64.tiles_n > blocks) blocks = t64.tiles_m * t64.tiles_n;
+  hipLaunchKernelGGL(gemm_gated_pair_kernel, dim3(blocks), dim3(256), lds, s, A, Bg, Bu, G, C, M, N, K, valid, t128, t64,
+                     few128, activation);
+  IRON_LAUNCH_CHECK();
+}
+
 template <bool B_KN = false>
 static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
                              const int* valid, hipStream_t s) {
@@ -1583,6 +1637,22 @@ extern "C" int iron_gemm_gated_bf16(const uint16_t* A, const uint16_t* B, const 
   tail.residual = G;
   tail.gated = activation;
   return gemm_with_tail("gemm_gated", A, B, G, C, M, N, K, tail, valid, stream);
+}
+
+extern "C" int iron_gemm_gated_pair_bf16(const uint16_t* A, const uint16_t* Bg, const uint16_t* Bu, uint16_t* G,
+                                         uint16_t* C, int M, int N, int K, int activation, const int* valid,
+                                         void* stream) {
+  IRON_REQUIRE(A && Bg && Bu && G && C, "gemm_gated_pair: null operand");
+  IRON_REQUIRE(activation == 1 || activation == 2, "gemm_gated_pair: activation (%d) is 1 (SiLU) or 2 (GELU, tanh form)",
+               activation);
+  IRON_REQUIRE(G != C, "gemm_gated_pair: the gate's product and the output are different buffers");
+  IRON_REQUIRE(K <= (1 << 22) && N <= (1 << 22),
+               "gemm_gated_pair: K (%d) and N (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", K, N);
+  IRON_REQUIRE(M >= 64 && N >= 64 && K > 0 && K % BK == 0,
+               "gemm_gated_pair: M (%d) and N (%d) at least 64, K (%d) a positive multiple of %d", M, N, K, BK);
+  IRON_REQUIRE((((uintptr_t)A | (uintptr_t)Bg | (uintptr_t)Bu | (uintptr_t)G | (uintptr_t)C) & 15) == 0,
+               "gemm_gated_pair: operands must be 16-byte aligned");
+  return launch_gemm_gated_pair(A, Bg, Bu, G, C, M, N, K, valid, activation, (hipStream_t)stream);
 }
 
 static int prefill_qkv(const uint16_t* x, const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,

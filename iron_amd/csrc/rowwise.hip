@@ -16,26 +16,36 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__
                                                       float eps, const int* __restrict__ valid,
                                                       const bf16_t* residual) {
   const int row = blockIdx.x;
-  if (row >= bound_or(valid, rows)) return;
   const int nchunk = cols >> 3;
+  const uint4* wr = reinterpret_cast<const uint4*>(w);
+  // The gains do not depend on the row or on the bound: their trip to memory goes out with the
+  // bound's own instead of after the row's sum (three dependent trips a launch were two too many).
+  uint4 gains[CHUNKS];
+#pragma unroll
+  for (int i = 0; i < CHUNKS; ++i) {
+    const int c = threadIdx.x + i * 256;
+    gains[i] = (w != nullptr && c < nchunk) ? wr[c] : make_uint4(0, 0, 0, 0);
+  }
+  if (row >= bound_or(valid, rows)) return;
   const uint4* xr = reinterpret_cast<const uint4*>(x + (size_t)row * cols);
   uint4* yr = reinterpret_cast<uint4*>(y + (size_t)row * cols);
-  const uint4* wr = reinterpret_cast<const uint4*>(w);
   // A residual (which y may be) the normed row is added to, rounded as the separate sum rounds.
   const uint4* rr = reinterpret_cast<const uint4*>(residual + (residual ? (size_t)row * cols : 0));
 
-  uint4 held[CHUNKS];
+  uint4 held[CHUNKS], added[CHUNKS];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < CHUNKS; ++i) {
-    int c = threadIdx.x + i * 256;
-    if (c < nchunk) {
-      held[i] = xr[c];
-      float f[8];
-      unpack8(held[i], f);
+    const int c = threadIdx.x + i * 256;
+    held[i] = c < nchunk ? xr[c] : make_uint4(0, 0, 0, 0);
+    added[i] = (residual != nullptr && c < nchunk) ? rr[c] : make_uint4(0, 0, 0, 0);
+  }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
-    }
+  for (int i = 0; i < CHUNKS; ++i) {
+    float f[8];
+    unpack8(held[i], f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
   }
   // Rows longer than CHUNKS*2048 elements: the rest is summed here and re-read below.
   for (int c = threadIdx.x + CHUNKS * 256; c < nchunk; c += 256) {
@@ -51,12 +61,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__
   const float total = part[0] + part[1] + part[2] + part[3];
   const float inv = 1.0f / sqrtf(total / (float)cols + eps);
 
-  auto emit = [&](int c, const uint4& v) {
+  auto emit = [&](int c, const uint4& v, const uint4& gain, const uint4& add) {
     float f[8];
     unpack8(v, f);
     if (w != nullptr) {
       float g[8];
-      unpack8(wr[c], g);
+      unpack8(gain, g);
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[j] = round_bf16(f[j] * inv) * g[j];
     } else {
@@ -65,7 +75,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__
     }
     if (residual != nullptr) {
       float r[8];
-      unpack8(rr[c], r);
+      unpack8(add, r);
 #pragma unroll
       for (int j = 0; j < 8; ++j) f[j] = r[j] + round_bf16(f[j]);
     }
@@ -74,9 +84,10 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* __restrict__
 #pragma unroll
   for (int i = 0; i < CHUNKS; ++i) {
     int c = threadIdx.x + i * 256;
-    if (c < nchunk) emit(c, held[i]);
+    if (c < nchunk) emit(c, held[i], gains[i], added[i]);
   }
-  for (int c = threadIdx.x + CHUNKS * 256; c < nchunk; c += 256) emit(c, xr[c]);
+  for (int c = threadIdx.x + CHUNKS * 256; c < nchunk; c += 256)
+    emit(c, xr[c], w != nullptr ? wr[c] : make_uint4(0, 0, 0, 0), residual != nullptr ? rr[c] : make_uint4(0, 0, 0, 0));
 }
 
 // ------------------------------------------------------------------- RoPE

@@ -93,6 +93,20 @@ def gemm_gated(A, B, G, C, *, M, N, K, activation="silu", valid=None):
                                      ptr(_word(valid, "valid")), current_stream()), "iron_gemm_gated_bf16")
 
 
+def gemm_gated_pair(A, Bg, Bu, G, C, *, M, N, K, activation="silu", valid=None):
+    """``G = A @ Bg.T``, ``C = act(G) * (A @ Bu.T)`` over many rows in one launch (weights ``(N, K)``)."""
+    kinds = {"silu": 1, "gelu_tanh": 2}
+    if activation not in kinds:
+        raise ValueError(f"gemm_gated_pair: activation {activation!r} is neither 'silu' nor 'gelu_tanh'")
+    _numel(_dev(A, "A"), M * K, "A")
+    _numel(_dev(Bg, "Bg"), N * K, "Bg")
+    _numel(_dev(Bu, "Bu"), N * K, "Bu")
+    _numel(_dev(G, "G"), M * N, "G")
+    _numel(_dev(C, "C"), M * N, "C")
+    check(lib().iron_gemm_gated_pair_bf16(ptr(A), ptr(Bg), ptr(Bu), ptr(G), ptr(C), M, N, K, kinds[activation],
+                                          ptr(_word(valid, "valid")), current_stream()), "iron_gemm_gated_pair_bf16")
+
+
 def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, residual_scale=1.0, epilogue=0):
     """One-row fusion: ``[RMSNorm ->] GEMV [-> + residual | gate/up -> SiLU -> Mul]``."""
     _numel(_dev(W, "W"), M * K, "W")

@@ -371,6 +371,32 @@ def test_gemm_gated_epilogue(cuda, M, Kdim, N, rows, activation):
     assert torch.equal(Gd[:lim], C[:lim])
 
 
+@pytest.mark.parametrize("M,Kdim,N,rows", [(2048, 2048, 8192, 512), (2048, 2048, 8192, 1281), (2048, 2048, 8192, 100),
+                                           (256, 512, 1024, None), (192, 128, 320, 70)])
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+def test_gemm_gated_pair_is_the_two_launches_bit_for_bit(cuda, M, Kdim, N, rows, activation):
+    """Both first projections of a gated feed-forward in one launch: the gate's product and the gated
+    output against the two launches they replace (the gate's GEMM, then the gated GEMM) bit for bit --
+    under row bounds that pick the 128 x 128 tiles, the 64 x 64 ones and neither whole -- and the gate's
+    product against the oracle's GEMM; rows past the bound are left as they were.  The first case is
+    Llama-3.2-1B's prompt chunk."""
+    rng = np.random.default_rng(M + N + 3)
+    A, Bg, Bu = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.05), bf(rng, N, Kdim, scale=0.05)
+    lim = M if rows is None else rows
+    if rows is not None:
+        A[rows:] = np.nan
+    bound = None if rows is None else word(rows, cuda)
+    dA, dBg, dBu = dev(A, cuda), dev(Bg, cuda), dev(Bu, cuda)
+    G2, C2 = out_like((M, N), cuda, fill=7.0), out_like((M, N), cuda, fill=7.0)
+    K.gemm(dA, dBg, G2, M=M, N=N, K=Kdim, b_col_maj=True, valid=bound)
+    K.gemm_gated(dA, dBu, G2, C2, M=M, N=N, K=Kdim, activation=activation, valid=bound)
+    G1, C1 = out_like((M, N), cuda, fill=7.0), out_like((M, N), cuda, fill=7.0)
+    K.gemm_gated_pair(dA, dBg, dBu, G1, C1, M=M, N=N, K=Kdim, activation=activation, valid=bound)
+    close(G1[:lim], ops.gemm(A[:lim], Bg, b_col_maj=True), rtol=1e-2, atol=1e-2)
+    assert torch.equal(G1[:lim], G2[:lim]) and torch.equal(C1[:lim], C2[:lim])
+    assert np.all(from_torch(C1)[lim:] == 7.0) and np.all(from_torch(G1)[lim:] == 7.0)
+
+
 @pytest.mark.parametrize("bound", [None, 512, 1281])
 @pytest.mark.parametrize("cache", [False, True])
 def test_prefill_qkv_at_the_decoder_s_width(cuda, bound, cache):

@@ -501,11 +501,11 @@ def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
     assert fused.decode_step.launches_per_replay == fused.decode_step.launches_per_call
     assert plain.decode_step.launches_per_replay == steps
     # the prompt chunk: per layer the three projections, two rotations and two cache writes become
-    # one launch, the feed-forward's SiLU and Mul ride its second projection's epilogue, each residual
-    # sum its projection's, and the last row's final norm and head are one
+    # one launch, the feed-forward's two first projections, SiLU and Mul another, each residual
+    # sum rides its projection's epilogue, and the last row's final norm and head are one
     psteps = len(fused.prompt_chunk.recording.steps)
     assert plain.prompt_chunk.launches_per_call == psteps
-    assert fused.prompt_chunk.launches_per_call == psteps - 10 * SCALED.num_hidden_layers - 1
+    assert fused.prompt_chunk.launches_per_call == psteps - 11 * SCALED.num_hidden_layers - 1
     prompt = np.random.default_rng(7).integers(0, SCALED.vocab_size, 8)
     a, b = fused.logits(prompt), plain.logits(prompt)
     assert np.abs(a - b).max() <= 0.02 * np.abs(b).max()
