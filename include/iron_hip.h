@@ -96,6 +96,15 @@ int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, float eps, c
                          uint16_t* q_out, uint16_t* keys, uint16_t* values, int hidden, int heads,
                          int kv_heads, int d, int cache_rows, const int* position, const int* angle_row,
                          int angle_rows, void* stream);
+/* The same for a decoder's first layer, whose input is the token's row of the embedding table
+ * (table_rows, hidden): the row is read at table[*token] (held inside the table), and also written to
+ * x (hidden), which the layer's residual sum reads -- the step's embedding lookup
+ * (iron/lm/blocks.py:349-383, iron/lm/causal.py:292-299) then needs no launch of its own. */
+int iron_decode_qkv_embed_bf16(const uint16_t* table, const int* token, int table_rows, uint16_t* x,
+                               const uint16_t* norm_w, float eps, const uint16_t* Wq, const uint16_t* Wk,
+                               const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out, uint16_t* keys,
+                               uint16_t* values, int hidden, int heads, int kv_heads, int d, int cache_rows,
+                               const int* position, const int* angle_row, int angle_rows, void* stream);
 
 /* A prompt chunk's three projections and the rotation of q and k in one launch (no single
  * counterpart in the reference: replaces 3 GEMM and 2 RoPE steps, iron/lm/blocks.py:617-648, and

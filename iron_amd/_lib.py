@@ -28,6 +28,10 @@ SIGNATURES = {
         c_int,
         [_P, _P, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P, c_int, _P],
     ),
+    "iron_decode_qkv_embed_bf16": (
+        c_int,
+        [_P, _P, c_int, _P, _P, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P, c_int, _P],
+    ),
     "iron_gemm_gated_pair_bf16": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "iron_prefill_qkv_bf16": (c_int, [_P] * 8 + [c_int] * 5 + [_P, _P]),
     "iron_prefill_qkv_cache_bf16": (c_int, [_P] * 8 + [c_int] * 6 + [_P, _P, _P]),

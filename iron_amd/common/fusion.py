@@ -160,6 +160,8 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
     fused: list[Fused] = []
     # decode_qkv launches whose RoPE row is a copy of one table row: (producing step, args, kw)
     rope_rows: list[tuple[int, dict, dict]] = []
+    # decode_qkv launches whose input row is a copy of one row of a table (the token's embedding)
+    embed_rows: list[tuple[int, dict, dict]] = []
     i = 0
     while i < len(steps):
         s = steps[i]
@@ -203,6 +205,11 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                     made_by = _row_copy(steps, i, rq.inputs["angles"], d)
                     if made_by is not None:
                         rope_rows.append((made_by, args, kw))
+                    # ... and the layer's input where it is one row of an embedding table
+                    looked_up = _row_copy(steps, i, s.inputs["x"], s.op.tile_size)
+                    if looked_up is not None and not any(
+                            h.buffer is s.inputs["x"].buffer for t in steps[looked_up + 1 : i] for h in t.inputs.values()):
+                        embed_rows.append((looked_up, args, kw))
             # the gated MLP's first half
             if (got is None and len(rest) >= 4 and gemv_row(rest[0], n) and gemv_row(rest[1], n) and once(n, 2)
                     and (_name(rest[2]) == "SiLU" or (_name(rest[2]) == "GELU" and rest[2].op.approximate == "tanh"))
@@ -376,6 +383,15 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
             a["angles"] = tensor(table).reshape(-1)[: table.index_rows * table.index_stride]
             kw["angle_row"] = word(table.index)
         fused.append(Fused("elided_rope_row", producer, 1, lambda: None, launches=0))
+    # The token's embedding row, copied out of its table for a first layer whose fused projections can
+    # read the table at the token themselves (and leave the copy where the residual sum reads it).
+    for producer, a, kw in embed_rows:
+        if any(f.first <= producer < f.first + f.count for f in fused):
+            continue
+        table = steps[producer].inputs["src"]
+        a["table"] = tensor(table).reshape(-1)[: table.index_rows * table.index_stride]
+        kw["token"] = word(table.index)
+        fused.append(Fused("elided_embedding_row", producer, 1, lambda: None, launches=0))
     return sorted(fused, key=lambda f: f.first)
 
 

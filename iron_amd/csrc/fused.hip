@@ -34,12 +34,25 @@ template <int CH, bool NORM>
 struct Activation {
   uint4 xv[CH], gv[CH];
   __device__ __forceinline__ void issue(const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw, int K) {
+    issue_gains(nw, K);
+    issue_row(x, K);
+  }
+  // ... or apart, where the row's address is itself on its way from memory: the gains (and the
+  // caller's weights) go out first and the row's loads once the address is in.
+  __device__ __forceinline__ void issue_gains(const bf16_t* __restrict__ nw, int K) {
+    const int chunks = K >> 3;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (NORM) gv[i] = c < chunks ? reinterpret_cast<const uint4*>(nw)[c] : make_uint4(0, 0, 0, 0);
+    }
+  }
+  __device__ __forceinline__ void issue_row(const bf16_t* __restrict__ x, int K) {
     const int chunks = K >> 3;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int c = threadIdx.x + 256 * i;
       xv[i] = c < chunks ? reinterpret_cast<const uint4*>(x)[c] : make_uint4(0, 0, 0, 0);
-      if (NORM) gv[i] = c < chunks ? reinterpret_cast<const uint4*>(nw)[c] : make_uint4(0, 0, 0, 0);
     }
   }
   // With NORM the block sums the squares together (one barrier).
@@ -151,7 +164,8 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
     const bf16_t* __restrict__ Wq, const bf16_t* __restrict__ Wk, const bf16_t* __restrict__ Wv,
     const bf16_t* __restrict__ angles, bf16_t* __restrict__ q_out, bf16_t* __restrict__ keys,
     bf16_t* __restrict__ values, int K, int heads, int kv_heads, int cache_rows,
-    const int* __restrict__ position, const int* __restrict__ angle_row, int angle_rows) {
+    const int* __restrict__ position, const int* __restrict__ angle_row, int angle_rows,
+    const bf16_t* __restrict__ x_table, const int* __restrict__ x_row, int x_rows) {
   constexpr int HALF = D / 2;
   __shared__ float scratch4[4];
   __shared__ float part[4][2];
@@ -172,10 +186,28 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   const float c_ahead = bf16_to_f32(angles[2 * j]), s_ahead = bf16_to_f32(angles[2 * j + 1]);
   const int pos_ahead = *position;
   Activation<CH, true> act;
-  act.issue(x, nw, K);
   uint4 w0[CH], w1[CH];
-  load_row<CH>(Wm + (size_t)r0 * K, K, w0);
-  load_row<CH>(Wm + (size_t)r1 * K, K, w1);
+  if (x_row == nullptr) {
+    act.issue(x, nw, K);
+    load_row<CH>(Wm + (size_t)r0 * K, K, w0);
+    load_row<CH>(Wm + (size_t)r1 * K, K, w1);
+  } else {
+    // The token's row of an embedding table, named by a device word (held inside the table): the row
+    // is read where it lies and the first block leaves the copy the layer's residual sum will read,
+    // so the step's gather needs no launch of its own.  Everything that does not wait for the word
+    // goes out ahead of it.
+    act.issue_gains(nw, K);
+    load_row<CH>(Wm + (size_t)r0 * K, K, w0);
+    load_row<CH>(Wm + (size_t)r1 * K, K, w1);
+    act.issue_row(x_table + (size_t)max(0, min(*x_row, x_rows - 1)) * K, K);
+    if (pair == 0) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        if (c < (K >> 3)) reinterpret_cast<uint4*>(const_cast<bf16_t*>(x))[c] = act.xv[i];
+      }
+    }
+  }
   float xf[CH][8];
   act.finish(eps, K, scratch4, xf);
   const float a0 = wave_sum(dot_row<CH>(w0, xf)), a1 = wave_sum(dot_row<CH>(w1, xf));
@@ -242,29 +274,50 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   IRON_REQUIRE(false, "gemv_fused: no kernel for this combination");
 }
 
-extern "C" int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, float eps,
-                                    const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,
-                                    const uint16_t* angles, uint16_t* q_out, uint16_t* keys,
-                                    uint16_t* values, int hidden, int heads, int kv_heads, int d,
-                                    int cache_rows, const int* position, const int* angle_row, int angle_rows,
-                                    void* stream) {
+static int decode_qkv(const uint16_t* x, const uint16_t* norm_w, float eps, const uint16_t* Wq, const uint16_t* Wk,
+                      const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out, uint16_t* keys, uint16_t* values,
+                      int hidden, int heads, int kv_heads, int d, int cache_rows, const int* position,
+                      const int* angle_row, int angle_rows, const uint16_t* x_table, const int* x_row, int x_rows,
+                      void* stream) {
   IRON_REQUIRE(x && norm_w && Wq && Wk && Wv && angles && q_out && keys && values && position,
                "decode_qkv: null operand");
   IRON_REQUIRE(hidden > 0 && hidden % 8 == 0, "decode_qkv: hidden (%d) must be a positive multiple of 8", hidden);
   IRON_REQUIRE(d == 64 || d == 128, "decode_qkv: d (%d) must be 64 or 128", d);
   IRON_REQUIRE(heads > 0 && kv_heads > 0 && cache_rows > 0, "decode_qkv: heads, kv_heads, cache_rows must be positive");
-  IRON_REQUIRE((((uintptr_t)x | (uintptr_t)norm_w | (uintptr_t)Wq | (uintptr_t)Wk | (uintptr_t)Wv) & 15) == 0,
+  IRON_REQUIRE((((uintptr_t)x | (uintptr_t)norm_w | (uintptr_t)Wq | (uintptr_t)Wk | (uintptr_t)Wv | (uintptr_t)x_table) & 15) == 0,
                "decode_qkv: operands must be 16-byte aligned");
   IRON_REQUIRE(hidden <= 8192, "decode_qkv: hidden (%d) exceeds 8192", hidden);
   IRON_REQUIRE(angle_row == nullptr || angle_rows > 0, "decode_qkv: a table of %d angle rows", angle_rows);
+  IRON_REQUIRE(x_row == nullptr || (x_table != nullptr && x_rows > 0), "decode_qkv: a row of a table of %d rows", x_rows);
   const int pairs = heads * (d / 2) + 2 * kv_heads * (d / 2);
   const int ch = hidden <= 2048 ? 1 : (hidden <= 4096 ? 2 : 4);
   hipStream_t s = (hipStream_t)stream;
 #define IRON_QKV(DD, C)                                                                             \
   if (d == DD && ch == C)                                                                           \
     hipLaunchKernelGGL((decode_qkv_kernel<DD, C>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
-                       angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row, angle_rows);
+                       angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row, angle_rows, \
+                       x_table, x_row, x_rows);
   IRON_QKV(64, 1) IRON_QKV(64, 2) IRON_QKV(64, 4) IRON_QKV(128, 1) IRON_QKV(128, 2) IRON_QKV(128, 4)
 #undef IRON_QKV
   IRON_LAUNCH_CHECK();
+}
+
+extern "C" int iron_decode_qkv_bf16(const uint16_t* x, const uint16_t* norm_w, float eps,
+                                    const uint16_t* Wq, const uint16_t* Wk, const uint16_t* Wv,
+                                    const uint16_t* angles, uint16_t* q_out, uint16_t* keys,
+                                    uint16_t* values, int hidden, int heads, int kv_heads, int d,
+                                    int cache_rows, const int* position, const int* angle_row, int angle_rows,
+                                    void* stream) {
+  return decode_qkv(x, norm_w, eps, Wq, Wk, Wv, angles, q_out, keys, values, hidden, heads, kv_heads, d, cache_rows,
+                    position, angle_row, angle_rows, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int iron_decode_qkv_embed_bf16(const uint16_t* table, const int* token, int table_rows, uint16_t* x,
+                                          const uint16_t* norm_w, float eps, const uint16_t* Wq, const uint16_t* Wk,
+                                          const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out, uint16_t* keys,
+                                          uint16_t* values, int hidden, int heads, int kv_heads, int d, int cache_rows,
+                                          const int* position, const int* angle_row, int angle_rows, void* stream) {
+  IRON_REQUIRE(table && token && table_rows > 0, "decode_qkv_embed: a table of %d rows and the word that names the row", table_rows);
+  return decode_qkv(x, norm_w, eps, Wq, Wk, Wv, angles, q_out, keys, values, hidden, heads, kv_heads, d, cache_rows,
+                    position, angle_row, angle_rows, table, token, table_rows, stream);
 }

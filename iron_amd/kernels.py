@@ -126,9 +126,11 @@ def gemv_fused(W, x, y, *, M, K, W2=None, norm_w=None, eps=0.0, residual=None, r
 
 
 def decode_qkv(x, norm_w, Wq, Wk, Wv, angles, q_out, keys, values, *, eps, hidden, heads, kv_heads, d,
-               cache_rows, position, angle_row=None):
+               cache_rows, position, angle_row=None, table=None, token=None):
     """Attention's first half for one token: norm, q/k/v projections, RoPE, cache writes.  ``angles``
-    is the token's row of the RoPE table, or with ``angle_row`` (a device word) the whole table."""
+    is the token's row of the RoPE table, or with ``angle_row`` (a device word) the whole table.  With
+    ``table`` and ``token`` (a device word) the input is that row of the embedding table, which the
+    launch also writes to ``x``."""
     _numel(_dev(x, "x"), hidden, "x")
     _numel(_dev(norm_w, "norm_w"), hidden, "norm_w")
     _numel(_dev(Wq, "Wq"), heads * d * hidden, "Wq")
@@ -142,6 +144,19 @@ def decode_qkv(x, norm_w, Wq, Wk, Wv, angles, q_out, keys, values, *, eps, hidde
     _numel(_dev(q_out, "q_out"), heads * d, "q_out")
     _numel(_dev(keys, "keys"), cache_rows * kv_heads * d, "keys")
     _numel(_dev(values, "values"), cache_rows * kv_heads * d, "values")
+    if table is not None:
+        _dev(table, "table")
+        if table.numel() % hidden or table.numel() < hidden:
+            raise ValueError(f"table: rows of {hidden}, got {table.numel()} elements")
+        check(
+            lib().iron_decode_qkv_embed_bf16(ptr(table), ptr(_word(token, "token")), table.numel() // hidden, ptr(x),
+                                             ptr(norm_w), float(eps), ptr(Wq), ptr(Wk), ptr(Wv), ptr(angles),
+                                             ptr(q_out), ptr(keys), ptr(values), hidden, heads, kv_heads, d, cache_rows,
+                                             ptr(_word(position, "position")), ptr(_word(angle_row, "angle_row")),
+                                             angles.numel() // d, current_stream()),
+            "iron_decode_qkv_embed_bf16",
+        )
+        return
     check(
         lib().iron_decode_qkv_bf16(ptr(x), ptr(norm_w), float(eps), ptr(Wq), ptr(Wk), ptr(Wv), ptr(angles),
                                    ptr(q_out), ptr(keys), ptr(values), hidden, heads, kv_heads, d, cache_rows,

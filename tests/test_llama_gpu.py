@@ -495,9 +495,10 @@ def test_fused_decode_step_matches_the_step_by_step_one(cuda, golden):
     steps = len(fused.decode_step.recording.steps)
     assert plain.decode_step.launches_per_call == steps
     # per layer 18 steps become 5 launches (qkv, attention, o+add, gate/up, down+add); the head 2 -> 1;
-    # the RoPE row's copy is not launched (the projections read the table at the position themselves), and
-    # a replay ends with the draw, which evaluates the step's carried and derived words itself.
-    assert fused.decode_step.launches_per_call == 1 + 5 * SCALED.num_hidden_layers + 2
+    # neither the RoPE row's copy nor the token's embedding row's is launched (the first layer's
+    # projections read both tables at the call's words themselves), and a replay ends with the draw,
+    # which evaluates the step's carried and derived words itself.
+    assert fused.decode_step.launches_per_call == 5 * SCALED.num_hidden_layers + 2
     assert fused.decode_step.launches_per_replay == fused.decode_step.launches_per_call
     assert plain.decode_step.launches_per_replay == steps
     # the prompt chunk: per layer the three projections, two rotations and two cache writes become
