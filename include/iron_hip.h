@@ -78,7 +78,10 @@ int iron_gemm_gated_pair_bf16(const uint16_t* A, const uint16_t* Bg, const uint1
  *   epilogue 0: y = bf16(W N(x));  1: y = bf16(residual_scale * bf16(W N(x)) + residual), one fused
  *   multiply-add (a scale of 1 is the plain sum; another is AXPY's, iron/lm/blocks.py:386-391);
  *   2: y = bf16(bf16(silu(bf16(W N(x)))) * bf16(W2 N(x)))   (gate, up -> SiLU -> Mul);
- *   3: the same with GELU by its tanh form for SiLU (Gemma's feed-forward).
+ *   3: the same with GELU by its tanh form for SiLU (Gemma's feed-forward);
+ *   4: y = bf16(bf16(gelu_tanh(bf16(W N(x)))) * residual), 5: the same with SiLU: a projection, its
+ *   activation and the product with a given row (`residual` holds it; Gemma 4's per-layer input gate,
+ *   iron/lm/blocks.py:793-796; norm_w must be NULL).
  * W, W2 (M,K); x, norm_w (K); residual, y (M).  K % 8 == 0. */
 int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const uint16_t* x,
                          const uint16_t* norm_w, float eps, const uint16_t* residual,
@@ -105,6 +108,20 @@ int iron_decode_qkv_embed_bf16(const uint16_t* table, const int* token, int tabl
                                const uint16_t* Wv, const uint16_t* angles, uint16_t* q_out, uint16_t* keys,
                                uint16_t* values, int hidden, int heads, int kv_heads, int d, int cache_rows,
                                const int* position, const int* angle_row, int angle_rows, void* stream);
+
+/* Between a token's q/k/v projections and its attention where the heads are normed one by one
+ * (Gemma's): RMSNorm of each q head (bit 0 of norms; gain q_gain or none), k head (bit 1; k_gain) and v
+ * head (bit 2; no gain), RoPE on q and k by the call's angle rows (q_angles, k_angles: `rotary`
+ * columns, cos/sin interleaved; the columns of a head past them pass through; NULL: not rotated), q ->
+ * q_out (heads, d), k -> keys[*row0] and v -> values[*row0], caches (cache_rows, kv_heads, d), and
+ * again at [*row1] where row1 is not NULL (a ring cache's mirror row).  k, v NULL: the layer reads
+ * another layer's cache and only q is done.  Each step computed as its own kernel computes it.
+ * Replaces up to 3 RMSNorm, 2 RoPE and 4 Copy steps (iron/lm/blocks.py:563-660,434-529). */
+int iron_decode_heads_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_gain,
+                           const uint16_t* k_gain, int norms, float eps, const uint16_t* q_angles,
+                           const uint16_t* k_angles, int rotary, int two_halves, uint16_t* q_out,
+                           uint16_t* keys, uint16_t* values, const int* row0, const int* row1,
+                           int cache_rows, int heads, int kv_heads, int d, void* stream);
 
 /* A prompt chunk's three projections and the rotation of q and k in one launch (no single
  * counterpart in the reference: replaces 3 GEMM and 2 RoPE steps, iron/lm/blocks.py:617-648, and

@@ -28,6 +28,10 @@ SIGNATURES = {
         c_int,
         [_P, _P, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P, c_int, _P],
     ),
+    "iron_decode_heads_bf16": (
+        c_int,
+        [_P, _P, _P, _P, _P, c_int, c_float, _P, _P, c_int, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P],
+    ),
     "iron_decode_qkv_embed_bf16": (
         c_int,
         [_P, _P, c_int, _P, _P, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P, c_int, _P],

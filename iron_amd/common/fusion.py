@@ -10,7 +10,9 @@ round:
   RMSNorm, GEMV gate, GEMV up, SiLU, ElementwiseMul      => iron_gemv_fused_bf16 (epilogue 2)
   ... with GELU (tanh) for SiLU                          => iron_gemv_fused_bf16 (epilogue 3)
   GEMV, ElementwiseAdd / AXPY (the residual)             => iron_gemv_fused_bf16 (epilogue 1)
-  RMSNorm, GEMV (the head)                               => iron_gemv_fused_bf16 (epilogue 0)
+  RMSNorm, GEMV (the head; or a layer's q, k, v)         => iron_gemv_fused_bf16 (epilogue 0) each
+  GEMV, GELU (tanh) or SiLU, Mul by a given row          => iron_gemv_fused_bf16 (epilogue 4 / 5)
+  RMSNorm per head of q/k/v, RoPE q/k, Copy k/v -> cache => iron_decode_heads_bf16
 
 in a prompt chunk's version (several rows, 64-wide heads),
 
@@ -157,6 +159,101 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                   activation="silu" if _name(sl) == "SiLU" else "gelu_tanh")
         return args, kw
 
+    def same_data(a, b) -> bool:
+        return (a is not None and b is not None and a.buffer is b.buffer and a.offset == b.offset
+                and a.elements == b.elements and _plain(a) and _plain(b))
+
+    def heads_finish_at(j):
+        """The launch for the steps from ``j`` on where they are what lies between a token's q/k/v
+        projections and its attention in a layer that norms its heads one by one: RMSNorm per head of
+        q (of k, of v), RoPE on q (and k), k's and v's copies into their cache rows -- or None."""
+        first = steps[j]
+        # the projections just ahead: q's product is what this norm reads; k's and v's follow it
+        back = j
+        while back > 0 and j - back < 3 and gemv_row(steps[back - 1]):
+            back -= 1
+        made = [g.outputs["C"] for g in steps[back:j]]
+        at = next((n for n, h in enumerate(made) if same_data(h, first.inputs["x"])), None)
+        if at is None or len(made) - at not in (1, 3):
+            return None
+        cur = {"q": made[at], "k": made[at + 1] if len(made) - at == 3 else None,
+               "v": made[at + 2] if len(made) - at == 3 else None}
+        d = first.op.tile_size
+        if any(h is not None and h.elements % d for h in cur.values()) or d % 16 or d > 2048:
+            return None
+        heads = cur["q"].elements // d
+        kv_heads = cur["k"].elements // d if cur["k"] is not None else 1
+        if cur["k"] is not None and cur["v"].elements != cur["k"].elements:
+            return None
+        p, norms, eps, gains = j, 0, None, {"q": None, "k": None}
+        for bit, name in enumerate(("q", "k", "v")):
+            st = steps[p] if p < len(steps) else None
+            if (cur[name] is None or st is None or _name(st) != "RMSNorm" or st.values or st.op.tile_size != d
+                    or not same_data(st.inputs["x"], cur[name]) or not once(cur[name]) or not _plain(st.outputs["y"])
+                    or (eps is not None and float(st.op.epsilon) != eps) or (name == "v" and st.op.weighted)):
+                continue
+            if st.op.weighted:
+                if not _plain(st.inputs["weight"]) or st.inputs["weight"].elements != d:
+                    return None
+                gains[name] = st.inputs["weight"]
+            norms |= 1 << bit
+            eps = float(st.op.epsilon)
+            cur[name] = st.outputs["y"]
+            p += 1
+        if not norms & 1:
+            return None
+        angles, rotary, two_halves = {"q": None, "k": None}, 0, True
+        for name in ("q", "k"):
+            st = steps[p] if p < len(steps) else None
+            if (cur[name] is None or st is None or _name(st) != "RoPE" or st.values or st.op.angle_rows != 1
+                    or st.op.row != d or st.op.cols % 16 or not same_data(st.inputs["x"], cur[name])
+                    or not once(cur[name]) or not _plain(st.inputs["angles"]) or not _plain(st.outputs["y"])
+                    or (rotary and (st.op.cols, st.op.two_halves) != (rotary, two_halves))):
+                continue
+            angles[name], rotary, two_halves = st.inputs["angles"], st.op.cols, bool(st.op.two_halves)
+            cur[name] = st.outputs["y"]
+            p += 1
+        # k's copies into its cache rows (the slot and, in a ring, its mirror), then v's into the same rows
+        caches, rows_at = {}, None
+        for name in ("k", "v"):
+            if cur[name] is None:
+                continue
+            found = []
+            while p < len(steps) and len(found) < 2 and _name(steps[p]) == "Copy" and not steps[p].values:
+                cp = steps[p]
+                src, dst = cp.inputs["src"], cp.outputs["dst"]
+                if not (same_data(src, cur[name]) and dst.index is not None and dst.ids is None and not dst.valid
+                        and dst.offset == 0 and dst.index_stride == cur[name].elements
+                        and dst.elements == cur[name].elements
+                        and (not found or dst.buffer is found[0].buffer)):
+                    break
+                found.append(dst)
+                p += 1
+            if not found or not once(cur[name], len(found)):
+                return None
+            if rows_at is None:
+                rows_at = [f.index for f in found]
+            elif [f.index for f in found] != rows_at or found[0].index_rows != caches["k"].index_rows:
+                return None
+            caches[name] = found[0]
+        if p - j < 2:
+            return None
+        args = dict(q=tensor(made[at]).reshape(-1), q_out=tensor(cur["q"]).reshape(-1))
+        kw = dict(heads=heads, kv_heads=kv_heads, d=d, eps=eps, norms=norms, rotary=rotary, two_halves=two_halves)
+        for name in ("q", "k"):
+            if gains[name] is not None:
+                args[f"{name}_gain"] = tensor(gains[name]).reshape(-1)
+            if angles[name] is not None:
+                args[f"{name}_angles"] = tensor(angles[name]).reshape(-1)
+        if caches:
+            kd, vd = caches["k"], caches["v"]
+            args |= dict(k=tensor(made[at + 1]).reshape(-1), v=tensor(made[at + 2]).reshape(-1),
+                         keys=tensor(kd)[: kd.index_rows * kd.index_stride],
+                         values=tensor(vd)[: vd.index_rows * vd.index_stride])
+            kw |= dict(cache_rows=kd.index_rows, row0=word(rows_at[0]),
+                       row1=word(rows_at[1]) if len(rows_at) > 1 else None)
+        return Fused("decode_heads", j, p - j, lambda a=args, kw=kw: kernels.decode_heads(**a, **kw))
+
     fused: list[Fused] = []
     # decode_qkv launches whose RoPE row is a copy of one table row: (producing step, args, kw)
     rope_rows: list[tuple[int, dict, dict]] = []
@@ -226,13 +323,24 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                                 y=tensor(mu.outputs["y"]).reshape(-1))
                     kw = dict(M=gg.op.M, K=gg.op.K, eps=float(s.op.epsilon), epilogue=2 if _name(si) == "SiLU" else 3)
                     got = Fused("norm_gate_up_silu_mul" if _name(si) == "SiLU" else "norm_gate_up_gelu_mul", i, 5, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
-            # the head: norm, then one projection
-            if got is None and rest and gemv_row(rest[0], n) and once(n, 1):
-                g0 = rest[0]
-                args = dict(W=tensor(g0.inputs["A"]), x=tensor(s.inputs["x"]).reshape(-1),
-                            norm_w=tensor(s.inputs["weight"]).reshape(-1), y=tensor(g0.outputs["C"]).reshape(-1))
-                kw = dict(M=g0.op.M, K=g0.op.K, eps=float(s.op.epsilon), epilogue=0)
-                got = Fused("norm_gemv", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+            # the head: norm, then one projection -- or a layer's q, k, v projections where something
+            # other than RoPE follows them (heads normed one by one): the norm rides each one's prologue
+            if got is None:
+                count = 0
+                while count < 3 and count < len(rest) and gemv_row(rest[count], n):
+                    count += 1
+                if count and once(n, count):
+                    calls = []
+                    for g0 in rest[:count]:
+                        args = dict(W=tensor(g0.inputs["A"]), x=tensor(s.inputs["x"]).reshape(-1),
+                                    norm_w=tensor(s.inputs["weight"]).reshape(-1), y=tensor(g0.outputs["C"]).reshape(-1))
+                        calls.append((args, dict(M=g0.op.M, K=g0.op.K, eps=float(s.op.epsilon), epilogue=0)))
+
+                    def norm_gemvs(calls=calls):
+                        for a, kw in calls:
+                            kernels.gemv_fused(**a, **kw)
+
+                    got = Fused("norm_gemv", i, 1 + count, norm_gemvs, launches=count)
         elif (_name(s) == "GEMM" and len(steps) - i >= 5
               and [_name(t) for t in steps[i + 1 : i + 5]] == ["GEMM", "GEMM", "RoPE", "RoPE"]):
             # a prompt chunk's projections and rotations
@@ -332,6 +440,25 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                             y=tensor(m.outputs["y"]).reshape(-1))
                 kw = dict(n=s.op.size, valid=word(m.values.get("valid")))
                 got = Fused("silu_mul", i, 2, lambda a=args, kw=kw: kernels.silu_mul(**a, **kw))
+        elif (gemv_row(s) and i + 2 < len(steps) and _name(steps[i + 2]) in ("RowwiseMul", "ElementwiseMul")
+              and (_name(steps[i + 1]) == "SiLU"
+                   or (_name(steps[i + 1]) == "GELU" and steps[i + 1].op.approximate == "tanh"))):
+            # a projection, its activation and the product with a given row (a per-layer input's gate)
+            ac, mu = steps[i + 1], steps[i + 2]
+            c, act = s.outputs["C"], ac.outputs["y"]
+            if _name(mu) == "RowwiseMul":   # one row of x by the row: the same product element by element
+                a, b = mu.inputs["x"], mu.inputs["row"]
+                other = None if mu.op.rows != 1 else (b if same_data(a, act) else (a if same_data(b, act) else None))
+            else:
+                a, b = mu.inputs["a"], mu.inputs["b"]
+                other = b if same_data(a, act) else (a if same_data(b, act) else None)
+            if (other is not None and same_data(ac.inputs["x"], c) and once(c) and once(act) and not ac.values
+                    and not mu.values and _plain(other) and other.elements == c.elements and _plain(mu.outputs["y"])
+                    and mu.outputs["y"].elements == c.elements and other.buffer is not act.buffer):
+                args = dict(W=tensor(s.inputs["A"]), x=tensor(s.inputs["B"]).reshape(-1),
+                            residual=tensor(other).reshape(-1), y=tensor(mu.outputs["y"]).reshape(-1))
+                kw = dict(M=s.op.M, K=s.op.K, epilogue=5 if _name(ac) == "SiLU" else 4)
+                got = Fused("gemv_act_mul", i, 3, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
         elif gemv_row(s) and i + 1 < len(steps) and _name(steps[i + 1]) in ("ElementwiseAdd", "AXPY"):
             ad = steps[i + 1]
             c = s.outputs["C"]
@@ -346,6 +473,8 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                             residual=tensor(other).reshape(-1), y=tensor(ad.outputs["y"]).reshape(-1))
                 kw = dict(M=s.op.M, K=s.op.K, epilogue=1, residual_scale=scale)
                 got = Fused("gemv_add", i, 2, lambda a=args, kw=kw: kernels.gemv_fused(**a, **kw))
+        if got is None and _name(s) == "RMSNorm" and s.op.rows >= 1 and not s.values:
+            got = heads_finish_at(i)
         if (got is None and _name(s) == "RMSNorm" and i + 1 < len(steps) and _name(steps[i + 1]) == "ElementwiseAdd"
                 and set(s.values) <= {"valid"}):
             # a block's output normed again before its residual (a sandwich layer): the sum rides the norm's pass

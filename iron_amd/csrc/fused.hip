@@ -102,7 +102,8 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[CH], const float (&xf)
   return acc;
 }
 
-enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2, EPI_GELU_MUL = 3 };   // 2 and 3: gate, up -> activation -> Mul
+enum { EPI_NONE = 0, EPI_ADD = 1, EPI_SILU_MUL = 2, EPI_GELU_MUL = 3,     // 2 and 3: gate, up -> activation -> Mul
+       EPI_GELU_ROW = 4, EPI_SILU_ROW = 5 };                               // activation -> Mul by a given row
 
 // y = E(W @ N(x)) for RPW rows a block; K <= CH * 2048.
 template <int RPW, int CH, bool NORM, int EPI>
@@ -121,7 +122,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
   // The residual a thread will add at the end is requested first, so that its trip to memory
   // passes under the weights' instead of after the block's last barrier.
   float res_ahead = 0.f;
-  if (EPI == EPI_ADD && threadIdx.x < RPW) res_ahead = bf16_to_f32(res[min(row0 + (int)threadIdx.x, M - 1)]);
+  if ((EPI == EPI_ADD || EPI == EPI_GELU_ROW || EPI == EPI_SILU_ROW) && threadIdx.x < RPW)
+    res_ahead = bf16_to_f32(res[min(row0 + (int)threadIdx.x, M - 1)]);
   Activation<CH, NORM> act;
   act.issue(x, nw, K);
   uint4 w[MATS][RPW][CH];
@@ -146,6 +148,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
     if (row < M) {
       float v = round_bf16(part[0][0][r] + part[1][0][r] + part[2][0][r] + part[3][0][r]);  // the GEMV's own rounding
       if (EPI == EPI_ADD) v = fmaf(res_scale, v, res_ahead);   // scale 1: the plain sum
+      if (EPI == EPI_GELU_ROW || EPI == EPI_SILU_ROW)          // the activation's own rounding, then the product's
+        v = round_bf16(EPI == EPI_SILU_ROW ? silu_f32(v) : gelu_tanh_f32(v)) * res_ahead;
       if (EPI == EPI_SILU_MUL || EPI == EPI_GELU_MUL) {
         const float u = round_bf16(part[0][MATS - 1][r] + part[1][MATS - 1][r] + part[2][MATS - 1][r] +
                                    part[3][MATS - 1][r]);
@@ -234,6 +238,138 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   }
 }
 
+
+// Between a token's q/k/v projections and its attention, where the heads are normed one by one (q and
+// k with learned gains, v without: Gemma's): RMSNorm per head, RoPE on q and k, and k's and v's rows
+// into their cache rows (twice where the cache is a ring: the slot and its mirror) -- up to nine
+// recorded steps, one launch.  A block a head row (q heads, then k's, then v's), 256 threads, each
+// step computed exactly as its own kernel computes it (the norm's sum in rmsnorm_kernel's order, its
+// two roundings; RoPE on the rounded row), so the rows are those kernels' bit for bit.
+struct HeadRows {
+  const bf16_t *q, *k, *v;            // (heads, d), (kv_heads, d) twice; k and v NULL where another layer owns the cache
+  const bf16_t *q_gain, *k_gain;      // (d); NULL: that norm has no gain
+  int norms;                          // bit 0: q is normed, 1: k, 2: v
+  float eps;
+  const bf16_t *q_angles, *k_angles;  // the call's RoPE rows (rotary columns, cos/sin interleaved); NULL: not rotated
+  int rotary, two_halves;             // columns RoPE turns (<= d; the rest pass through)
+  bf16_t* q_out;                      // (heads, d)
+  bf16_t* dst[2][2];                  // [k, v][copy]: caches (cache_rows, kv_heads, d); NULL: no such copy
+  const int* row[2][2];               // the cache row each copy goes to
+  int cache_rows, heads, kv_heads, d;
+};
+
+__global__ __launch_bounds__(256) void decode_heads_kernel(HeadRows a) {
+  __shared__ float part[4];
+  __shared__ __align__(16) bf16_t held[2048];
+  const int t = threadIdx.x, d = a.d, nchunk = d >> 3;
+  const int b = blockIdx.x;
+  const int kind = b < a.heads ? 0 : (b < a.heads + a.kv_heads ? 1 : 2);   // q, k, v
+  const int head = kind == 0 ? b : b - a.heads - (kind - 1) * a.kv_heads;
+  const bf16_t* src = (kind == 0 ? a.q : kind == 1 ? a.k : a.v) + (size_t)head * d;
+  const bf16_t* gain = kind == 0 ? a.q_gain : (kind == 1 ? a.k_gain : nullptr);
+  const bf16_t* angles = kind == 0 ? a.q_angles : (kind == 1 ? a.k_angles : nullptr);
+  const bool normed = (a.norms >> kind) & 1;
+  // Where the row goes: q to its output, k and v to their cache rows.
+  int rows[2] = {0, 0};
+  if (kind != 0) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      if (a.dst[kind - 1][c] != nullptr) rows[c] = *a.row[kind - 1][c];
+  }
+
+  uint4 xv = make_uint4(0, 0, 0, 0), gv = make_uint4(0, 0, 0, 0);
+  if (t < nchunk) {
+    xv = reinterpret_cast<const uint4*>(src)[t];
+    if (normed && gain != nullptr) gv = reinterpret_cast<const uint4*>(gain)[t];
+  }
+  float f[8];
+  unpack8(xv, f);
+  if (normed) {
+    float ss = 0.f;
+    if (t < nchunk) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
+    }
+    ss = wave_sum(ss);
+    if ((t & 63) == 0) part[t >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf((part[0] + part[1] + part[2] + part[3]) / (float)d + a.eps);
+    if (gain != nullptr) {
+      float g[8];
+      unpack8(gv, g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = round_bf16(f[j] * inv) * g[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) f[j] = f[j] * inv;
+    }
+    xv = pack8(f);
+  }
+  if (angles != nullptr) {
+    if (t < nchunk) reinterpret_cast<uint4*>(held)[t] = xv;
+    __syncthreads();
+    uint4 oa = make_uint4(0, 0, 0, 0), ob = oa;
+    const int j = t, turning = a.rotary >> 4;   // thread j turns 8 column pairs
+    if (j < turning) {
+      float cs0[8], cs1[8], x1[8], x2[8], y1[8], y2[8];
+      unpack8(reinterpret_cast<const uint4*>(angles + 16 * j)[0], cs0);
+      unpack8(reinterpret_cast<const uint4*>(angles + 16 * j)[1], cs1);
+      const float c[8] = {cs0[0], cs0[2], cs0[4], cs0[6], cs1[0], cs1[2], cs1[4], cs1[6]};
+      const float sn[8] = {cs0[1], cs0[3], cs0[5], cs0[7], cs1[1], cs1[3], cs1[5], cs1[7]};
+      if (a.two_halves) {
+        const int half = a.rotary >> 1;
+        unpack8(*reinterpret_cast<const uint4*>(held + 8 * j), x1);
+        unpack8(*reinterpret_cast<const uint4*>(held + half + 8 * j), x2);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          y1[i] = x1[i] * c[i] - x2[i] * sn[i];
+          y2[i] = x2[i] * c[i] + x1[i] * sn[i];
+        }
+        oa = pack8(y1);
+        ob = pack8(y2);
+      } else {
+        float lo[8], hi[8];
+        unpack8(*reinterpret_cast<const uint4*>(held + 16 * j), lo);
+        unpack8(*reinterpret_cast<const uint4*>(held + 16 * j + 8), hi);
+        const float e[8] = {lo[0], lo[2], lo[4], lo[6], hi[0], hi[2], hi[4], hi[6]};
+        const float o[8] = {lo[1], lo[3], lo[5], lo[7], hi[1], hi[3], hi[5], hi[7]};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          y1[i] = e[i] * c[i] - o[i] * sn[i];
+          y2[i] = o[i] * c[i] + e[i] * sn[i];
+        }
+        const float r0[8] = {y1[0], y2[0], y1[1], y2[1], y1[2], y2[2], y1[3], y2[3]};
+        const float r1[8] = {y1[4], y2[4], y1[5], y2[5], y1[6], y2[6], y1[7], y2[7]};
+        oa = pack8(r0);
+        ob = pack8(r1);
+      }
+    }
+    __syncthreads();   // every pair has been read before any is replaced
+    if (j < turning) {
+      if (a.two_halves) {
+        *reinterpret_cast<uint4*>(held + 8 * j) = oa;
+        *reinterpret_cast<uint4*>(held + (a.rotary >> 1) + 8 * j) = ob;
+      } else {
+        *reinterpret_cast<uint4*>(held + 16 * j) = oa;
+        *reinterpret_cast<uint4*>(held + 16 * j + 8) = ob;
+      }
+    }
+    __syncthreads();
+    if (t < nchunk) xv = reinterpret_cast<const uint4*>(held)[t];
+  }
+  if (t >= nchunk) return;
+  if (kind == 0) {
+    reinterpret_cast<uint4*>(a.q_out + (size_t)head * d)[t] = xv;
+    return;
+  }
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    bf16_t* cache = a.dst[kind - 1][c];
+    if (cache == nullptr || rows[c] < 0 || rows[c] >= a.cache_rows) continue;
+    reinterpret_cast<uint4*>(cache + ((size_t)rows[c] * a.kv_heads + head) * d)[t] = xv;
+  }
+}
+
 }  // namespace iron
 
 using namespace iron;
@@ -244,8 +380,9 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
                                     void* stream) {
   IRON_REQUIRE(W && x && y, "gemv_fused: null operand");
   IRON_REQUIRE(M > 0 && K > 0 && K % 8 == 0, "gemv_fused: M (%d) positive, K (%d) a positive multiple of 8", M, K);
-  IRON_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemv_fused: epilogue (%d) is 0, 1, 2 or 3", epilogue);
-  IRON_REQUIRE(epilogue != EPI_ADD || residual, "gemv_fused: epilogue 1 adds a residual; none given");
+  IRON_REQUIRE(epilogue >= 0 && epilogue <= 5, "gemv_fused: epilogue (%d) is 0 to 5", epilogue);
+  IRON_REQUIRE((epilogue != EPI_ADD && epilogue != EPI_GELU_ROW && epilogue != EPI_SILU_ROW) || residual,
+               "gemv_fused: epilogues 1, 4 and 5 take a second row (the residual, the factor); none given");
   IRON_REQUIRE((epilogue != EPI_SILU_MUL && epilogue != EPI_GELU_MUL) || W2, "gemv_fused: epilogues 2 and 3 take a second matrix; none given");
   IRON_REQUIRE((((uintptr_t)W | (uintptr_t)W2 | (uintptr_t)x | (uintptr_t)norm_w) & 15) == 0,
                "gemv_fused: operands must be 16-byte aligned");
@@ -269,6 +406,9 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   IRON_FUSED(1, 4, false, 2) IRON_FUSED(1, 4, true, 2) IRON_FUSED(1, 8, false, 2) IRON_FUSED(1, 8, true, 2)
   IRON_FUSED(2, 1, false, 3) IRON_FUSED(2, 1, true, 3) IRON_FUSED(1, 2, false, 3) IRON_FUSED(1, 2, true, 3)
   IRON_FUSED(1, 4, false, 3) IRON_FUSED(1, 4, true, 3) IRON_FUSED(1, 8, false, 3) IRON_FUSED(1, 8, true, 3)
+  IRON_FUSED(1, 1, false, 4) IRON_FUSED(1, 2, false, 4) IRON_FUSED(1, 4, false, 4) IRON_FUSED(1, 8, false, 4)
+  IRON_FUSED(1, 1, false, 5) IRON_FUSED(1, 2, false, 5) IRON_FUSED(1, 4, false, 5) IRON_FUSED(1, 8, false, 5)
+  IRON_FUSED(2, 1, false, 4) IRON_FUSED(4, 1, false, 4) IRON_FUSED(2, 1, false, 5) IRON_FUSED(4, 1, false, 5)
 #undef IRON_FUSED_NE
 #undef IRON_FUSED
   IRON_REQUIRE(false, "gemv_fused: no kernel for this combination");
@@ -320,4 +460,42 @@ extern "C" int iron_decode_qkv_embed_bf16(const uint16_t* table, const int* toke
   IRON_REQUIRE(table && token && table_rows > 0, "decode_qkv_embed: a table of %d rows and the word that names the row", table_rows);
   return decode_qkv(x, norm_w, eps, Wq, Wk, Wv, angles, q_out, keys, values, hidden, heads, kv_heads, d, cache_rows,
                     position, angle_row, angle_rows, table, token, table_rows, stream);
+}
+
+extern "C" int iron_decode_heads_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* q_gain,
+                                      const uint16_t* k_gain, int norms, float eps, const uint16_t* q_angles,
+                                      const uint16_t* k_angles, int rotary, int two_halves, uint16_t* q_out,
+                                      uint16_t* keys, uint16_t* values, const int* row0, const int* row1,
+                                      int cache_rows, int heads, int kv_heads, int d, void* stream) {
+  IRON_REQUIRE(q && q_out, "decode_heads: null operand");
+  IRON_REQUIRE((k == nullptr) == (v == nullptr), "decode_heads: k and v come together or not at all");
+  IRON_REQUIRE(k == nullptr || (keys && values && row0 && cache_rows > 0),
+               "decode_heads: k and v go to caches of %d rows at the row a device word names", cache_rows);
+  IRON_REQUIRE(heads > 0 && kv_heads > 0 && d > 0 && d % 16 == 0 && d <= 2048,
+               "decode_heads: heads (%d), kv_heads (%d) positive, d (%d) a multiple of 16 up to 2048", heads, kv_heads, d);
+  IRON_REQUIRE(norms >= 0 && norms < 8, "decode_heads: norms (%d) is a mask of q (1), k (2), v (4)", norms);
+  IRON_REQUIRE((q_angles == nullptr && k_angles == nullptr) || (rotary > 0 && rotary <= d && rotary % 16 == 0),
+               "decode_heads: RoPE turns %d columns of a head of %d (a positive multiple of 16)", rotary, d);
+  IRON_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)q_gain | (uintptr_t)k_gain | (uintptr_t)q_angles |
+                 (uintptr_t)k_angles | (uintptr_t)q_out | (uintptr_t)keys | (uintptr_t)values) & 15) == 0,
+               "decode_heads: operands must be 16-byte aligned");
+  HeadRows a{};
+  a.q = q; a.k = k; a.v = v;
+  a.q_gain = q_gain; a.k_gain = k_gain;
+  a.norms = norms; a.eps = eps;
+  a.q_angles = q_angles; a.k_angles = k_angles;
+  a.rotary = rotary; a.two_halves = two_halves;
+  a.q_out = q_out;
+  if (k != nullptr) {
+    a.dst[0][0] = keys; a.dst[1][0] = values;
+    a.row[0][0] = a.row[1][0] = row0;
+    if (row1 != nullptr) {
+      a.dst[0][1] = keys; a.dst[1][1] = values;
+      a.row[0][1] = a.row[1][1] = row1;
+    }
+  }
+  a.cache_rows = cache_rows; a.heads = heads; a.kv_heads = kv_heads; a.d = d;
+  const int blocks = heads + (k != nullptr ? 2 * kv_heads : 0);
+  hipLaunchKernelGGL(decode_heads_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+  IRON_LAUNCH_CHECK();
 }

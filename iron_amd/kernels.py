@@ -166,6 +166,26 @@ def decode_qkv(x, norm_w, Wq, Wk, Wv, angles, q_out, keys, values, *, eps, hidde
     )
 
 
+def decode_heads(q, q_out, *, heads, kv_heads, d, eps, norms=0, k=None, v=None, q_gain=None, k_gain=None,
+                 q_angles=None, k_angles=None, rotary=0, two_halves=True, keys=None, values=None, row0=None,
+                 row1=None, cache_rows=0):
+    """Per-head norms, RoPE and the cache rows of one token's q, k, v (``iron_decode_heads_bf16``)."""
+    _numel(_dev(q, "q"), heads * d, "q")
+    _numel(_dev(q_out, "q_out"), heads * d, "q_out")
+    for name, t, n in (("k", k, kv_heads * d), ("v", v, kv_heads * d), ("q_gain", q_gain, d), ("k_gain", k_gain, d),
+                       ("q_angles", q_angles, rotary), ("k_angles", k_angles, rotary),
+                       ("keys", keys, cache_rows * kv_heads * d), ("values", values, cache_rows * kv_heads * d)):
+        if t is not None:
+            _numel(_dev(t, name), n, name)
+    check(
+        lib().iron_decode_heads_bf16(ptr(q), ptr(k), ptr(v), ptr(q_gain), ptr(k_gain), int(norms), float(eps),
+                                     ptr(q_angles), ptr(k_angles), int(rotary), int(two_halves), ptr(q_out), ptr(keys),
+                                     ptr(values), ptr(_word(row0, "row0")), ptr(_word(row1, "row1")), int(cache_rows),
+                                     heads, kv_heads, d, current_stream()),
+        "iron_decode_heads_bf16",
+    )
+
+
 def prefill_qkv(x, Wq, Wk, Wv, angles, q_out, k_out, v_out, *, rows, hidden, heads, kv_heads, d, valid=None):
     """A prompt chunk's q/k/v projections with q and k turned by RoPE, one launch."""
     _numel(_dev(x, "x"), rows * hidden, "x")

@@ -196,6 +196,29 @@ def test_the_gpu_matches_the_host_step_by_step_past_a_ring(cuda, global_head_dim
 
 
 @pytest.mark.gpu
+def test_the_fused_decode_step_matches_the_step_by_step_one(cuda, w):
+    """The one-row fusions of Gemma 4's layers -- the input norm riding the q, k, v projections, the
+    per-head norms, RoPE and cache rows (ring and mirror) as one launch, the per-layer input's gate in
+    its projection's epilogue -- against every recorded step launched on its own: the same logits
+    within bf16 rounding across a ring's wrap, in well under three quarters of the launches."""
+    fused, plain = Gemma4(TOY, w), Gemma4(TOY, w)
+    fused.load_versions(fuse=True)
+    plain.load_versions(fuse=False)
+    try:
+        steps = len(plain.decode_step.recording.steps)
+        assert plain.decode_step.launches_per_call == steps
+        assert fused.decode_step.launches_per_call <= 0.6 * steps
+        tokens = np.random.default_rng(14).integers(0, TOY.vocab_size, 140)
+        for n in (30, 31, 32, 139, 140):     # prompt chunks, then single decode steps; the rings hold 128 rows
+            a, b = fused.logits(tokens[:n]), plain.logits(tokens[:n])
+            assert np.abs(a - b).max() <= 0.02 * np.abs(b).max(), n
+        assert fused.generate(tokens[:100], 40) == list(fused.session.draw(tokens[:100], 40, each=True))
+    finally:
+        fused.release()
+        plain.release()
+
+
+@pytest.mark.gpu
 def test_check_mode_judges_every_step_of_gemma_against_its_reference(cuda, w):
     """Every recorded step launched on its own and judged against its operator's reference by the
     operator's own tolerance: the per-head norms, GELU, the capped logits and the constant rows too."""

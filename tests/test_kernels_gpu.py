@@ -814,6 +814,77 @@ def test_mha_512_wide_heads_prefill_and_decode(cuda):
         close(O, want)
 
 
+@pytest.mark.parametrize("H,G,d,rotary,ring,own_kv", [(4, 1, 128, 128, True, True), (4, 1, 256, 64, False, True),
+                                                       (8, 2, 512, 512, True, True), (4, 1, 128, 128, False, False),
+                                                       (16, 8, 64, 64, False, True)])
+def test_decode_heads_is_the_separate_launches_bit_for_bit(cuda, H, G, d, rotary, ring, own_kv):
+    """What lies between a token's projections and its attention where heads are normed one by one:
+    per-head RMSNorm of q and k (gains) and v (none), RoPE on q and k (all of a head's columns, or the
+    leading ones), k's and v's rows into their caches (twice for a ring) -- one launch against the
+    launches of the separate operators bit for bit, and q's norm against the oracle."""
+    rng = np.random.default_rng(H + d)
+    rows = 24
+    q, k, v = bf(rng, H, d), bf(rng, G, d), bf(rng, G, d)
+    gq, gk = bf(rng, d, scale=0.3) + 1, bf(rng, d, scale=0.3) + 1
+    angles = bf(rng, 1, rotary)
+    dq, dk, dv, dgq, dgk, da = (dev(x, cuda) for x in (q, k, v, round_bf16(gq), round_bf16(gk), angles))
+    # the separate launches
+    def normed(x, gain, n):
+        y = out_like((n, d), cuda)
+        K.rmsnorm(x, gain, y, rows=n, cols=d, eps=1e-6)
+        return y
+
+    def roped(x, n):
+        y = out_like((n, d), cuda)
+        K.rope(x, da, y, rows=n, cols=rotary, angle_rows=1, row_cols=d)
+        return y
+
+    want_q = roped(normed(dq, dgq, H), H)
+    close(normed(dq, dgq, H), ops.rms_norm(q, round_bf16(gq), epsilon=1e-6))
+    row0, row1 = word(5, cuda), word(5 + rows // 2, cuda)
+    got_q = out_like((H, d), cuda, fill=float("nan"))
+    if not own_kv:
+        K.decode_heads(dq, got_q, heads=H, kv_heads=G, d=d, eps=1e-6, norms=1, q_gain=dgq, q_angles=da, rotary=rotary)
+        assert torch.equal(got_q, want_q)
+        return
+    want_k, want_v = roped(normed(dk, dgk, G), G), normed(dv, None, G)
+    keys, values = out_like((rows, G, d), cuda, fill=3.0), out_like((rows, G, d), cuda, fill=3.0)
+    K.decode_heads(dq, got_q, heads=H, kv_heads=G, d=d, eps=1e-6, norms=7, k=dk, v=dv, q_gain=dgq, k_gain=dgk,
+                   q_angles=da, k_angles=da, rotary=rotary, keys=keys, values=values, row0=row0,
+                   row1=row1 if ring else None, cache_rows=rows)
+    assert torch.equal(got_q, want_q)
+    held = [5, 5 + rows // 2] if ring else [5]
+    for r in range(rows):
+        if r in held:
+            assert torch.equal(keys[r], want_k) and torch.equal(values[r], want_v), r
+        else:
+            assert bool((keys[r] == 3.0).all()) and bool((values[r] == 3.0).all()), r
+
+
+@pytest.mark.parametrize("M,Kdim", [(128, 512), (256, 2048), (3000, 1536), (128, 8192)])
+@pytest.mark.parametrize("activation", ["gelu_tanh", "silu"])
+def test_gemv_with_an_activation_and_a_row_in_its_epilogue(cuda, M, Kdim, activation):
+    """A projection of one row, its activation and the product with a given row (Gemma 4's per-layer
+    input gate) in one launch: link by link against the oracle, and bit for bit against this library's
+    own separate launches."""
+    rng = np.random.default_rng(M + Kdim)
+    W, x, row = bf(rng, M, Kdim, scale=0.05), bf(rng, Kdim), bf(rng, M)
+    dW, dx, drow = dev(W, cuda), dev(x, cuda), dev(row, cuda)
+    y = out_like((M,), cuda)
+    K.gemv_fused(dW, dx, y, M=M, K=Kdim, residual=drow, epilogue=4 if activation == "gelu_tanh" else 5)
+    u, a, want = out_like((M,), cuda), out_like((M,), cuda), out_like((M,), cuda)
+    K.gemv(dW, dx, u, M=M, K=Kdim)
+    close(u, ops.gemv(W, x))
+    if activation == "gelu_tanh":
+        K.unary(u, a, "gelu_tanh", n=M)
+        close(a, ops.gelu(from_torch(u), approximate="tanh"))
+    else:
+        K.silu(u, a, n=M)
+        close(a, ops.silu(from_torch(u)))
+    K.mul(a, drow, want, n=M)
+    assert torch.equal(y, want)
+
+
 @pytest.mark.parametrize("L", [1024, 4096, 16384])
 def test_mha_decode_llama_shape(cuda, L):
     rng = np.random.default_rng(15)
