@@ -106,6 +106,21 @@ __device__ __forceinline__ uint4 load_stream(const uint4* p) {
   u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+// `bytes` bytes as a bounded buffer: a 16-byte load at an offset past their end returns zeros, so a
+// thread with no chunk of a row takes no branch around its load.  (Behind such a branch the compiler
+// waits for the load where it stands, to move what arrived into the register the join expects, and
+// a kernel's loads that were to be in flight together become one trip to memory after another.)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t bounded_bytes(const void* base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 load_bounded(__amdgpu_buffer_rsrc_t run, int offset) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(run, offset, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint4 load_bounded_stream(__amdgpu_buffer_rsrc_t run, int offset) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(run, offset, 0, 2);   // 2: non-temporal
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 __device__ __forceinline__ void store_stream(uint4* p, const uint4& v) {
   u32x4 w = {v.x, v.y, v.z, v.w};
   __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(p));

@@ -34,26 +34,21 @@ template <int CH, bool NORM>
 struct Activation {
   uint4 xv[CH], gv[CH];
   __device__ __forceinline__ void issue(const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw, int K) {
-    issue_gains(nw, K);
     issue_row(x, K);
+    issue_gains(nw, K);
   }
   // ... or apart, where the row's address is itself on its way from memory: the gains (and the
   // caller's weights) go out first and the row's loads once the address is in.
   __device__ __forceinline__ void issue_gains(const bf16_t* __restrict__ nw, int K) {
-    const int chunks = K >> 3;
+    if (!NORM) return;
+    const __amdgpu_buffer_rsrc_t run = bounded_bytes(nw, 2 * K);
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (NORM) gv[i] = c < chunks ? reinterpret_cast<const uint4*>(nw)[c] : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < CH; ++i) gv[i] = load_bounded(run, 16 * ((int)threadIdx.x + 256 * i));
   }
   __device__ __forceinline__ void issue_row(const bf16_t* __restrict__ x, int K) {
-    const int chunks = K >> 3;
+    const __amdgpu_buffer_rsrc_t run = bounded_bytes(x, 2 * K);
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      xv[i] = c < chunks ? reinterpret_cast<const uint4*>(x)[c] : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < CH; ++i) xv[i] = load_bounded(run, 16 * ((int)threadIdx.x + 256 * i));
   }
   // With NORM the block sums the squares together (one barrier).
   __device__ __forceinline__ void finish(float eps, int K, float* scratch4, float (&xf)[CH][8]) {
@@ -79,14 +74,12 @@ struct Activation {
   }
 };
 
+// A weight row's chunks of this thread (zeros past the row's end), streamed past the caches.
 template <int CH>
 __device__ __forceinline__ void load_row(const bf16_t* __restrict__ row, int K, uint4 (&w)[CH]) {
-  const int chunks = K >> 3;
+  const __amdgpu_buffer_rsrc_t run = bounded_bytes(row, 2 * K);
 #pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int c = threadIdx.x + 256 * i;
-    w[i] = c < chunks ? load_stream(reinterpret_cast<const uint4*>(row) + c) : make_uint4(0, 0, 0, 0);
-  }
+  for (int i = 0; i < CH; ++i) w[i] = load_bounded_stream(run, 16 * ((int)threadIdx.x + 256 * i));
 }
 
 template <int CH>
@@ -162,7 +155,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
 
 // Attention's first half for one token.  A block takes a PAIR of projection rows: for q and k
 // the rows (h, j) and (h, j + D/2) that RoPE rotates together, for v two adjacent rows.
-template <int D, int CH>
+// TABLE: x is to be read from row *x_row of x_table (and left in x by the first block).
+template <int D, int CH, bool TABLE>
 __global__ __launch_bounds__(256) void decode_qkv_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw, float eps,
     const bf16_t* __restrict__ Wq, const bf16_t* __restrict__ Wk, const bf16_t* __restrict__ Wv,
@@ -191,7 +185,7 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   const int pos_ahead = *position;
   Activation<CH, true> act;
   uint4 w0[CH], w1[CH];
-  if (x_row == nullptr) {
+  if (!TABLE) {
     act.issue(x, nw, K);
     load_row<CH>(Wm + (size_t)r0 * K, K, w0);
     load_row<CH>(Wm + (size_t)r1 * K, K, w1);
@@ -433,10 +427,16 @@ static int decode_qkv(const uint16_t* x, const uint16_t* norm_w, float eps, cons
   const int ch = hidden <= 2048 ? 1 : (hidden <= 4096 ? 2 : 4);
   hipStream_t s = (hipStream_t)stream;
 #define IRON_QKV(DD, C)                                                                             \
-  if (d == DD && ch == C)                                                                           \
-    hipLaunchKernelGGL((decode_qkv_kernel<DD, C>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
-                       angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row, angle_rows, \
-                       x_table, x_row, x_rows);
+  if (d == DD && ch == C) {                                                                         \
+    if (x_row == nullptr)                                                                           \
+      hipLaunchKernelGGL((decode_qkv_kernel<DD, C, false>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
+                         angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row,        \
+                         angle_rows, x_table, x_row, x_rows);                                                          \
+    else                                                                                            \
+      hipLaunchKernelGGL((decode_qkv_kernel<DD, C, true>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv,  \
+                         angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row,        \
+                         angle_rows, x_table, x_row, x_rows);                                                          \
+  }
   IRON_QKV(64, 1) IRON_QKV(64, 2) IRON_QKV(64, 4) IRON_QKV(128, 1) IRON_QKV(128, 2) IRON_QKV(128, 4)
 #undef IRON_QKV
   IRON_LAUNCH_CHECK();
