@@ -163,7 +163,7 @@ def bench_decode_kernels(torch, K, dev, n, rng):
     qkv_bytes = 2 * ((H + 2 * G) * D * E + 2 * E + (H + 2 * G) * D)
     caches = pool(2 * L * G * D * 2, lambda: (drawn(L, G, D, scale=1.0), drawn(L, G, D, scale=1.0)))
     ws = pool(qkv_bytes, lambda: (drawn(H * D, E), drawn(G * D, E), drawn(G * D, E)))
-    add("norm + q/k/v + RoPE + cache write", "decode_qkv_kernel<64,1>", 16, qkv_bytes,
+    add("norm + q/k/v + RoPE + cache write", "decode_qkv_kernel<64,1,false>", 16, qkv_bytes,
         [(lambda w=w, c=caches[i % len(caches)]: K.decode_qkv(x, gain, w[0], w[1], w[2], angles, q, c[0], c[1], eps=1e-5,
                                                                hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
                                                                position=position)) for i, w in enumerate(ws)])
@@ -189,13 +189,13 @@ def bench_decode_kernels(torch, K, dev, n, rng):
     del ws
     # down projection + residual
     ws = pool(2 * E * F, lambda: drawn(E, F))
-    add("down projection + residual", "gemv_fused_kernel<1,4,false,1>", 16, 2 * (E * F + F + 2 * E),
+    add("down projection + residual", "gemv_fused_kernel<2,4,false,1>", 16, 2 * (E * F + F + 2 * E),
         [(lambda w=w: K.gemv_fused(w, m, y, M=E, K=F, residual=x, epilogue=1)) for w in ws])
     del ws
     # final norm + head
     ws = pool(2 * V * E, lambda: drawn(V, E))
     logits = torch.empty(V, dtype=torch.bfloat16, device=dev)
-    add("final norm + LM head", "gemv_fused_kernel<4,1,true,0>", 1, 2 * (V * E + 2 * E + V),
+    add("final norm + LM head", "gemv_fused_kernel<2,1,true,0>", 1, 2 * (V * E + 2 * E + V),
         [(lambda w=w: K.gemv_fused(w, x, logits, M=V, K=E, norm_w=gain, eps=1e-5, epilogue=0)) for w in ws])
     del ws
     torch.cuda.empty_cache()
@@ -626,9 +626,9 @@ DOMINANT_TRAFFIC_SOURCE = ("profiles/llama1b_decode_step_hbm_counters.txt (rocpr
                            "arguments have changed since finds no entry and reports null)")
 DOMINANT_TRAFFIC_BYTES: dict[str, int] = {
     "gemv_fused_kernel<2,1,true,2>": 67_358_000,     # norm + gate/up + SiLU*mul: 67.227 MB fetched + 0.131 written
-    "gemv_fused_kernel<1,4,false,1>": 33_788_000,    # down projection + residual: 33.755 + 0.033
-    "gemv_fused_kernel<4,1,true,0>": 526_460_000,    # final norm + LM head: 525.43 + 1.03
-    "decode_qkv_kernel<64,1>": 12_750_000,           # norm + q/k/v + RoPE + cache rows: 12.70 + 0.05
+    "gemv_fused_kernel<2,4,false,1>": 33_788_000,    # down projection + residual: 33.755 + 0.033
+    "gemv_fused_kernel<2,1,true,0>": 526_460_000,    # final norm + LM head: 525.43 + 1.03
+    "decode_qkv_kernel<64,1,false>": 12_750_000,           # norm + q/k/v + RoPE + cache rows: 12.70 + 0.05
     "gemv_fused_kernel<1,1,false,1>": 8_500_000,     # o projection + residual: 8.47 + 0.03
 }
 

@@ -114,9 +114,11 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
   const int row0 = blockIdx.x * RPW;
   // The residual a thread will add at the end is requested first, so that its trip to memory
   // passes under the weights' instead of after the block's last barrier.
-  float res_ahead = 0.f;
-  if ((EPI == EPI_ADD || EPI == EPI_GELU_ROW || EPI == EPI_SILU_ROW) && threadIdx.x < RPW)
-    res_ahead = bf16_to_f32(res[min(row0 + (int)threadIdx.x, M - 1)]);
+  // (Every thread asks, the ones that add nothing for the block's last row again: behind a branch
+  // for the few that need it, the wave that took it would wait for the word then and there.)
+  bf16_t res_word = 0;
+  if (EPI == EPI_ADD || EPI == EPI_GELU_ROW || EPI == EPI_SILU_ROW)
+    res_word = res[min(row0 + min((int)threadIdx.x, RPW - 1), M - 1)];
   Activation<CH, NORM> act;
   act.issue(x, nw, K);
   uint4 w[MATS][RPW][CH];
@@ -140,6 +142,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
     const int r = threadIdx.x, row = row0 + r;
     if (row < M) {
       float v = round_bf16(part[0][0][r] + part[1][0][r] + part[2][0][r] + part[3][0][r]);  // the GEMV's own rounding
+      const float res_ahead = bf16_to_f32(res_word);
       if (EPI == EPI_ADD) v = fmaf(res_scale, v, res_ahead);   // scale 1: the plain sum
       if (EPI == EPI_GELU_ROW || EPI == EPI_SILU_ROW)          // the activation's own rounding, then the product's
         v = round_bf16(EPI == EPI_SILU_ROW ? silu_f32(v) : gelu_tanh_f32(v)) * res_ahead;
@@ -177,12 +180,6 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   else if (pair < q_pairs + k_pairs) { kind = 1; Wm = Wk; const int p = pair - q_pairs; const int h = p / HALF; j = p % HALF; r0 = h * D + j; r1 = r0 + HALF; }
   else { kind = 2; Wm = Wv; const int p = pair - q_pairs - k_pairs; r0 = 2 * p; r1 = r0 + 1; }
 
-  // `angles` is the step's row itself, or a whole table whose row a device word names (held inside).
-  if (angle_row != nullptr) angles += (size_t)max(0, min(*angle_row, angle_rows - 1)) * D;
-  // What the block's last thread needs after the last barrier is requested first: the pair's
-  // angle and the position word ride under the weights' trip to memory.
-  const float c_ahead = bf16_to_f32(angles[2 * j]), s_ahead = bf16_to_f32(angles[2 * j + 1]);
-  const int pos_ahead = *position;
   Activation<CH, true> act;
   uint4 w0[CH], w1[CH];
   if (!TABLE) {
@@ -206,6 +203,16 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
       }
     }
   }
+  // `angles` is the step's row itself, or a whole table whose row a device word names (held inside).
+  // What the block's last thread needs after the last barrier -- the pair's angle and the position
+  // word -- is asked for here, behind the rows' loads (the word that names the angles' row is a trip
+  // to memory of its own, which nothing above waits for) and under their trip to memory.
+  // (The two words pinned here, among the loads in flight: left free, the compiler moves the position's
+  // load down to its use after the last barrier, a trip to memory at the kernel's very end.)
+  int pos_ahead = *position, angle_at = angle_row != nullptr ? *angle_row : 0;
+  asm volatile("" : "+s"(pos_ahead), "+s"(angle_at));
+  angles += (size_t)max(0, min(angle_at, angle_rows - 1)) * D;
+  const float c_ahead = bf16_to_f32(angles[2 * j]), s_ahead = bf16_to_f32(angles[2 * j + 1]);
   float xf[CH][8];
   act.finish(eps, K, scratch4, xf);
   const float a0 = wave_sum(dot_row<CH>(w0, xf)), a1 = wave_sum(dot_row<CH>(w1, xf));
@@ -384,8 +391,13 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   const bool norm = norm_w != nullptr;
   IRON_REQUIRE(K <= 8 * 2048, "gemv_fused: K (%d) exceeds %d", K, 8 * 2048);
   const int ch = K <= 2048 ? 1 : (K <= 4096 ? 2 : (K <= 8192 ? 4 : 8));
-  // Rows a block takes: two where the matrix is tall and a row is short, else one.
-  const int rpw = (epilogue == EPI_SILU_MUL || epilogue == EPI_GELU_MUL) ? (ch == 1 ? 2 : 1) : (ch == 1 && M > 2048 ? (M >= 65536 ? 4 : 2) : 1);
+  // Rows a block takes (measured inside a decoder's step, on 256 CUs): two where the matrix is tall
+  // and a row is short, and for 16 KB rows of a matrix of a few thousand; else one.
+  const bool pair_of_matrices = epilogue == EPI_SILU_MUL || epilogue == EPI_GELU_MUL;
+  const bool plain_or_sum = epilogue == EPI_NONE || epilogue == EPI_ADD;
+  const int rpw = pair_of_matrices ? (ch == 1 ? 2 : 1)
+                  : (ch == 1 && M > 2048) ? 2
+                  : (ch == 4 && M >= 2048 && plain_or_sum) ? 2 : 1;
   const int blocks = (M + rpw - 1) / rpw;
 #define IRON_FUSED(R, C, NRM, E)                                                                   \
   if (rpw == R && ch == C && norm == NRM && epilogue == E) {                                       \
@@ -395,14 +407,14 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   }
 #define IRON_FUSED_NE(R, C)                                                                        \
   IRON_FUSED(R, C, false, 0) IRON_FUSED(R, C, true, 0) IRON_FUSED(R, C, false, 1) IRON_FUSED(R, C, true, 1)
-  IRON_FUSED_NE(1, 1) IRON_FUSED_NE(2, 1) IRON_FUSED_NE(4, 1) IRON_FUSED_NE(1, 2) IRON_FUSED_NE(1, 4) IRON_FUSED_NE(1, 8)
+  IRON_FUSED_NE(1, 1) IRON_FUSED_NE(2, 1) IRON_FUSED_NE(1, 2) IRON_FUSED_NE(1, 4) IRON_FUSED_NE(2, 4) IRON_FUSED_NE(1, 8)
   IRON_FUSED(2, 1, false, 2) IRON_FUSED(2, 1, true, 2) IRON_FUSED(1, 2, false, 2) IRON_FUSED(1, 2, true, 2)
   IRON_FUSED(1, 4, false, 2) IRON_FUSED(1, 4, true, 2) IRON_FUSED(1, 8, false, 2) IRON_FUSED(1, 8, true, 2)
   IRON_FUSED(2, 1, false, 3) IRON_FUSED(2, 1, true, 3) IRON_FUSED(1, 2, false, 3) IRON_FUSED(1, 2, true, 3)
   IRON_FUSED(1, 4, false, 3) IRON_FUSED(1, 4, true, 3) IRON_FUSED(1, 8, false, 3) IRON_FUSED(1, 8, true, 3)
   IRON_FUSED(1, 1, false, 4) IRON_FUSED(1, 2, false, 4) IRON_FUSED(1, 4, false, 4) IRON_FUSED(1, 8, false, 4)
   IRON_FUSED(1, 1, false, 5) IRON_FUSED(1, 2, false, 5) IRON_FUSED(1, 4, false, 5) IRON_FUSED(1, 8, false, 5)
-  IRON_FUSED(2, 1, false, 4) IRON_FUSED(4, 1, false, 4) IRON_FUSED(2, 1, false, 5) IRON_FUSED(4, 1, false, 5)
+  IRON_FUSED(2, 1, false, 4) IRON_FUSED(2, 1, false, 5)
 #undef IRON_FUSED_NE
 #undef IRON_FUSED
   IRON_REQUIRE(false, "gemv_fused: no kernel for this combination");
