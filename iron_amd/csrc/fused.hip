@@ -396,7 +396,7 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   const bool pair_of_matrices = epilogue == EPI_SILU_MUL || epilogue == EPI_GELU_MUL;
   const bool plain_or_sum = epilogue == EPI_NONE || epilogue == EPI_ADD;
   const int rpw = pair_of_matrices ? (ch == 1 ? 2 : 1)
-                  : (ch == 1 && M > 2048) ? 2
+                  : (ch == 1 && M > 2048) ? (M >= 65536 ? 4 : 2)
                   : (ch == 4 && M >= 2048 && plain_or_sum) ? 2 : 1;
   const int blocks = (M + rpw - 1) / rpw;
 #define IRON_FUSED(R, C, NRM, E)                                                                   \
@@ -407,7 +407,7 @@ extern "C" int iron_gemv_fused_bf16(const uint16_t* W, const uint16_t* W2, const
   }
 #define IRON_FUSED_NE(R, C)                                                                        \
   IRON_FUSED(R, C, false, 0) IRON_FUSED(R, C, true, 0) IRON_FUSED(R, C, false, 1) IRON_FUSED(R, C, true, 1)
-  IRON_FUSED_NE(1, 1) IRON_FUSED_NE(2, 1) IRON_FUSED_NE(1, 2) IRON_FUSED_NE(1, 4) IRON_FUSED_NE(2, 4) IRON_FUSED_NE(1, 8)
+  IRON_FUSED_NE(1, 1) IRON_FUSED_NE(2, 1) IRON_FUSED_NE(4, 1) IRON_FUSED_NE(1, 2) IRON_FUSED_NE(1, 4) IRON_FUSED_NE(2, 4) IRON_FUSED_NE(1, 8)
   IRON_FUSED(2, 1, false, 2) IRON_FUSED(2, 1, true, 2) IRON_FUSED(1, 2, false, 2) IRON_FUSED(1, 2, true, 2)
   IRON_FUSED(1, 4, false, 2) IRON_FUSED(1, 4, true, 2) IRON_FUSED(1, 8, false, 2) IRON_FUSED(1, 8, true, 2)
   IRON_FUSED(2, 1, false, 3) IRON_FUSED(2, 1, true, 3) IRON_FUSED(1, 2, false, 3) IRON_FUSED(1, 2, true, 3)
