@@ -603,6 +603,59 @@ def test_fused_kernels_against_the_oracle_at_llama_1b_width(cuda):
         close(lg, ops.gemv(Wh, n))
 
 
+@pytest.mark.parametrize("E,F,H,G,D", [(4096, 14336, 32, 8, 128), (3072, 8192, 24, 8, 128), (1992, 5000, 3, 1, 64),
+                                       (8192, 3000, 8, 8, 128), (264, 16384, 2, 2, 64)])
+def test_fused_kernels_at_other_widths(cuda, E, F, H, G, D):
+    """The one-row fusions where a row is not the 1B model's: two, four and eight chunks a thread,
+    rows whose last chunks a thread has none of (the bounded loads' zeros), an odd count of rows, and
+    rows shorter than a block's reach -- each against the oracle's steps composed on the host."""
+    import torch
+
+    from iron_amd import kernels as K
+    from iron_amd.bf16 import from_torch, round_bf16, to_torch
+    from oracle import ops
+
+    rng = np.random.default_rng(E + F)
+    L, pos = 16, 5
+
+    def bf(*shape, scale=1.0):
+        return round_bf16(rng.standard_normal(shape, dtype=np.float32) * np.float32(scale))
+
+    def dev(a):
+        return to_torch(a).to(cuda)
+
+    def close(got, want, atol=2e-2):
+        got = from_torch(got).reshape(want.shape)
+        assert np.all(np.abs(got - want) <= atol + 1e-2 * np.abs(want)), np.abs(got - want).max()
+
+    x, g = bf(E), round_bf16(rng.uniform(0.9, 1.1, E))
+    n = ops.rms_norm(x[None], g, epsilon=1e-5)[0]
+    Wq, Wk, Wv = bf(H * D, E, scale=0.02), bf(G * D, E, scale=0.02), bf(G * D, E, scale=0.02)
+    table = round_bf16(ops.rope_angles(D, L))
+    keys, values = dev(np.zeros((L, G, D), np.float32)), dev(np.zeros((L, G, D), np.float32))
+    q_out = torch.empty(H * D, dtype=torch.bfloat16, device=cuda)
+    K.decode_qkv(dev(x), dev(g), dev(Wq), dev(Wk), dev(Wv), dev(table), q_out, keys, values, eps=1e-5,
+                 hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
+                 position=torch.tensor([pos], dtype=torch.int32, device=cuda),
+                 angle_row=torch.tensor([pos], dtype=torch.int32, device=cuda))
+    close(q_out, ops.rope(ops.gemv(Wq, n).reshape(H, D), table[pos : pos + 1]).reshape(-1))
+    close(keys[pos], ops.rope(ops.gemv(Wk, n).reshape(G, D), table[pos : pos + 1]))
+    close(values[pos], ops.gemv(Wv, n).reshape(G, D))
+    Wg, Wu, Wd = bf(F, E, scale=0.02), bf(F, E, scale=0.02), bf(E, F, scale=0.02)
+    m = torch.empty(F, dtype=torch.bfloat16, device=cuda)
+    K.gemv_fused(dev(Wg), dev(x), m, M=F, K=E, W2=dev(Wu), norm_w=dev(g), eps=1e-5, epilogue=2)
+    want_m = ops.mul(ops.silu(ops.gemv(Wg, n)), ops.gemv(Wu, n))
+    close(m, want_m)
+    y = torch.empty(E, dtype=torch.bfloat16, device=cuda)
+    K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, residual=dev(x), epilogue=1)
+    close(y, ops.add(x, ops.gemv(Wd, want_m)))
+    K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, norm_w=None, epilogue=0)
+    close(y, ops.gemv(Wd, want_m))
+    row = bf(E)
+    K.gemv_fused(dev(Wd), dev(want_m), y, M=E, K=F, residual=dev(row), epilogue=5)
+    close(y, ops.mul(ops.silu(ops.gemv(Wd, want_m)), row))
+
+
 def test_biased_projections_match_hugging_face_on_the_gpu(cuda):
     """q, k, v and o with a bias (RowwiseAdd after each projection) against the reference's second
     golden fixture: prompt, greedy decode under the HIP graph, and a prompt of several chunks."""
