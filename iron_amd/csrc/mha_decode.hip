@@ -709,84 +709,6 @@ __global__ __launch_bounds__(4 * D) void mha_decode_either_merge_kernel(
   O[(size_t)head * D + t] = f32_to_bf16(ls > 0.f ? as / ls : 0.f);
 }
 
-// Many queries, a block a (query row, head): the same scan as above per query, over the keys its
-// mask leaves.  The shapes the MFMA prompt kernel does not take (512-wide heads: a 512-wide pair of
-// K and V tiles does not fit its stage buffers and registers); what a row costs is its keys' bytes.
-template <int D>
-__global__ __launch_bounds__(1024) void mha_prefill_rows_kernel(
-    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
-    bf16_t* __restrict__ O, int group, int seq, int seq_len, int kv_len, float scale_log2, int causal,
-    int window, long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
-    const int* __restrict__ valid, const int* __restrict__ kv_valid, const int* __restrict__ kv_first, int kv_rows) {
-  constexpr int LPR = D / 8, RW = 64 / LPR, WAVES = 16, U = 8;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int sub = lane % LPR, rg = lane / LPR;
-  const int head = blockIdx.x, row = blockIdx.y, kvh = head / group;
-  if (kv_first) {   // the keys are a window of a longer buffer, rows *kv_first on (held inside it)
-    const long first_row = max(0, min(*kv_first, kv_rows - kv_len));
-    K += first_row * kv_row_stride;
-    V += first_row * kv_row_stride;
-  }
-
-  const int q_tokens = valid ? bound_or(valid, seq) : seq_len;
-  const int kv_tokens = kv_valid ? bound_or(kv_valid, kv_len) : (kv_len - seq + q_tokens);
-  const bool masked = causal || window >= 0;
-  const int offset = masked ? (kv_tokens - q_tokens) : 0;
-  bf16_t* out = O + (size_t)head * q_head_stride + (size_t)row * q_row_stride;
-  if (row >= q_tokens || offset < 0) {   // a row past the bound: zeros
-    if (threadIdx.x < D) out[threadIdx.x] = 0;
-    return;
-  }
-  const int qpos = offset + row;
-  int hi = kv_tokens, lo = 0;
-  if (causal) hi = min(hi, qpos + 1);
-  else if (window >= 0) hi = min(hi, qpos + window + 1);
-  if (window >= 0) lo = max(0, qpos - window);
-
-  float m[1], l[1], acc[1][8];
-  decode_scan<D, 1, U, false>(Q + (size_t)head * q_head_stride + (size_t)row * q_row_stride,
-                              K + (size_t)kvh * kv_head_stride, V + (size_t)kvh * kv_head_stride, 0,
-                              lo + wave * U * RW, hi, WAVES * U * RW, kv_row_stride, scale_log2, m, l, acc);
-
-  __shared__ float sm[WAVES];
-  __shared__ float sl[WAVES];
-  __shared__ float sacc[WAVES][D];
-  if (rg == 0) {
-    if (sub == 0) {
-      sm[wave] = m[0];
-      sl[wave] = l[0];
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) sacc[wave][sub * 8 + i] = acc[0][i];
-  }
-  __syncthreads();
-  if (threadIdx.x < D) {
-    const int dd = threadIdx.x;
-    float mx = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, sm[w]);
-    const float ref = (mx == -INFINITY) ? 0.f : mx;
-    float lt = 0.f, at = 0.f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      const float e = exp2f(sm[w] - ref);
-      lt += sl[w] * e;
-      at += sacc[w][dd] * e;
-    }
-    out[dd] = f32_to_bf16(lt > 0.f ? at / lt : 0.f);
-  }
-}
-
-int launch_prefill_rows512(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, int heads, int group,
-                           int seq, int seq_len, int kv_len, float scale_log2, int causal, int window,
-                           long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
-                           const int* valid, const int* kv_valid, const int* kv_first, int kv_rows, void* stream) {
-  hipLaunchKernelGGL(mha_prefill_rows_kernel<512>, dim3(heads, seq), dim3(1024), 0, (hipStream_t)stream, Q, K, V, O,
-                     group, seq, seq_len, kv_len, scale_log2, causal, window, q_row_stride, q_head_stride,
-                     kv_row_stride, kv_head_stride, valid, kv_valid, kv_first, kv_rows);
-  return 0;
-}
-
 template <int D, int G>
 static void launch_decode(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, float* part,
                           int kv_heads, int kv_len, float scale_log2, int window, long row_stride,

@@ -386,6 +386,252 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   }
 }
 
+// ---- 512-wide heads (Gemma 4's global layers)
+//
+// A 64-key tile pair of 512-wide rows, or a wave's 32 queries of output, fit neither the stages nor
+// the registers of the kernel above.  Here a wave owns 16 queries, the columns of a 16-wide MFMA tile
+// (v_mfma_f32_16x16x32_bf16), as the G heads of a KV group are in decode attention: S^T = K Q^T over
+// 32-key tiles (two 16-key MFMA tiles, the 512 columns in 16 k-steps, Q^T held in registers), a lane
+// then owns one query column, its four lanes exchanging their maximum only when one passes the
+// column's reference; the probabilities, rounded to bf16, are the B operand of O^T = V^T P^T as they
+// stand, and O^T is 32 tiles of 16 output columns, 128 accumulator registers a lane.  A block is eight
+// waves (128 queries of one head) that share the K and V tiles: 32 keys x 1 KB each, two stages of
+// 64 KB, sent from global memory straight into LDS a row an instruction; a row's 16-byte chunks are
+// XORed by key & 15 in K (a fragment read is 16 keys at one chunk: all banks once) and by
+// 2 (key & 3) in V (the transposing read).  Masks, bounds and the block order are the kernel's above.
+template <int D>
+__global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
+    const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
+    bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
+    int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
+    long kv_head_stride, const int* __restrict__ valid, const int* __restrict__ kv_valid,
+    const int* __restrict__ kv_first, int kv_rows) {
+  constexpr int ROWB = D * 2;            // bytes of a tile row
+  constexpr int KS = D / 32;             // 32-wide k-steps of S^T
+  constexpr int DT = D / 16;             // 16-row tiles of O^T
+  constexpr int CPR = D / 8;             // 16-byte chunks a row has
+  constexpr int TK = 32;                 // keys a tile
+  constexpr int W = 8;                   // waves: two a SIMD, which holds a wave to 256 registers, all of them ordinary
+  constexpr int BQW = 16 * W;            // queries of a block
+  constexpr int TILE = TK * ROWB;
+  constexpr int STAGE = 2 * TILE;
+  constexpr int INST = TK / W;           // rows of K (and of V) a wave loads per tile, one an instruction
+  static_assert(CPR == 64, "a row is one 1 KB load: 64 lanes x 16 bytes");
+  extern __shared__ __align__(1024) char smem_wide[];   // 2 * STAGE bytes
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, q = lane >> 4;   // query column, quarter of the k slots
+  const int j = blockIdx.x % heads;
+  const int head = (heads % 8 == 0) ? (j % 8) * (heads / 8) + j / 8 : j;
+  const int kvh = head / group;
+  const int qb = (int)(gridDim.x / heads) - 1 - (int)(blockIdx.x / heads);
+  const int q0 = qb * BQW;
+
+  const int q_tokens = valid ? bound_or(valid, seq) : seq_len;
+  const int kv_tokens = kv_valid ? bound_or(kv_valid, kv_len) : (kv_len - seq + q_tokens);
+  const bool masked_any = causal || window >= 0;
+  const int offset = masked_any ? (kv_tokens - q_tokens) : 0;
+
+  const int my_q = q0 + wave * 16 + n;
+  const bool q_live = my_q < q_tokens;
+  const int qpos = offset + my_q;
+  const int wq_lo = offset + q0 + wave * 16;
+  const int wq_hi = offset + min(q0 + wave * 16 + 15, q_tokens - 1);
+
+  bf16_t* Oh = O + (size_t)head * q_head_stride;
+  if (q0 >= q_tokens || offset < 0) {   // rows of this block past the bound: zeros
+    for (int i = tid; i < BQW * CPR; i += 64 * W) {
+      const int r = q0 + i / CPR, c = (i % CPR) * 8;
+      if (r < seq) *reinterpret_cast<uint4*>(Oh + (size_t)r * q_row_stride + c) = make_uint4(0, 0, 0, 0);
+    }
+    return;
+  }
+
+  // Q^T fragments (B operand): lane holds query n, d = 32 s + 8 q .. + 7.
+  bf16x8 qf[KS];
+  {
+    const bf16_t* qp = Q + (size_t)head * q_head_stride + (size_t)my_q * q_row_stride + 8 * q;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (q_live) v = *reinterpret_cast<const uint4*>(qp + 32 * s);
+      qf[s] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  f32x4 oacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_ref = -INFINITY, l_run = 0.f;   // the column's reference maximum (raw scores), this lane's sum
+
+  const int q_last = min(q0 + BQW, q_tokens) - 1;
+  int kv_hi = kv_tokens;
+  if (causal) kv_hi = min(kv_hi, offset + q_last + 1);
+  else if (window >= 0) kv_hi = min(kv_hi, offset + q_last + window + 1);
+  int kv_lo = 0;
+  if (window >= 0) kv_lo = max(0, offset + q0 - window) / TK * TK;
+  const int ntiles = (kv_hi - kv_lo + TK - 1) / TK;
+
+  if (ntiles > 0) {
+    const long first_row = kv_first ? max(0, min(*kv_first, kv_rows - kv_len)) : 0;
+    const bf16_t* Kh = K + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
+    const bf16_t* Vh = V + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
+    const int row_bytes = (int)kv_row_stride * 2;
+    // Load i of a wave is tile row wave INST + i: lane l lands at physical chunk l and fetches the
+    // logical chunk the row's swizzle maps there (the offsets are made where they are used: two
+    // vector instructions a load, against sixteen registers held through the loop).
+    const int lane16 = lane << 4;
+    const int reach = (kv_tokens - kv_lo - 1) * row_bytes + ROWB;
+    const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(Kh + (long)kv_lo * kv_row_stride), 0, reach, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(Vh + (long)kv_lo * kv_row_stride), 0, reach, 0x00020000);
+    const int tile_bytes = TK * row_bytes;
+    auto issue = [&](int tile, int buf) {
+      char* st = smem_wide + buf * STAGE;
+      const int at = tile * tile_bytes;
+#pragma unroll
+      for (int i = 0; i < INST; ++i) {
+        const int r = wave * INST + i, row_at = at + r * row_bytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rows, IRON_LDS_PTR(st + r * 1024), 16,
+                                                 (int)(lane16 ^ ((r & 15) << 4)) + row_at, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rows, IRON_LDS_PTR(st + TILE + r * 1024), 16,
+                                                 (int)(lane16 ^ ((r & 3) << 5)) + row_at, 0, 0, 0);
+      }
+    };
+    issue(0, 0);
+
+    // K fragment (tile t, k-step s): key 16 t + n, logical chunk 4 s + q, physical (4 s + q) ^ n: with
+    // s = 4 a + b that is 16 a + (4 (b ^ (n >> 2)) | (q ^ (n & 3))) -- four bases a lane, the rest immediates.
+    int k_frag[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) k_frag[b] = n * ROWB + (((4 * (b ^ (n >> 2))) | (q ^ (n & 3))) << 4);
+    // V^T fragment (output tile dt): the lanes of quarter q point at key rows 4 q + 0..3 (k slots
+    // 8 q + 0..3; the same 16 rows on for slots 8 q + 4..7, as S^T's second tile lies in P), 4 of the
+    // tile's 16 columns each; chunk 2 dt + (lane & 3) / 2, swizzled.  dt = 4 k + r: four bases, 128 k on.
+    const int v_swz = ((lane >> 2) & 3) << 1;
+    const unsigned lds_base = (unsigned)(size_t)IRON_LDS_PTR(smem_wide);
+    unsigned v_frag[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      v_frag[r] = lds_base + TILE + (4 * q + ((lane & 15) >> 2)) * ROWB +
+                  (((2 * r + ((lane & 3) >> 1)) ^ v_swz) << 4) + ((lane & 1) << 3);
+
+    // The keys this lane's query may see: one range of positions for the whole loop.
+    int see_hi = kv_tokens - 1, see_lo = 0;
+    if (causal) see_hi = min(see_hi, qpos);
+    else if (window >= 0) see_hi = min(see_hi, qpos + window);
+    if (window >= 0) see_lo = max(0, qpos - window);
+    const unsigned see_span = see_hi >= see_lo ? (unsigned)(see_hi - see_lo) : 0u;
+    if (see_hi < see_lo) see_lo = 1 << 30;
+
+    auto tile_step = [&](int tile, auto buf_c) {
+      constexpr int buf = decltype(buf_c)::value;
+      const int kv0 = kv_lo + tile * TK;
+      wait_vmcnt<0>();    // this wave's share of the tile has landed
+      block_barrier();    // everyone's has; everyone is done with the tile before
+      issue(min(tile + 1, ntiles - 1), buf ^ 1);
+      if (causal && kv0 > wq_hi) return;   // the tile lies past every query of this wave
+      const char* kt = smem_wide + buf * STAGE;
+      // S^T = K Q^T for the tile's two 16-key halves.
+      f32x4 sacc[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        sacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int a = 0; a < KS / 4; ++a) {
+          bf16x8 kf[4];
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            kf[b] = *reinterpret_cast<const bf16x8*>(kt + k_frag[b] + t * 16 * ROWB + a * 256);
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b], qf[4 * a + b], sacc[t], 0, 0, 0);
+        }
+      }
+      // Element i of half t is key kv0 + 16 t + 4 q + i, query n.
+      bool edge = kv0 + TK > kv_tokens;
+      if (causal) edge |= kv0 + TK - 1 > wq_lo;
+      else if (window >= 0) edge |= kv0 + TK - 1 > wq_lo + window;
+      if (window >= 0) edge |= kv0 < wq_hi - window;
+      bool out[2][4];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          out[t][i] = edge && (unsigned)(kv0 + 16 * t + 4 * q + i - see_lo) > see_span;
+          if (out[t][i]) sacc[t][i] = -INFINITY;
+        }
+      float lm = sacc[0][0];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lm = fmaxf(lm, sacc[t][i]);
+      if (__builtin_amdgcn_ballot_w64(lm > m_ref) != 0) {
+        float mx = fmaxf(lm, __shfl_xor(lm, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_ref, mx);
+        // A column that had seen no key has zero sums to rescale; one that still has none keeps -inf.
+        const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_ref - m_new) * scale_log2);
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
+        m_ref = m_new;
+      }
+      const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * scale_log2;
+      float p[8];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float e = __builtin_amdgcn_exp2f(fmaf(sacc[t][i], scale_log2, -mc));
+          if (out[t][i]) e = 0.f;   // also where the scale is 0 and -inf * 0 is no number
+          p[4 * t + i] = e;
+          l_run += e;
+        }
+      const bf16x8 pf = __builtin_bit_cast(bf16x8, pack8(p));
+      // O^T += V^T P^T, four output tiles' fragments requested at a time.
+#pragma unroll
+      for (int k = 0; k < DT / 4; ++k) {
+        TrFrag vf[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const unsigned at = v_frag[r] + (buf * STAGE + 128 * k);
+          vf[r].lo = lds_read_tr16_at<0>(at);
+          vf[r].hi = lds_read_tr16_at<16 * ROWB>(at);
+        }
+        lds_tr_wait(vf[0], vf[1]);
+        lds_tr_wait(vf[2], vf[3]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          oacc[4 * k + r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tr_join(vf[r]), pf, oacc[4 * k + r], 0, 0, 0);
+      }
+    };
+    using buf0 = std::integral_constant<int, 0>;
+    using buf1 = std::integral_constant<int, 1>;
+    for (int tile = 0; tile < ntiles; tile += 2) {
+      tile_step(tile, buf0{});
+      if (tile + 1 < ntiles) tile_step(tile + 1, buf1{});
+    }
+    wait_vmcnt<0>();   // the idle fetch of the last iteration lands before the block's LDS is released
+  }
+
+  // The lane's sum over its own keys -> the column's; normalize and store: lane holds query n,
+  // columns 16 dt + 4 q + 0..3.
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  const float inv = (q_live && l_run > 0.f) ? 1.0f / l_run : 0.f;
+  if (my_q < seq) {
+    bf16_t* op = Oh + (size_t)my_q * q_row_stride + 4 * q;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<uint2*>(op + 16 * dt) = make_uint2(pack_bf16(oacc[dt][0] * inv, oacc[dt][1] * inv),
+                                                           pack_bf16(oacc[dt][2] * inv, oacc[dt][3] * inv));
+  }
+}
+
 struct PrefillArgs {
   const uint16_t *Q, *K, *V;
   uint16_t* O;
@@ -413,12 +659,6 @@ static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
                      a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid, a.kv_first, a.kv_rows);
   return 0;
 }
-
-// Row-wise attention for 512-wide heads (mha_decode.hip).
-int launch_prefill_rows512(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, int heads, int group,
-                           int seq, int seq_len, int kv_len, float scale_log2, int causal, int window,
-                           long q_row_stride, long q_head_stride, long kv_row_stride, long kv_head_stride,
-                           const int* valid, const int* kv_valid, const int* kv_first, int kv_rows, void* stream);
 
 }  // namespace iron
 
@@ -452,11 +692,15 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
                (long)kv_len * kv_row * 2);
   const float scale_log2 = scale * 1.4426950408889634f;
   if (d == 512) {
-    IRON_REQUIRE(seq <= 65535, "mha_prefill: at d = 512 seq (%d) is a grid dimension, at most 65535", seq);
-    const int rc512 = launch_prefill_rows512(Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal,
-                                             window, q_row, q_head, kv_row, kv_head, valid, kv_valid, kv_first, kv_rows,
-                                             stream);
-    if (rc512 != 0) return rc512;
+    constexpr size_t lds = 2 * 2 * 32 * 512 * 2;   // two stages of a 32-key K tile and V tile
+    static LdsOptIn opt_in;
+    if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_prefill_wide_kernel<512>), lds); e != hipSuccess) {
+      set_error("mha_prefill: %s", hipGetErrorString(e));
+      return (int)e;
+    }
+    hipLaunchKernelGGL(mha_prefill_wide_kernel<512>, dim3(((seq + 127) / 128) * heads), dim3(512), lds, (hipStream_t)stream, Q, K,
+                       V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window, q_row, q_head,
+                       kv_row, kv_head, valid, kv_valid, kv_first, kv_rows);
     IRON_LAUNCH_CHECK();
   }
   const int blocks = ((seq + BQ - 1) / BQ) * heads;

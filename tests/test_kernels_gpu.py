@@ -740,6 +740,35 @@ def test_mha_prefill_d256_ragged_windowed_and_bounded(cuda):
     close(got[:rows], want[:rows])
 
 
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_mha_prefill_512_wide_heads_over_many_tiles(cuda, interleaved):
+    """512-wide heads past a block's 64 queries and a tile's 32 keys: several heads a KV head, a ragged
+    causal sequence, a window that drops whole tiles, no mask at all, a chunk at the end of a longer
+    cache under bounds on both sides, and an unscaled product."""
+    rng = np.random.default_rng(24)
+    H, G, d, S = 4, 2, 512, 333
+    Q, Kc, Vc = bf(rng, S, H, d) * 0.25, bf(rng, S, G, d) * 0.25, bf(rng, S, G, d)
+    if not interleaved:
+        Q, Kc, Vc = (np.ascontiguousarray(a.transpose(1, 0, 2)) for a in (Q, Kc, Vc))
+    for causal, window in ((True, None), (True, 70), (False, 45), (False, None)):
+        got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=S, causal=causal,
+                                window=window, interleaved=interleaved)
+        close(got, want)
+    C, L, rows, kv = 192, 700, 130, 611
+    Q, Kc, Vc = bf(rng, C, H, d) * 0.25, bf(rng, L, G, d) * 0.25, bf(rng, L, G, d)
+    Q[rows:], Kc[kv:], Vc[kv:] = np.nan, np.nan, np.nan
+    if not interleaved:
+        Q, Kc, Vc = (np.ascontiguousarray(a.transpose(1, 0, 2)) for a in (Q, Kc, Vc))
+    got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=C, seq_len=C, kv_len=L, valid=rows, kv_valid=kv,
+                            scale=1.0, interleaved=interleaved)
+    if interleaved:
+        assert np.all(got[rows:] == 0)
+        close(got[:rows], want[:rows])
+    else:
+        assert np.all(got[:, rows:] == 0)
+        close(got[:, :rows], want[:, :rows])
+
+
 @pytest.mark.parametrize("d,H,G", [(64, 8, 2), (128, 4, 1), (256, 4, 1), (512, 4, 1)])
 def test_mha_over_a_window_of_a_longer_buffer(cuda, d, H, G):
     """Keys that are a run of rows of a longer buffer, from a row a device word names (a ring cache's
@@ -787,8 +816,8 @@ def test_mha_over_a_window_of_a_longer_buffer(cuda, d, H, G):
 
 
 def test_mha_512_wide_heads_prefill_and_decode(cuda):
-    """512-wide heads (a global layer's of Gemma 4): the row-wise prompt kernel under every mask and
-    a bound, and the one-query kernel on either side of 2048 keys."""
+    """512-wide heads (a global layer's of Gemma 4): the prompt kernel under every mask and a bound,
+    and the one-query kernel on either side of 2048 keys."""
     rng = np.random.default_rng(22)
     H, G, d, S, L = 4, 1, 512, 70, 200
     Q, Kc, Vc = bf(rng, S, H, d) * 0.25, bf(rng, L, G, d) * 0.25, bf(rng, L, G, d)
