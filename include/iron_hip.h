@@ -232,8 +232,8 @@ int iron_softmax_bf16(const void* x, int x_is_f32, const float* addend, uint16_t
  * q_tokens = *valid (or seq_len), kv_tokens = *kv_valid (or kv_len - seq + q_tokens).
  * causal masks key > position; window >= 0 also masks key < position - window (and, when not
  * causal, key > position + window); window < 0 = none.  Rows >= q_tokens of O are zeros.
- * d in {64, 128, 256, 512} (MFMA tiles throughout: 32 queries a wave on 32x32x16 tiles up to 256,
- * 16 a wave on 16x16x32 tiles at 512); heads % kv_heads == 0.
+ * d in {64, 128, 256, 512} (MFMA tiles throughout: 32 queries a wave on 32x32x16 tiles at 64 and
+ * 128, groups of 16 on 16x16x32 tiles at 256 and 512); heads % kv_heads == 0.
  * Replaces kernels.linalg.mha + partial_softmax + matmul_PV:
  * iron/operators/mha.py:191,574-667,1073-1116. */
 int iron_mha_prefill_bf16(const uint16_t* Q, const uint16_t* K, const uint16_t* V, uint16_t* O,

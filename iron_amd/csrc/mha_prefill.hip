@@ -30,6 +30,7 @@ __device__ __forceinline__ float max_with_other_half(float x) {
 constexpr int BQ = 128;   // query rows per block (four waves of 32; 64 where a block is two)
 constexpr int BKV = 64;   // key rows per tile
 constexpr int kFewBlocks = 256;          // launches of fewer blocks than this halve their blocks' queries
+constexpr int kWideBigBlocks = 512;     // wide heads: launches of at least this many 128-query blocks keep that size
 constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks split each block's tiles over two halves
 
 // K and V tiles go straight from global memory into LDS (buffer loads with the LDS bit, no register staging), as
@@ -50,7 +51,7 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 // W: the waves that share a tile's loads, each with 32 of the block's 32 W queries.  Four; two
 // where four would leave CUs without a block (a short prompt), so that twice as many blocks go out.
 template <int D, int SPLIT, int W = 4>
-__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(D <= 128 && W == 4 ? 2 : 1))) void mha_prefill_kernel(
+__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(W == 4 ? 2 : 1))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -386,21 +387,26 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   }
 }
 
-// ---- 512-wide heads (Gemma 4's global layers)
+// ---- 256- and 512-wide heads (Gemma's)
 //
-// A 64-key tile pair of 512-wide rows, or a wave's 32 queries of output, fit neither the stages nor
-// the registers of the kernel above.  Here a wave owns 16 queries, the columns of a 16-wide MFMA tile
-// (v_mfma_f32_16x16x32_bf16), as the G heads of a KV group are in decode attention: S^T = K Q^T over
-// 32-key tiles (two 16-key MFMA tiles, the 512 columns in 16 k-steps, Q^T held in registers), a lane
-// then owns one query column, its four lanes exchanging their maximum only when one passes the
-// column's reference; the probabilities, rounded to bf16, are the B operand of O^T = V^T P^T as they
-// stand, and O^T is 32 tiles of 16 output columns, 128 accumulator registers a lane.  A block is eight
-// waves (128 queries of one head) that share the K and V tiles: 32 keys x 1 KB each, two stages of
-// 64 KB, sent from global memory straight into LDS a row an instruction; a row's 16-byte chunks are
+// A 64-key tile pair of 512-wide rows, or a wave's 32 queries of 512-wide output, fit neither the
+// stages nor the registers of the kernel above (and at 256 it is down to one wave a SIMD).  Here a
+// wave owns QN groups of 16 queries, each the columns of a 16-wide MFMA tile
+// (v_mfma_f32_16x16x32_bf16), as the heads of a KV group are in decode attention: S^T = K Q^T over
+// 32-key tiles (two 16-key MFMA tiles, the D columns in D / 32 k-steps, Q^T held in registers), a
+// lane then owns one query column a group, its four lanes exchanging their maximum only when one
+// passes the column's reference; the probabilities, rounded to bf16, are the B operand of
+// O^T = V^T P^T as they stand, and O^T is D / 16 tiles of 16 output columns a group.  One group at
+// 512 and two at 256 are the same 128 accumulator and 64 Q^T registers a lane; with two, every K and
+// V^T fragment read out of LDS serves two MFMAs (the LDS reads are what bounds the kernel).  W waves
+// (16 QN W queries of one head; two waves a SIMD, which holds a wave to 256 registers, all of them
+// ordinary -- given 512 the compiler kept the accumulators in accumulation registers and copied all
+// 128 around the conditional rescale on every tile) share the K and V tiles: 32 keys each, two
+// stages, sent from global memory straight into LDS 1 KB an instruction; a row's 16-byte chunks are
 // XORed by key & 15 in K (a fragment read is 16 keys at one chunk: all banks once) and by
 // 2 (key & 3) in V (the transposing read).  Masks, bounds and the block order are the kernel's above.
-template <int D>
-__global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
+template <int D, int QN, int W>
+__global__ __launch_bounds__(64 * W, 2) void mha_prefill_wide_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -411,12 +417,13 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
   constexpr int DT = D / 16;             // 16-row tiles of O^T
   constexpr int CPR = D / 8;             // 16-byte chunks a row has
   constexpr int TK = 32;                 // keys a tile
-  constexpr int W = 8;                   // waves: two a SIMD, which holds a wave to 256 registers, all of them ordinary
-  constexpr int BQW = 16 * W;            // queries of a block
+  constexpr int WQ = 16 * QN;            // queries of a wave
+  constexpr int BQW = WQ * W;            // and of a block
   constexpr int TILE = TK * ROWB;
   constexpr int STAGE = 2 * TILE;
-  constexpr int INST = TK / W;           // rows of K (and of V) a wave loads per tile, one an instruction
-  static_assert(CPR == 64, "a row is one 1 KB load: 64 lanes x 16 bytes");
+  constexpr int RPI = 1024 / ROWB;       // rows a 1 KB load covers
+  constexpr int INST = TK / RPI / W;     // loads of K (and of V) a wave issues per tile
+  static_assert(CPR * RPI == 64 && INST >= 1 && KS % 4 == 0 && DT % 4 == 0, "the tile splits into whole 1 KB loads a wave");
   extern __shared__ __align__(1024) char smem_wide[];   // 2 * STAGE bytes
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -433,11 +440,16 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
   const bool masked_any = causal || window >= 0;
   const int offset = masked_any ? (kv_tokens - q_tokens) : 0;
 
-  const int my_q = q0 + wave * 16 + n;
-  const bool q_live = my_q < q_tokens;
-  const int qpos = offset + my_q;
-  const int wq_lo = offset + q0 + wave * 16;
-  const int wq_hi = offset + min(q0 + wave * 16 + 15, q_tokens - 1);
+  int my_q[QN], qpos[QN];
+  bool q_live[QN];
+#pragma unroll
+  for (int u = 0; u < QN; ++u) {
+    my_q[u] = q0 + wave * WQ + 16 * u + n;
+    q_live[u] = my_q[u] < q_tokens;
+    qpos[u] = offset + my_q[u];
+  }
+  const int wq_lo = offset + q0 + wave * WQ;
+  const int wq_hi = offset + min(q0 + wave * WQ + WQ - 1, q_tokens - 1);
 
   bf16_t* Oh = O + (size_t)head * q_head_stride;
   if (q0 >= q_tokens || offset < 0) {   // rows of this block past the bound: zeros
@@ -448,21 +460,27 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
     return;
   }
 
-  // Q^T fragments (B operand): lane holds query n, d = 32 s + 8 q .. + 7.
-  bf16x8 qf[KS];
-  {
-    const bf16_t* qp = Q + (size_t)head * q_head_stride + (size_t)my_q * q_row_stride + 8 * q;
+  // Q^T fragments (B operand): lane holds query n of its group, d = 32 s + 8 q .. + 7.
+  bf16x8 qf[QN][KS];
+#pragma unroll
+  for (int u = 0; u < QN; ++u) {
+    const bf16_t* qp = Q + (size_t)head * q_head_stride + (size_t)my_q[u] * q_row_stride + 8 * q;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       uint4 v = make_uint4(0, 0, 0, 0);
-      if (q_live) v = *reinterpret_cast<const uint4*>(qp + 32 * s);
-      qf[s] = __builtin_bit_cast(bf16x8, v);
+      if (q_live[u]) v = *reinterpret_cast<const uint4*>(qp + 32 * s);
+      qf[u][s] = __builtin_bit_cast(bf16x8, v);
     }
   }
-  f32x4 oacc[DT];
+  f32x4 oacc[QN][DT];
+  float m_ref[QN], l_run[QN];   // a column's reference maximum (raw scores), this lane's sum
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_ref = -INFINITY, l_run = 0.f;   // the column's reference maximum (raw scores), this lane's sum
+  for (int u = 0; u < QN; ++u) {
+    m_ref[u] = -INFINITY;
+    l_run[u] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[u][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   const int q_last = min(q0 + BQW, q_tokens) - 1;
   int kv_hi = kv_tokens;
@@ -477,10 +495,14 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
     const bf16_t* Kh = K + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
     const bf16_t* Vh = V + (size_t)kvh * kv_head_stride + first_row * kv_row_stride;
     const int row_bytes = (int)kv_row_stride * 2;
-    // Load i of a wave is tile row wave INST + i: lane l lands at physical chunk l and fetches the
-    // logical chunk the row's swizzle maps there (the offsets are made where they are used: two
-    // vector instructions a load, against sixteen registers held through the loop).
-    const int lane16 = lane << 4;
+    // Load i of a wave covers tile rows (wave INST + i) RPI + lane / CPR: a lane lands at physical
+    // chunk lane % CPR of its row and fetches the logical chunk the row's swizzle maps there.  The
+    // first row of a load is even where a load has two, so the row's low bit is the lane's own and
+    // the rest of the swizzle is the load's (a scalar): two vector instructions a load, made where
+    // they are used, against sixteen registers held through the loop.
+    const int l_row = lane / CPR, l_ch = lane % CPR;
+    const int k_lane = l_row * row_bytes + ((l_ch ^ l_row) << 4);
+    const int v_lane = l_row * row_bytes + ((l_ch ^ (l_row << 1)) << 4);
     const int reach = (kv_tokens - kv_lo - 1) * row_bytes + ROWB;
     const __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t*>(Kh + (long)kv_lo * kv_row_stride), 0, reach, 0x00020000);
@@ -492,11 +514,11 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
       const int at = tile * tile_bytes;
 #pragma unroll
       for (int i = 0; i < INST; ++i) {
-        const int r = wave * INST + i, row_at = at + r * row_bytes;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rows, IRON_LDS_PTR(st + r * 1024), 16,
-                                                 (int)(lane16 ^ ((r & 15) << 4)) + row_at, 0, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rows, IRON_LDS_PTR(st + TILE + r * 1024), 16,
-                                                 (int)(lane16 ^ ((r & 3) << 5)) + row_at, 0, 0, 0);
+        const int piece = wave * INST + i, r = piece * RPI, row_at = at + r * row_bytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rows, IRON_LDS_PTR(st + piece * 1024), 16,
+                                                 (int)(k_lane ^ ((r & 15) << 4)) + row_at, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rows, IRON_LDS_PTR(st + TILE + piece * 1024), 16,
+                                                 (int)(v_lane ^ ((r & 3) << 5)) + row_at, 0, 0, 0);
       }
     };
     issue(0, 0);
@@ -517,13 +539,19 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
       v_frag[r] = lds_base + TILE + (4 * q + ((lane & 15) >> 2)) * ROWB +
                   (((2 * r + ((lane & 3) >> 1)) ^ v_swz) << 4) + ((lane & 1) << 3);
 
-    // The keys this lane's query may see: one range of positions for the whole loop.
-    int see_hi = kv_tokens - 1, see_lo = 0;
-    if (causal) see_hi = min(see_hi, qpos);
-    else if (window >= 0) see_hi = min(see_hi, qpos + window);
-    if (window >= 0) see_lo = max(0, qpos - window);
-    const unsigned see_span = see_hi >= see_lo ? (unsigned)(see_hi - see_lo) : 0u;
-    if (see_hi < see_lo) see_lo = 1 << 30;
+    // The keys a lane's query may see: one range of positions for the whole loop.
+    int see_lo[QN];
+    unsigned see_span[QN];
+#pragma unroll
+    for (int u = 0; u < QN; ++u) {
+      int see_hi = kv_tokens - 1;
+      see_lo[u] = 0;
+      if (causal) see_hi = min(see_hi, qpos[u]);
+      else if (window >= 0) see_hi = min(see_hi, qpos[u] + window);
+      if (window >= 0) see_lo[u] = max(0, qpos[u] - window);
+      see_span[u] = see_hi >= see_lo[u] ? (unsigned)(see_hi - see_lo[u]) : 0u;
+      if (see_hi < see_lo[u]) see_lo[u] = 1 << 30;
+    }
 
     auto tile_step = [&](int tile, auto buf_c) {
       constexpr int buf = decltype(buf_c)::value;
@@ -533,11 +561,12 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
       issue(min(tile + 1, ntiles - 1), buf ^ 1);
       if (causal && kv0 > wq_hi) return;   // the tile lies past every query of this wave
       const char* kt = smem_wide + buf * STAGE;
-      // S^T = K Q^T for the tile's two 16-key halves.
-      f32x4 sacc[2];
+      // S^T = K Q^T for the tile's two 16-key halves, every K fragment for all the wave's groups.
+      f32x4 sacc[QN][2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        sacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < QN; ++u) sacc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int a = 0; a < KS / 4; ++a) {
           bf16x8 kf[4];
@@ -546,53 +575,59 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
             kf[b] = *reinterpret_cast<const bf16x8*>(kt + k_frag[b] + t * 16 * ROWB + a * 256);
 #pragma unroll
           for (int b = 0; b < 4; ++b)
-            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b], qf[4 * a + b], sacc[t], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < QN; ++u)
+              sacc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b], qf[u][4 * a + b], sacc[u][t], 0, 0, 0);
         }
       }
-      // Element i of half t is key kv0 + 16 t + 4 q + i, query n.
+      // Element i of half t is key kv0 + 16 t + 4 q + i, query n of the group.
       bool edge = kv0 + TK > kv_tokens;
       if (causal) edge |= kv0 + TK - 1 > wq_lo;
       else if (window >= 0) edge |= kv0 + TK - 1 > wq_lo + window;
       if (window >= 0) edge |= kv0 < wq_hi - window;
-      bool out[2][4];
+      bf16x8 pf[QN];
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int u = 0; u < QN; ++u) {
+        bool out[2][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          out[t][i] = edge && (unsigned)(kv0 + 16 * t + 4 * q + i - see_lo) > see_span;
-          if (out[t][i]) sacc[t][i] = -INFINITY;
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            out[t][i] = edge && (unsigned)(kv0 + 16 * t + 4 * q + i - see_lo[u]) > see_span[u];
+            if (out[t][i]) sacc[u][t][i] = -INFINITY;
+          }
+        float lm = sacc[u][0][0];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) lm = fmaxf(lm, sacc[u][t][i]);
+        if (__builtin_amdgcn_ballot_w64(lm > m_ref[u]) != 0) {
+          float mx = fmaxf(lm, __shfl_xor(lm, 16, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          const float m_new = fmaxf(m_ref[u], mx);
+          // A column that had seen no key has zero sums to rescale; one that still has none keeps -inf.
+          const float alpha = (m_ref[u] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_ref[u] - m_new) * scale_log2);
+          l_run[u] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[u][dt][i] *= alpha;
+          m_ref[u] = m_new;
         }
-      float lm = sacc[0][0];
+        const float mc = (m_ref[u] == -INFINITY) ? 0.f : m_ref[u] * scale_log2;
+        float p[8];
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lm = fmaxf(lm, sacc[t][i]);
-      if (__builtin_amdgcn_ballot_w64(lm > m_ref) != 0) {
-        float mx = fmaxf(lm, __shfl_xor(lm, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_ref, mx);
-        // A column that had seen no key has zero sums to rescale; one that still has none keeps -inf.
-        const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_ref - m_new) * scale_log2);
-        l_run *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
-        m_ref = m_new;
+          for (int i = 0; i < 4; ++i) {
+            float e = __builtin_amdgcn_exp2f(fmaf(sacc[u][t][i], scale_log2, -mc));
+            if (out[t][i]) e = 0.f;   // also where the scale is 0 and -inf * 0 is no number
+            p[4 * t + i] = e;
+            l_run[u] += e;
+          }
+        pf[u] = __builtin_bit_cast(bf16x8, pack8(p));
       }
-      const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * scale_log2;
-      float p[8];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float e = __builtin_amdgcn_exp2f(fmaf(sacc[t][i], scale_log2, -mc));
-          if (out[t][i]) e = 0.f;   // also where the scale is 0 and -inf * 0 is no number
-          p[4 * t + i] = e;
-          l_run += e;
-        }
-      const bf16x8 pf = __builtin_bit_cast(bf16x8, pack8(p));
-      // O^T += V^T P^T, four output tiles' fragments requested at a time.
+      // O^T += V^T P^T, four output tiles' fragments requested at a time, each for all the groups.
 #pragma unroll
       for (int k = 0; k < DT / 4; ++k) {
         TrFrag vf[4];
@@ -606,7 +641,9 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
         lds_tr_wait(vf[2], vf[3]);
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          oacc[4 * k + r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tr_join(vf[r]), pf, oacc[4 * k + r], 0, 0, 0);
+#pragma unroll
+          for (int u = 0; u < QN; ++u)
+            oacc[u][4 * k + r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tr_join(vf[r]), pf[u], oacc[u][4 * k + r], 0, 0, 0);
       }
     };
     using buf0 = std::integral_constant<int, 0>;
@@ -618,17 +655,20 @@ __global__ __launch_bounds__(512) void mha_prefill_wide_kernel(
     wait_vmcnt<0>();   // the idle fetch of the last iteration lands before the block's LDS is released
   }
 
-  // The lane's sum over its own keys -> the column's; normalize and store: lane holds query n,
-  // columns 16 dt + 4 q + 0..3.
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-  const float inv = (q_live && l_run > 0.f) ? 1.0f / l_run : 0.f;
-  if (my_q < seq) {
-    bf16_t* op = Oh + (size_t)my_q * q_row_stride + 4 * q;
+  // The lane's sum over its own keys -> the column's; normalize and store: lane holds query n of the
+  // group, columns 16 dt + 4 q + 0..3.
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      *reinterpret_cast<uint2*>(op + 16 * dt) = make_uint2(pack_bf16(oacc[dt][0] * inv, oacc[dt][1] * inv),
-                                                           pack_bf16(oacc[dt][2] * inv, oacc[dt][3] * inv));
+  for (int u = 0; u < QN; ++u) {
+    float l_tot = l_run[u] + __shfl_xor(l_run[u], 16, 64);
+    l_tot += __shfl_xor(l_tot, 32, 64);
+    const float inv = (q_live[u] && l_tot > 0.f) ? 1.0f / l_tot : 0.f;
+    if (my_q[u] < seq) {
+      bf16_t* op = Oh + (size_t)my_q[u] * q_row_stride + 4 * q;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<uint2*>(op + 16 * dt) = make_uint2(pack_bf16(oacc[u][dt][0] * inv, oacc[u][dt][1] * inv),
+                                                             pack_bf16(oacc[u][dt][2] * inv, oacc[u][dt][3] * inv));
+    }
   }
 }
 
@@ -657,6 +697,22 @@ static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
   hipLaunchKernelGGL((mha_prefill_kernel<D, SPLIT, W>), dim3(blocks), dim3(64 * W * SPLIT), lds, (hipStream_t)stream, a.Q,
                      a.K, a.V, a.O, a.heads, a.group, a.seq, a.seq_len, a.kv_len, a.scale_log2, a.causal, a.window,
                      a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid, a.kv_first, a.kv_rows);
+  return 0;
+}
+
+template <int D, int QN, int W>
+static int launch_prefill_wide(const PrefillArgs& a, void* stream) {
+  constexpr size_t lds = (size_t)2 * 2 * 32 * D * 2;   // two stages of a 32-key K tile and V tile
+  constexpr int block_queries = 16 * QN * W;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_prefill_wide_kernel<D, QN, W>), lds); e != hipSuccess) {
+    set_error("mha_prefill: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  hipLaunchKernelGGL((mha_prefill_wide_kernel<D, QN, W>), dim3(((a.seq + block_queries - 1) / block_queries) * a.heads),
+                     dim3(64 * W), lds, (hipStream_t)stream, a.Q, a.K, a.V, a.O, a.heads, a.group, a.seq, a.seq_len, a.kv_len,
+                     a.scale_log2, a.causal, a.window, a.q_row, a.q_head, a.kv_row, a.kv_head, a.valid, a.kv_valid,
+                     a.kv_first, a.kv_rows);
   return 0;
 }
 
@@ -691,18 +747,6 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
                "mha_prefill: the keys of a head span %ld bytes, more than the 2^31 its loads' 32-bit offsets reach",
                (long)kv_len * kv_row * 2);
   const float scale_log2 = scale * 1.4426950408889634f;
-  if (d == 512) {
-    constexpr size_t lds = 2 * 2 * 32 * 512 * 2;   // two stages of a 32-key K tile and V tile
-    static LdsOptIn opt_in;
-    if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_prefill_wide_kernel<512>), lds); e != hipSuccess) {
-      set_error("mha_prefill: %s", hipGetErrorString(e));
-      return (int)e;
-    }
-    hipLaunchKernelGGL(mha_prefill_wide_kernel<512>, dim3(((seq + 127) / 128) * heads), dim3(512), lds, (hipStream_t)stream, Q, K,
-                       V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window, q_row, q_head,
-                       kv_row, kv_head, valid, kv_valid, kv_first, kv_rows);
-    IRON_LAUNCH_CHECK();
-  }
   const int blocks = ((seq + BQ - 1) / BQ) * heads;
   // Few blocks (a short sequence): the longest block's chain of tiles bounds the launch, so its
   // tiles are split over two halves of eight waves.  Many blocks fill the chip better four waves each.
@@ -710,11 +754,20 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
   PrefillArgs a{Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window,
                 q_row, q_head, kv_row, kv_head, valid, kv_valid, kv_first, kv_rows};
   int rc;
+  // Wide heads: 16-query groups on 16x16x32 tiles.  Blocks of 128 queries (eight waves) once those
+  // fill the chip twice over, of 64 (four waves) below that; at 256, where two groups a wave fit the
+  // registers, launches of a thousand blocks and more take two (half the LDS reads a flop: 32 heads at
+  // S = 4096 382 against 424 us; at 2048 it is the other way round, 154 against 119).
+  if (d == 512) rc = blocks >= kWideBigBlocks ? launch_prefill_wide<512, 1, 8>(a, stream) : launch_prefill_wide<512, 1, 4>(a, stream);
+  else if (d == 256)
+    rc = blocks >= 2 * kWideBigBlocks ? launch_prefill_wide<256, 2, 4>(a, stream)
+         : blocks >= kWideBigBlocks   ? launch_prefill_wide<256, 1, 8>(a, stream)
+                                      : launch_prefill_wide<256, 1, 4>(a, stream);
   // Fewer blocks of 128 queries than CUs (a short prompt): blocks of 64, two waves a part.
-  if (d == 64 && blocks < kFewBlocks) rc = launch_prefill<64, 2, 2>(a, ((seq + 63) / 64) * heads, stream);
+  else if (d == 64 && blocks < kFewBlocks) rc = launch_prefill<64, 2, 2>(a, ((seq + 63) / 64) * heads, stream);
   else if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
-  else if (d == 128) rc = split ? launch_prefill<128, 2>(a, blocks, stream) : launch_prefill<128, 1>(a, blocks, stream);
-  else rc = launch_prefill<256, 1>(a, blocks, stream);
+  else if (split) rc = launch_prefill<128, 2>(a, blocks, stream);
+  else rc = launch_prefill<128, 1>(a, blocks, stream);
   if (rc != 0) return rc;
   IRON_LAUNCH_CHECK();
 }

@@ -740,6 +740,28 @@ def test_mha_prefill_d256_ragged_windowed_and_bounded(cuda):
     close(got[:rows], want[:rows])
 
 
+@pytest.mark.parametrize("d,H,G,S,window", [(512, 32, 8, 2048, None), (256, 32, 8, 2048, 300), (256, 32, 4, 4096, None),
+                                             (512, 16, 16, 1100, None)])
+def test_mha_prefill_wide_heads_at_every_block_shape_on_sampled_queries(cuda, d, H, G, S, window):
+    """256- and 512-wide heads where the launch has blocks enough for its larger shapes (128-query
+    blocks of eight waves; at 256 two query groups a wave from a thousand blocks on): the whole
+    output would take the oracle minutes, so every head of a sample of queries -- tile and block
+    edges, both ends, random rows -- is checked against the oracle's attention of that one query."""
+    rng = np.random.default_rng(d + S)
+    Q, Kc, Vc = bf(rng, S, H, d) * 0.25, bf(rng, S, G, d) * 0.25, bf(rng, S, G, d)
+    O = out_like(Q.shape, cuda, fill=float("nan"))
+    K.mha_prefill(dev(Q, cuda), dev(Kc, cuda), dev(Vc, cuda), O, heads=H, kv_heads=G, d=d, seq=S, seq_len=S,
+                  kv_len=S, scale=1.0, causal=True, window=window, q_interleaved=True, kv_interleaved=True)
+    got = from_torch(O)
+    assert not np.isnan(got).any()
+    for r in sorted({0, 1, 15, 16, 31, 32, 33, 63, 64, 127, 128, 129, 255, 256, S - 129, S - 128, S - 1,
+                     *rng.integers(0, S, 8).tolist()}):
+        lo = 0 if window is None else max(0, r - window)
+        want = ops.mha(Q[r : r + 1], Kc[lo : r + 1], Vc[lo : r + 1], num_heads=H, num_KV_heads=G, seq_len=1,
+                       kv_len=r + 1 - lo, d=d, causal=True, scale=1.0, heads_interleaved=True, kv_interleaved=True)
+        close(got[r : r + 1], want)
+
+
 @pytest.mark.parametrize("interleaved", [True, False])
 def test_mha_prefill_512_wide_heads_over_many_tiles(cuda, interleaved):
     """512-wide heads past a block's 64 queries and a tile's 32 keys: several heads a KV head, a ragged
