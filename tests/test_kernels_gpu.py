@@ -865,6 +865,31 @@ def test_mha_512_wide_heads_prefill_and_decode(cuda):
         close(O, want)
 
 
+@pytest.mark.parametrize("E,H,G,d", [(2048, 32, 8, 64), (1000, 3, 1, 128), (4096, 8, 2, 128)])
+def test_decode_qkv_reading_its_row_from_the_embedding_table(cuda, E, H, G, d):
+    """A token's first layer: the fused q/k/v launch handed the embedding table and the word that names
+    the row, against the same launch handed the row itself -- every output bit for bit, the row left
+    in ``x`` for the residual sum, and a word past either end of the table held inside it."""
+    rng = np.random.default_rng(E + d)
+    vocab, L, pos = 77, 16, 9
+    table, g = bf(rng, vocab, E), round_bf16(rng.uniform(0.9, 1.1, E).astype(np.float32))
+    Wq, Wk, Wv = bf(rng, H * d, E, scale=0.02), bf(rng, G * d, E, scale=0.02), bf(rng, G * d, E, scale=0.02)
+    angles = round_bf16(ops.rope_angles(d, L))
+    dt, dg, dq, dk, dv, da = (dev(a, cuda) for a in (table, g, Wq, Wk, Wv, angles))
+    position, angle_row = word(pos, cuda), word(pos, cuda)
+    for token in (0, 41, vocab - 1, vocab + 5, -3):
+        held = min(max(token, 0), vocab - 1)
+        want_q, want_k, want_v = out_like((H * d,), cuda), out_like((L, G, d), cuda, fill=2.0), out_like((L, G, d), cuda, fill=2.0)
+        K.decode_qkv(dev(table[held], cuda), dg, dq, dk, dv, da, want_q, want_k, want_v, eps=1e-5, hidden=E, heads=H,
+                     kv_heads=G, d=d, cache_rows=L, position=position, angle_row=angle_row)
+        x = out_like((E,), cuda, fill=float("nan"))
+        got_q, got_k, got_v = out_like((H * d,), cuda), out_like((L, G, d), cuda, fill=2.0), out_like((L, G, d), cuda, fill=2.0)
+        K.decode_qkv(x, dg, dq, dk, dv, da, got_q, got_k, got_v, eps=1e-5, hidden=E, heads=H, kv_heads=G, d=d,
+                     cache_rows=L, position=position, angle_row=angle_row, table=dt, token=word(token, cuda))
+        assert torch.equal(got_q, want_q) and torch.equal(got_k, want_k) and torch.equal(got_v, want_v), token
+        assert np.array_equal(from_torch(x), table[held]), token
+
+
 @pytest.mark.parametrize("H,G,d,rotary,ring,own_kv", [(4, 1, 128, 128, True, True), (4, 1, 256, 64, False, True),
                                                        (8, 2, 512, 512, True, True), (4, 1, 128, 128, False, False),
                                                        (16, 8, 64, 64, False, True)])
