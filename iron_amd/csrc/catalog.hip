@@ -102,18 +102,20 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const bf16_t* __restrict
   uint4* yr = reinterpret_cast<uint4*>(y + (size_t)row * cols);
   const uint4* wr = reinterpret_cast<const uint4*>(w);
 
+  // Every piece a thread keeps is asked for before any is used (as bounded loads: a thread past the
+  // row's end reads zeros and takes no branch, behind which the compiler would wait for each load
+  // where it stands).
   uint4 held[CHUNKS];
+  const __amdgpu_buffer_rsrc_t row_bytes = bounded_bytes(xr, 2 * cols);
+#pragma unroll
+  for (int i = 0; i < CHUNKS; ++i) held[i] = load_bounded(row_bytes, 16 * ((int)threadIdx.x + i * 256));
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < CHUNKS; ++i) {
-    const int c = threadIdx.x + i * 256;
-    if (c < nchunk) {
-      held[i] = xr[c];
-      float f[8];
-      unpack8(held[i], f);
+    float f[8];
+    unpack8(held[i], f);   // zeros past the end add nothing
 #pragma unroll
-      for (int j = 0; j < 8; ++j) s += f[j];
-    }
+    for (int j = 0; j < 8; ++j) s += f[j];
   }
   for (int c = threadIdx.x + CHUNKS * 256; c < nchunk; c += 256) {
     float f[8];
@@ -171,19 +173,36 @@ __global__ __launch_bounds__(256) void softmax_kernel(const void* __restrict__ x
   const int n = bound_or(length, cols);
   const size_t base = (size_t)row * cols;
   const int pieces = cols >> 3, live = (n + 7) >> 3;   // pieces of the row, and those with a column under n
-  // The capped logits of piece c; columns from n on are -inf (they weigh nothing).
-  auto logits = [&](int c, float (&z)[8]) {
+  // Piece c as it lies in memory (zeros past the row's end: the loads are bounded, no branch), and the
+  // capped logits made of it; columns from n on are -inf (they weigh nothing).
+  struct Raw {
+    uint4 a, b;      // the piece's 8 logits: 16 bytes of bf16 (a), or 32 of float32 (a, b)
+    uint4 pa, pb;    // the addend's 8 float32
+  };
+  const __amdgpu_buffer_rsrc_t x_row = bounded_bytes(reinterpret_cast<const char*>(x) + base * (F32 ? 4 : 2), cols * (F32 ? 4 : 2));
+  const __amdgpu_buffer_rsrc_t add_row = bounded_bytes(addend != nullptr ? addend + base : nullptr, addend != nullptr ? cols * 4 : 0);
+  auto fetch = [&](int c, Raw& r) {
     if (F32) {
-      const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(x) + base) + 2 * c;
-      const float4 a = p[0], b = p[1];
-      z[0] = a.x; z[1] = a.y; z[2] = a.z; z[3] = a.w; z[4] = b.x; z[5] = b.y; z[6] = b.z; z[7] = b.w;
+      r.a = load_bounded(x_row, 32 * c);
+      r.b = load_bounded(x_row, 32 * c + 16);
     } else {
-      unpack8(reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(x) + base)[c], z);
+      r.a = load_bounded(x_row, 16 * c);
     }
     if (addend != nullptr) {
-      const float4* p = reinterpret_cast<const float4*>(addend + base) + 2 * c;
-      const float4 a = p[0], b = p[1];
-      z[0] += a.x; z[1] += a.y; z[2] += a.z; z[3] += a.w; z[4] += b.x; z[5] += b.y; z[6] += b.z; z[7] += b.w;
+      r.pa = load_bounded(add_row, 32 * c);
+      r.pb = load_bounded(add_row, 32 * c + 16);
+    }
+  };
+  auto capped = [&](int c, const Raw& r, float (&z)[8]) {
+    if (F32) {
+      z[0] = __uint_as_float(r.a.x); z[1] = __uint_as_float(r.a.y); z[2] = __uint_as_float(r.a.z); z[3] = __uint_as_float(r.a.w);
+      z[4] = __uint_as_float(r.b.x); z[5] = __uint_as_float(r.b.y); z[6] = __uint_as_float(r.b.z); z[7] = __uint_as_float(r.b.w);
+    } else {
+      unpack8(r.a, z);
+    }
+    if (addend != nullptr) {
+      z[0] += __uint_as_float(r.pa.x); z[1] += __uint_as_float(r.pa.y); z[2] += __uint_as_float(r.pa.z); z[3] += __uint_as_float(r.pa.w);
+      z[4] += __uint_as_float(r.pb.x); z[5] += __uint_as_float(r.pb.y); z[6] += __uint_as_float(r.pb.z); z[7] += __uint_as_float(r.pb.w);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -191,13 +210,22 @@ __global__ __launch_bounds__(256) void softmax_kernel(const void* __restrict__ x
       if (8 * c + j >= n) z[j] = -INFINITY;
     }
   };
+  auto logits = [&](int c, float (&z)[8]) {
+    Raw r;
+    fetch(c, r);
+    capped(c, r, z);
+  };
+  // The pieces a thread keeps are all asked for before any is used.
   float held[CHUNKS][8];
   float m = -INFINITY;
+  {
+    Raw raw[CHUNKS];
 #pragma unroll
-  for (int i = 0; i < CHUNKS; ++i) {
-    const int c = threadIdx.x + i * 256;
-    if (c < live) {
-      logits(c, held[i]);
+    for (int i = 0; i < CHUNKS; ++i) fetch(threadIdx.x + i * 256, raw[i]);
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int c = threadIdx.x + i * 256;
+      capped(c, raw[i], held[i]);   // -inf from column n on, so also for a thread past the live pieces
 #pragma unroll
       for (int j = 0; j < 8; ++j) m = fmaxf(m, held[i][j]);
     }
