@@ -207,7 +207,8 @@ def bench_decode_kernels(torch, K, dev, n, rng):
 
 def bench_attention(torch, K, dev, n, rng):
     """GQA causal attention, 32 q / 8 kv heads, d 64, scale 1/8: prefill at S = 512, 2048, 8192 (MFMA bound)
-    and one query over caches of 1024, 4096, 16384 keys (HBM bound)."""
+    and one query over caches of 1024, 4096, 16384 keys (HBM bound); beside them prefill at S = 2048 with
+    256- and 512-wide heads."""
     H, G, D = 32, 8, 64
     out = {"prefill": [], "decode": []}
 
@@ -233,6 +234,25 @@ def bench_attention(torch, K, dev, n, rng):
         out["prefill"].append({"S": S, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
                                "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
                                "checked_outputs": checked})
+    # Wider heads (not a BASELINE configuration; Gemma's 256- and 512-wide ones), unscaled, S = 2048.
+    out["prefill_wide_heads"] = []
+    for Dw in (256, 512):
+        S = 2048
+        Q, Kc, Vc = rand(S, H, Dw) * 0.25, rand(S, G, Dw) * 0.25, rand(S, G, Dw)
+        O = torch.empty_like(Q)
+        launches = [lambda: K.mha_prefill(Q, Kc, Vc, O, heads=H, kv_heads=G, d=Dw, seq=S, kv_len=S, scale=1.0,
+                                          q_interleaved=True, kv_interleaved=True)] * 4
+        us = graph_time_us(torch, launches, max(1, n // 40))
+        checked = 0
+        for i in sorted({0, 15, 16, 127, 128, S // 2 - 1, S - 1}):
+            qf = Q[i].float().reshape(G, H // G, Dw)
+            scores = torch.einsum("ghd,lgd->ghl", qf, Kc[: i + 1].float())
+            want = torch.einsum("ghl,lgd->ghd", torch.softmax(scores, dim=-1), Vc[: i + 1].float()).reshape(H, Dw)
+            checked += verified(torch, f"prefill attention d={Dw} row {i}", O[i], want)
+        flops = 4.0 * H * Dw * S * (S + 1) / 2
+        out["prefill_wide_heads"].append({"d": Dw, "S": S, "us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 1),
+                                          "frac_mfma": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                          "checked_outputs": checked})
     for L in (1024, 4096, 16384):
         copies = max(2, min(64, int(np.ceil(400e6 / (L * G * D * 4)))))
         Q = rand(1, H, D)
