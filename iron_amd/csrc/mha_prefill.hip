@@ -41,7 +41,10 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 //
 // At least two waves a SIMD caps the register budget at 256, which makes the compiler keep MFMA
 // accumulators in ordinary VGPRs: the softmax reads S and rescales O in place instead of copying
-// every value out of (and back into) accumulation registers.
+// every value out of (and back into) accumulation registers.  The eight-wave form at d = 64 is held
+// to 128 registers and two stages (64 KB), so that a CU holds two blocks at different places of their
+// loops (S = 4096: 118 -> 95 us); three four-wave blocks a CU measured slower than two (S = 8192:
+// 382 against 365 us).
 //
 // SPLIT = 2: eight waves; waves 4..7 serve the same four groups of 32 queries as waves 0..3 but take
 // the odd key tiles (their own loads, their own stage buffers), and the two halves' (max, sum, O)
@@ -51,7 +54,7 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 // W: the waves that share a tile's loads, each with 32 of the block's 32 W queries.  Four; two
 // where four would leave CUs without a block (a short prompt), so that twice as many blocks go out.
 template <int D, int SPLIT, int W = 4>
-__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(W == 4 ? 2 : 1))) void mha_prefill_kernel(
+__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(W == 4 ? (D == 64 && SPLIT == 2 ? 4 : 2) : 1))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   constexpr int KS = D / 16;             // k16 steps of S^T
   constexpr int DT = D / 32;             // 32-row tiles of O^T
   constexpr int CPR = D / 8;             // 16-byte chunks a row has
-  constexpr int STAGES = D == 64 ? 3 : 2;
+  constexpr int STAGES = D == 64 && !(SPLIT == 2 && W == 4) ? 3 : 2;
   constexpr int TILE = BKV * ROWB;       // bytes of a K (or V) tile
   constexpr int STAGE = 2 * TILE;
   constexpr int BQW = 32 * W;            // query rows of this block
@@ -687,7 +690,7 @@ struct PrefillArgs {
 // The stage buffers are dynamic LDS (more than the 64 KB a kernel may declare statically).
 template <int D, int SPLIT, int W = 4>
 static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
-  constexpr int STAGES = D == 64 ? 3 : 2;
+  constexpr int STAGES = D == 64 && !(SPLIT == 2 && W == 4) ? 3 : 2;
   constexpr size_t lds = (size_t)SPLIT * STAGES * 2 * BKV * D * 2;
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT, W>), lds); e != hipSuccess) {
