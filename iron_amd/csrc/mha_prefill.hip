@@ -29,7 +29,8 @@ __device__ __forceinline__ float max_with_other_half(float x) {
 
 constexpr int BQ = 128;   // query rows per block (four waves of 32; 64 where a block is two)
 constexpr int BKV = 64;   // key rows per tile
-constexpr int kFewBlocks = 256;          // launches of fewer blocks than this halve their blocks' queries
+constexpr int kCUs = 256;                // compute units the block orders below assume
+constexpr int kFewBlocks = 512;          // launches of fewer blocks than this halve their blocks' queries (S = 1024 at 32 heads: 18.5 -> 13.9 us)
 constexpr int kWideBigBlocks = 512;     // wide heads: launches of at least this many 128-query blocks keep that size
 constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks split each block's tiles over two halves
 
@@ -43,7 +44,7 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 // accumulators in ordinary VGPRs: the softmax reads S and rescales O in place instead of copying
 // every value out of (and back into) accumulation registers.  The eight-wave form at d = 64 is held
 // to 128 registers and two stages (64 KB), so that a CU holds two blocks at different places of their
-// loops (S = 4096: 118 -> 95 us); three four-wave blocks a CU measured slower than two (S = 8192:
+// loops (S = 4096: 118 -> 95 us; the 64-query blocks of short prompts likewise); three four-wave blocks a CU measured slower than two (S = 8192:
 // 382 against 365 us).
 //
 // SPLIT = 2: eight waves; waves 4..7 serve the same four groups of 32 queries as waves 0..3 but take
@@ -54,7 +55,7 @@ constexpr int kSplitMaxBlocks = 1024;   // launches of up to this many blocks sp
 // W: the waves that share a tile's loads, each with 32 of the block's 32 W queries.  Four; two
 // where four would leave CUs without a block (a short prompt), so that twice as many blocks go out.
 template <int D, int SPLIT, int W = 4>
-__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(W == 4 ? (D == 64 && SPLIT == 2 ? 4 : 2) : 1))) void mha_prefill_kernel(
+__global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(W == 4 ? (D == 64 && SPLIT == 2 ? 4 : 2) : (D == 64 && SPLIT == 2 ? 2 : 1)))) void mha_prefill_kernel(
     const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K, const bf16_t* __restrict__ V,
     bf16_t* __restrict__ O, int heads, int group, int seq, int seq_len, int kv_len, float scale_log2,
     int causal, int window, long q_row_stride, long q_head_stride, long kv_row_stride,
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   constexpr int KS = D / 16;             // k16 steps of S^T
   constexpr int DT = D / 32;             // 32-row tiles of O^T
   constexpr int CPR = D / 8;             // 16-byte chunks a row has
-  constexpr int STAGES = D == 64 && !(SPLIT == 2 && W == 4) ? 3 : 2;
+  constexpr int STAGES = D == 64 && SPLIT == 1 ? 3 : 2;
   constexpr int TILE = BKV * ROWB;       // bytes of a K (or V) tile
   constexpr int STAGE = 2 * TILE;
   constexpr int BQW = 32 * W;            // query rows of this block
@@ -87,7 +88,12 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   const int j = blockIdx.x % heads;
   const int head = (heads % 8 == 0) ? (j % 8) * (heads / 8) + j / 8 : j;
   const int kvh = head / group;
-  const int qb = (int)(gridDim.x / heads) - 1 - (int)(blockIdx.x / heads);
+  // A launch whose blocks are all resident two a CU (more blocks than CUs, no more than twice as
+  // many): the second half of the ids runs from the lightest query block up, so the two blocks a CU
+  // holds -- ids i and i + 256 -- are a heavy one and a light one, and every CU has the same work.
+  const int nqb = (int)(gridDim.x / heads), at = (int)(blockIdx.x / heads);
+  const bool folded = causal && gridDim.x > kCUs && gridDim.x <= 2 * kCUs && SPLIT == 2 && W == 4 && D == 64;
+  const int qb = folded && at >= (nqb + 1) / 2 ? at - (nqb + 1) / 2 : nqb - 1 - at;
   const int q0 = qb * BQW;
 
   const int q_tokens = valid ? bound_or(valid, seq) : seq_len;
@@ -690,7 +696,7 @@ struct PrefillArgs {
 // The stage buffers are dynamic LDS (more than the 64 KB a kernel may declare statically).
 template <int D, int SPLIT, int W = 4>
 static int launch_prefill(const PrefillArgs& a, int blocks, void* stream) {
-  constexpr int STAGES = D == 64 && !(SPLIT == 2 && W == 4) ? 3 : 2;
+  constexpr int STAGES = D == 64 && SPLIT == 1 ? 3 : 2;
   constexpr size_t lds = (size_t)SPLIT * STAGES * 2 * BKV * D * 2;
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&mha_prefill_kernel<D, SPLIT, W>), lds); e != hipSuccess) {
@@ -766,7 +772,7 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
     rc = blocks >= 2 * kWideBigBlocks ? launch_prefill_wide<256, 2, 4>(a, stream)
          : blocks >= kWideBigBlocks   ? launch_prefill_wide<256, 1, 8>(a, stream)
                                       : launch_prefill_wide<256, 1, 4>(a, stream);
-  // Fewer blocks of 128 queries than CUs (a short prompt): blocks of 64, two waves a part.
+  // Fewer blocks of 128 queries than two a CU (a short prompt): blocks of 64, two waves a part.
   else if (d == 64 && blocks < kFewBlocks) rc = launch_prefill<64, 2, 2>(a, ((seq + 63) / 64) * heads, stream);
   else if (d == 64) rc = split ? launch_prefill<64, 2>(a, blocks, stream) : launch_prefill<64, 1>(a, blocks, stream);
   else if (split) rc = launch_prefill<128, 2>(a, blocks, stream);
