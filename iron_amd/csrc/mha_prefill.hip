@@ -758,8 +758,9 @@ static int mha_prefill(const uint16_t* Q, const uint16_t* K, const uint16_t* V, 
   const float scale_log2 = scale * 1.4426950408889634f;
   const int blocks = ((seq + BQ - 1) / BQ) * heads;
   // Few blocks (a short sequence): the longest block's chain of tiles bounds the launch, so its
-  // tiles are split over two halves of eight waves.  Many blocks fill the chip better four waves each.
-  const bool split = blocks <= kSplitMaxBlocks;
+  // tiles are split over two halves of eight waves.  Many blocks fill the chip better four waves each
+  // (at d = 64, where two eight-wave blocks share a CU, only from S = 16384 at 32 heads on: S = 8192 365 -> 353-360 us).
+  const bool split = blocks <= (d == 64 ? 4 * kSplitMaxBlocks : kSplitMaxBlocks);
   PrefillArgs a{Q, K, V, O, heads, heads / kv_heads, seq, seq_len, kv_len, scale_log2, causal, window,
                 q_row, q_head, kv_row, kv_head, valid, kv_valid, kv_first, kv_rows};
   int rc;
