@@ -441,9 +441,9 @@ __global__ __launch_bounds__(64 * W, 2) void mha_prefill_wide_kernel(
   const int j = blockIdx.x % heads;
   const int head = (heads % 8 == 0) ? (j % 8) * (heads / 8) + j / 8 : j;
   const int kvh = head / group;
-  // (Two blocks a CU where the stages are 64 KB: a heavy and a light query block, as above.)
+  // (Two four-wave blocks a CU where the stages are 64 KB: a heavy and a light query block, as above.)
   const int nqb = (int)(gridDim.x / heads), at = (int)(blockIdx.x / heads);
-  const bool folded = causal && D == 256 && gridDim.x > kCUs && gridDim.x <= 2 * kCUs;
+  const bool folded = causal && D == 256 && W == 4 && gridDim.x > kCUs && gridDim.x <= 2 * kCUs;
   const int qb = folded && at >= (nqb + 1) / 2 ? at - (nqb + 1) / 2 : nqb - 1 - at;
   const int q0 = qb * BQW;
 
