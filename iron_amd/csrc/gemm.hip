@@ -279,6 +279,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A,
 // __syncthreads() carries would wait for every outstanding load (vmcnt(0)) and drain the
 // prefetch; each wave instead waits until only the younger stages are in flight.
 constexpr int NT_STAGES = 4;
+constexpr int PAIR_STAGES = 3;   // of the two-product body: 48 KB each
 
 // B_KN (128 x 128 and 256 x 256 tiles): B is (K,N) row-major.  Its tile lands in LDS as stored, a
 // row a k (a wave instruction moves 4 k-rows x 256 B, or 2 x 512 B; chunks swizzled by the row so
@@ -1474,6 +1475,183 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   IRON_LAUNCH_CHECK();
 }
 
+// A gated feed-forward's two first projections on one 128 x 128 tile position AT ONCE: a stage is the
+// A tile and both weights' tiles (48 KB, three stages), an A fragment read out of LDS serves both
+// products, and the gated epilogue has both accumulators in registers in the same layout, so the
+// gate's product is stored (rounded, as the separate product stores it) and never read back.
+// Against the same body run twice this fetches A once instead of twice (a quarter of the bytes a
+// CU draws from L2 and a quarter of its LDS fragment reads).  Each product's MFMAs run in the order
+// of the single-product body, so G and C are the separate launches' bit for bit.
+__device__ __forceinline__ void gemm_nt16_pair_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Bg,
+                                                    const bf16_t* __restrict__ Bu, bf16_t* __restrict__ G,
+                                                    bf16_t* __restrict__ C, int M, int N, int K,
+                                                    const int* __restrict__ valid, int tiles_m, int tiles_n,
+                                                    int patched, int activation) {
+  constexpr int NT_BM = 128, NT_BN = 128;
+  constexpr int PART = NT_BM * BK * 2;             // a 128 x 64 tile's 16 KB: A, then the gate's, then the up projection's
+  constexpr int STAGE = 3 * PART, STAGES = PAIR_STAGES;
+  constexpr int INST = NT_BM / 8 / 4;              // 1 KB loads of each part a wave issues per stage
+  constexpr int LOADS = 3 * INST;
+  static_assert(BK == 64 && INST == 4, "two 32-wide k-steps a stage, twelve loads a wave");
+  extern __shared__ __align__(16) char smem_nt[];
+  const int Mv = bound_or(valid, M);
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
+  const int m0 = tm * NT_BM;
+  if (m0 >= Mv) return;
+  const int n0 = tn * NT_BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = lane >> 3, pch = lane & 7;
+  int a_voff[INST], b_voff[INST];
+#pragma unroll
+  for (int i = 0; i < INST; ++i) {
+    const int r = (wave * INST + i) * 8 + lrow;
+    const int lch = pch ^ ((r >> 1) & 7);
+    // Rows past the end re-read the last row; what they produce is never stored.
+    a_voff[i] = (int)(((size_t)(min(m0 + r, M - 1) - m0) * K + lch * 8) * 2);
+    b_voff[i] = (int)(((size_t)(min(n0 + r, N - 1) - n0) * K + lch * 8) * 2);
+  }
+  const bf16_t* a_tile = A + (size_t)m0 * K;
+  const bf16_t* g_tile = Bg + (size_t)n0 * K;
+  const bf16_t* u_tile = Bu + (size_t)n0 * K;
+  auto issue_one = [&](char* st, int kt, int idx) {   // idx: 0..3 A, 4..7 the gate's weights, 8..11 the up projection's
+    const int k0 = kt * BK, part = idx / INST, piece = idx % INST;
+    const bf16_t* from = part == 0 ? a_tile : (part == 1 ? g_tile : u_tile);
+    const __amdgpu_buffer_rsrc_t rows = stage_rows(from + k0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rows, IRON_LDS_PTR(st + part * PART + (wave * INST + piece) * 1024), 16,
+                                             (int)(part == 0 ? a_voff[piece] : b_voff[piece]), 0, 0, 0);
+  };
+
+  f32x4 accg[4][4], accu[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) accg[i][j][e] = accu[i][j][e] = 0.f;
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+#pragma unroll
+    for (int idx = 0; idx < LOADS; ++idx) issue_one(smem_nt + s * STAGE, min(s, nk - 1), idx);
+
+  // Fragments: lane -> row fr of a 16-row tile, 16-byte chunk kq of the k-step's four.
+  const int fr = lane & 15, kq = lane >> 4;
+  const int swz = (fr >> 1) & 7;   // tile rows are multiples of 16 apart: one swizzle for all
+  const int a_row = (wm * 64 + fr) * 128, b_row = (wn * 64 + fr) * 128;
+  auto a_frag = [&](const char* st, int ks, int i) {
+    return *reinterpret_cast<const bf16x8*>(st + a_row + i * 16 * 128 + (((ks * 4 + kq) ^ swz) << 4));
+  };
+  auto b_frag = [&](const char* st, int part, int ks, int j) {
+    return *reinterpret_cast<const bf16x8*>(st + part * PART + b_row + j * 16 * 128 + (((ks * 4 + kq) ^ swz) << 4));
+  };
+
+  wait_vmcnt<(STAGES - 2) * LOADS>();   // stage 0 has landed once only the younger one is out
+  block_barrier();
+  bf16x8 af[2][4], bg[2][4], bu[2][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) bg[0][i] = b_frag(smem_nt, 1, 0, i);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) bu[0][i] = b_frag(smem_nt, 2, 0, i);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) af[0][i] = a_frag(smem_nt, 0, i);
+  for (int kt = 0; kt < nk; ++kt) {
+    // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
+    // (into buffers nobody reads any more) rather than branch: every iteration issues the same
+    // loads, which keeps the wait counts exact and the scheduling region whole.
+    const int kn = min(kt + STAGES - 1, nk - 1);
+    char* nst = smem_nt + ((kt + STAGES - 1) % STAGES) * STAGE;
+    const char* st = smem_nt + (kt % STAGES) * STAGE;
+    const char* st1 = smem_nt + ((kt + 1) % STAGES) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      if (ks == 1) {
+        // The stage's one barrier, before its second k-step (whose fragments are in registers): of
+        // the loads in flight the oldest LOADS are stage kt+1's, then the half of stage kt+2's
+        // issued so far; after it nobody reads stage kt any more.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait_vmcnt<LOADS / 2>();
+        block_barrier();
+      }
+      const char* from = ks == 0 ? st : st1;
+      const int nks = ks ^ 1;
+      // Source order is issue order (nothing crosses a sched_barrier): after an MFMA one fragment
+      // read of the next k-step (the weights' first: its first MFMAs need all of them) or one load.
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (j < 4) mfma_16x16x32_in_place(accg[i][j], bg[ks][j], af[ks][i]);
+          else mfma_16x16x32_in_place(accu[i][j - 4], bu[ks][j - 4], af[ks][i]);
+          __builtin_amdgcn_sched_barrier(0);
+          const int slot = i * 8 + j;
+          if (slot < 4) bg[nks][slot] = b_frag(from, 1, nks, slot);
+          else if (slot < 8) bu[nks][slot - 4] = b_frag(from, 2, nks, slot - 4);
+          else if (slot < 12) af[nks][slot - 8] = a_frag(from, nks, slot - 8);
+          else if ((slot & 1) && slot < 12 + LOADS) issue_one(nst, kn, ks * (LOADS / 2) + (slot - 13) / 2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+  }
+
+  wait_vmcnt<0>();   // the idle fetches of the last iterations land ...
+  block_barrier();   // ... in every wave, and every wave is done with the stages, before LDS is reused
+
+  // Output through LDS, a product at a time: the wave lays its 64 x 64 out row-major (rows padded by
+  // 16 bytes) and each lane then owns 8 consecutive columns of a row, so a row of the tile leaves as
+  // one 128-byte segment.  First the gate's product as it is stored; then, made in the accumulators'
+  // own layout, bf16(bf16(act(bf16 g)) * bf16 u).
+  constexpr int OROWB = 64 * 2 + 16;
+  char* ot = smem_nt + wave * (64 * OROWB);
+  const int out_row = lane >> 3, out_col = (lane & 7) * 8;
+  const int out_n = n0 + wn * 64 + out_col;
+  const bool whole = (N & 7) == 0 && out_n + 8 <= N;
+  auto leave = [&](bf16_t* to) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int row = r * 8 + out_row, m = m0 + wm * 64 + row;
+      const uint4 v = *reinterpret_cast<const uint4*>(ot + row * OROWB + out_col * 2);
+      if (m >= Mv || out_n >= N) continue;
+      bf16_t* p = to + (size_t)m * N + out_n;
+      if (whole) {
+        *reinterpret_cast<uint4*>(p) = v;
+      } else {
+        const bf16_t* h = reinterpret_cast<const bf16_t*>(&v);
+        for (int e = 0; e < 8 && out_n + e < N; ++e) p[e] = h[e];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();   // the rows are read before the next product overwrites them
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<uint2*>(ot + (i * 16 + fr) * OROWB + (j * 16 + 4 * kq) * 2) =
+          make_uint2(pack_bf16(accg[i][j][0], accg[i][j][1]), pack_bf16(accg[i][j][2], accg[i][j][3]));
+  leave(G);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float c[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        c[e] = round_bf16(gate_of(activation, round_bf16(accg[i][j][e]))) * round_bf16(accu[i][j][e]);
+      *reinterpret_cast<uint2*>(ot + (i * 16 + fr) * OROWB + (j * 16 + 4 * kq) * 2) =
+          make_uint2(pack_bf16(c[0], c[1]), pack_bf16(c[2], c[3]));
+    }
+  leave(C);
+}
+
 // A gated feed-forward's two first projections over many rows as ONE launch: a block computes its
 // tile of the gate's product and stores it (rounded, as the separate product stores it), then
 // computes the same tile of the second product, whose epilogue reads the gate tile back -- the one
@@ -1492,9 +1670,7 @@ __global__ __launch_bounds__(256) void gemm_gated_pair_kernel(const bf16_t* __re
   gate.gated = activation;
   if (Mv > few128) {
     if (bid >= t128.tiles_m * t128.tiles_n) return;
-    gemm_nt16_body<false>(A, Bg, G, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, none);
-    __syncthreads();   // the gate tile's stores are acknowledged, and every wave is done with the stage buffers
-    gemm_nt16_body<false>(A, Bu, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, gate);
+    gemm_nt16_pair_body(A, Bg, Bu, G, C, M, N, K, valid, t128.tiles_m, t128.tiles_n, t128.patched, activation);
   } else {
     if (bid >= t64.tiles_m * t64.tiles_n) return;
     gemm_nt64_body<8>(A, Bg, G, M, N, K, valid, t64.tiles_m, t64.tiles_n, t64.patched, none);
@@ -1515,7 +1691,8 @@ static int launch_gemm_gated_pair(const bf16_t* A, const bf16_t* Bg, const bf16_
     return Tiling{tile_rows, tile_cols, patched_order(tile_rows, tile_cols)};
   };
   const Tiling t128 = tiling((M + 127) / 128, n128), t64 = tiling((few128 + 63) / 64, n64);
-  constexpr size_t lds = (size_t)NT_STAGES * 256 * BK * 2;
+  constexpr size_t lds = (size_t)PAIR_STAGES * 3 * 128 * BK * 2;   // the two-product body's stages, more than the others'
+  static_assert(lds >= (size_t)NT_STAGES * 256 * BK * 2, "the 64 x 64 body's stages fit too");
   static LdsOptIn opt_in;
   if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_gated_pair_kernel), lds); e != hipSuccess) {
     set_error("gemm_gated_pair: %s", hipGetErrorString(e));
