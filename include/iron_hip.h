@@ -56,6 +56,25 @@ int iron_gemv_bf16_tuned(const uint16_t* W, const uint16_t* x, uint16_t* y, int 
 int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R, uint16_t* C, int M,
                             int N, int K, float residual_scale, const int* valid, void* stream);
 
+/* The same product and sum for few rows over a long K, and the RMSNorm of the rows it leaves:
+ * C = bf16(residual_scale * bf16(A B^T) + R), Y = RMSNorm(C) * gain as iron_rmsnorm_bf16 computes it
+ * (Y is bit for bit what that call makes of C), for the rows under *valid (or M), in two launches.
+ * While the bound leaves 128 x 128 tiles for no more than half the chip (512 live rows of a 2048-row
+ * prompt chunk at N = 2048), each tile's K is dealt over 4 or 2 blocks that leave float32 sums in
+ * `workspace`, and the second launch adds a row's slices in slice order before it rounds: the sums
+ * are the same whatever ran first, and differ from iron_gemm_residual_bf16's in the last bits of the
+ * float32 sum only.  A (M,K), B (N,K), R and C (M,N), gain (N), Y (M,N); C may be R, Y neither.
+ * iron_gemm_residual_norm_workspace_bytes(M, N, K): the workspace's size (any contents), 0 for a
+ * shape this entry refuses (M < 128, N not a multiple of 128 up to 8192, K under 4096 or not a
+ * multiple of 256).
+ * Replaces GEMM (down_proj), ElementwiseAdd / AXPY and the next RMSNorm
+ * (iron/lm/blocks.py:723-733, then :688 of the next layer or the final norm). */
+int64_t iron_gemm_residual_norm_workspace_bytes(int M, int N, int K);
+int iron_gemm_residual_norm_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R,
+                                 const uint16_t* gain, uint16_t* C, uint16_t* Y, int M, int N, int K,
+                                 float residual_scale, float eps, const int* valid, void* workspace,
+                                 void* stream);
+
 /* C = bf16(bf16(act(G)) * bf16(A B^T)) for the rows under *valid (or M): a gated feed-forward's second
  * projection with the activated gate in its epilogue; activation 1: SiLU, 2: GELU by its tanh form.
  * A (M,K), B (N,K), G and C (M,N); K % 64 == 0, M, N >= 64.  C may be G.

@@ -22,6 +22,8 @@ SIGNATURES = {
     "iron_gemv_bf16": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "iron_gemv_bf16_tuned": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, c_int, c_int, _P]),
     "iron_gemm_residual_bf16": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, _P]),
+    "iron_gemm_residual_norm_workspace_bytes": (c_int64, [c_int, c_int, c_int]),
+    "iron_gemm_residual_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, c_float, _P, _P, _P]),
     "iron_gemm_gated_bf16": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "iron_gemv_fused_bf16": (c_int, [_P, _P, _P, _P, c_float, _P, c_float, _P, c_int, c_int, c_int, _P]),
     "iron_decode_qkv_bf16": (

@@ -22,6 +22,7 @@ in a prompt chunk's version (several rows, 64-wide heads),
   GEMM (up), SiLU or GELU (tanh) of the gate, Mul        => iron_gemm_gated_bf16
   SiLU, ElementwiseMul (no such product before them)     => iron_silu_mul_bf16
   GEMM, ElementwiseAdd / AXPY (the residual)             => iron_gemm_residual_bf16
+  ... few rows over a long K, and the RMSNorm after them => iron_gemm_residual_norm_bf16
 
 and in either,
 
@@ -47,6 +48,7 @@ class Fused:
     count: int
     launch: Callable[[], None]
     launches: int = 1      # 0: a step other launches made needless (nothing runs for it)
+    scratch_bytes: int = 0  # device memory of its own the launch needs, live over the run
 
 
 class _Anything:
@@ -62,7 +64,7 @@ class _Anything:
 def match(recording) -> list[Fused]:
     """The runs ``plan`` would fuse, without binding any tensor: for the arena plan, which must
     keep every buffer a run touches alive across the whole run."""
-    return plan(recording, lambda h: _Anything(), lambda e: None)
+    return plan(recording, lambda h: _Anything(), lambda e: None, lambda first, nbytes: _Anything())
 
 
 def _plain(h) -> bool:
@@ -84,11 +86,14 @@ def _same_view(a, b) -> bool:
             and a.index is None and a.ids is None and b.index is None and b.ids is None)
 
 
-def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) -> list[Fused]:
+def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any],
+         scratch: Callable[[int, int], Any] | None = None) -> list[Fused]:
     """The fused launches of ``recording``'s steps, by the first step each covers.
 
     ``tensor(handle)`` is the device tensor behind a handle, ``word(expr)`` the device word
-    of a per-call expression.
+    of a per-call expression, ``scratch(first, nbytes)`` the device memory placed for the run
+    that starts at step ``first`` (``Fused.scratch_bytes`` of it); without ``scratch`` no run
+    that needs memory of its own is planned.
     """
     from .. import kernels
 
@@ -417,6 +422,22 @@ def plan(recording, tensor: Callable[[Any], Any], word: Callable[[Any], Any]) ->
                 args = dict(A=tensor(s.inputs["A"]), B=tensor(s.inputs["B"]), R=tensor(other), C=tensor(ad.outputs["y"]))
                 kw = dict(M=s.op.M, N=s.op.N, K=s.op.K, residual_scale=scale, valid=word(gv))
                 got = Fused("gemm_add", i, 2, lambda a=args, kw=kw: kernels.gemm_residual(**a, **kw))
+                # ... and the norm of the rows it leaves (the next layer's input norm after a down
+                # projection): few rows over a long K are dealt over several blocks a tile, and the
+                # launch that adds their sums up stands where the norm's stood
+                nm = steps[i + 2] if i + 2 < len(steps) else None
+                need = kernels.gemm_residual_norm_workspace_bytes(s.op.M, s.op.N, s.op.K) if scratch and nm else 0
+                if (need and _name(nm) == "RMSNorm" and nm.op.weighted and nm.op.rows == s.op.M
+                        and nm.op.tile_size == s.op.N and set(nm.values) <= {"valid"} and nm.values.get("valid") == gv
+                        and _same_view(nm.inputs["x"], ad.outputs["y"])
+                        and all(h.index is None and h.ids is None for h in (*nm.inputs.values(), nm.outputs["y"]))
+                        and nm.outputs["y"].buffer is not ad.outputs["y"].buffer
+                        and nm.outputs["y"].buffer is not other.buffer):
+                    args = dict(args, gain=tensor(nm.inputs["weight"]), Y=tensor(nm.outputs["y"]),
+                                workspace=scratch(i, need))
+                    kw = dict(kw, eps=float(nm.op.epsilon))
+                    got = Fused("gemm_add_norm", i, 3, lambda a=args, kw=kw: kernels.gemm_residual_norm(**a, **kw),
+                                launches=2, scratch_bytes=need)
         elif _name(s) == "GEMM" and (gated := gated_at(i + 1, s)) is not None:
             # a gated feed-forward's two first projections over many rows: one launch computes both
             # products tile by tile, the activated gate riding the second one's epilogue

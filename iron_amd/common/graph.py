@@ -1133,9 +1133,16 @@ class CompiledGraph:
         if self.fuse:
             from . import fusion
 
-            runs = [(f.first, f.first + f.count - 1) for f in fusion.match(recording)]
+            matched = fusion.match(recording)
+            runs = [(f.first, f.first + f.count - 1) for f in matched]
         for b, first, last in recording.transients(runs):
             self.transient_offsets[id(b)] = pool.place(LiveRange(b.nbytes, first, last))
+        # Memory a fused run needs for itself (partial sums), live over its steps, by the run's first step.
+        self.scratch_offsets: dict[int, int] = {}
+        if self.fuse:
+            for f in matched:
+                if f.scratch_bytes:
+                    self.scratch_offsets[f.first] = pool.place(LiveRange(f.scratch_bytes, f.first, f.first + f.count - 1))
         # The per-call words: one slot per declared value, then one per derived expression.
         self.slots: dict[str, int] = {v.name: i for i, v in enumerate(recording.values)}
         self.exprs: dict[Affine, int] = {}
@@ -1173,6 +1180,10 @@ class CompiledGraph:
         return self.exprs[expr]
 
     # -- loading -------------------------------------------------------------
+    def _scratch(self, first: int, nbytes: int):
+        """The float32 words placed for the fused run that starts at step ``first``."""
+        return self.arena.view(self.arena.resident_bytes + self.scratch_offsets[first], (nbytes // 4,), np.float32)
+
     def _tensor(self, h: Handle):
         b = h.buffer
         if b.kind == "resident":
@@ -1249,7 +1260,7 @@ class CompiledGraph:
         if self.fuse:
             from . import fusion
 
-            self._fused = {f.first: f for f in fusion.plan(self.recording, self._tensor, self.word)}
+            self._fused = {f.first: f for f in fusion.plan(self.recording, self._tensor, self.word, self._scratch)}
         self.input_tensors = [self._tensor(h) for h in self.recording.inputs]
         self.output_tensors = [self._tensor(h) for h in self.recording.outputs]
         self._loaded_generation = self.arena.generation

@@ -311,6 +311,12 @@ struct QkvTail {
   // projections write one), and the chunk's rows go to rows *kv_row0 on, when kv_row0 is not NULL.
   const int* kv_row0;
   int kv_rows;
+  // Of a plain product on the 128 x 128 tiles, one block of several that share a tile's K: columns
+  // k_begin .. k_begin + k_len of A and B (k_len 0: all of them), the float32 sums left at `partial`
+  // (an (M, N) array of this slice's) instead of C; tile_plus1: the tile's number + 1 where the
+  // kernel deals tiles itself instead of by the block's id.
+  int k_begin, k_len, tile_plus1;
+  float* partial;
 };
 
 __device__ __forceinline__ float gate_of(int kind, float g) { return kind == 2 ? gelu_tanh_f32(g) : silu_f32(g); }
@@ -543,6 +549,12 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
 
   int tm, tn;
   tile_of_block(blockIdx.x, tiles_m, tiles_n, patched, tm, tn);
+  if constexpr (!QKV) {
+    if (qkv.tile_plus1 > 0) {
+      tm = (qkv.tile_plus1 - 1) / tiles_n;
+      tn = (qkv.tile_plus1 - 1) % tiles_n;
+    }
+  }
   const int m0 = tm * NT_BM;
   if (m0 >= Mv) return;
   const bf16_t* B = B_;
@@ -580,8 +592,9 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
       b_voff[i] = (int)(((size_t)kr * N + ((lane & 15) ^ kn_swizzle(kr)) * 8) * 2);
     }
   }
-  const bf16_t* a_tile = A + (size_t)m0 * K;
-  const bf16_t* b_tile = B_KN ? B + n0 : B + (size_t)n0 * K;
+  const int k_first = QKV || B_KN ? 0 : qkv.k_begin;
+  const bf16_t* a_tile = A + (size_t)m0 * K + k_first;
+  const bf16_t* b_tile = B_KN ? B + n0 : B + (size_t)n0 * K + k_first;
   auto issue_one = [&](char* st, int kt, int idx) {
     const int k0 = kt * BK;
     if (idx < INST) {
@@ -620,7 +633,7 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
     }
   }
 
-  const int nk = K / BK;
+  const int nk = (!QKV && !B_KN && qkv.k_len > 0 ? qkv.k_len : K) / BK;
 #pragma unroll
   for (int s = 0; s < NT_STAGES - 1; ++s)
 #pragma unroll
@@ -738,6 +751,22 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
     }
   }
 
+  if constexpr (!QKV && !B_KN) {
+    if (qkv.partial != nullptr) {
+      // A slice of K: the float32 sums as they are, four columns of a row a lane and tile.
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + wm * 64 + i * 16 + fr;
+        if (m >= Mv) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = n0 + wn * 64 + j * 16 + 4 * kq;
+          if (n + 4 <= N) *reinterpret_cast<f32x4*>(qkv.partial + (size_t)m * N + n) = acc[i][j];
+        }
+      }
+      return;
+    }
+  }
   // Output through LDS: the wave lays its 64 x 64 out row-major (rows padded by 16 bytes, which
   // spreads the 8-byte writes and the 16-byte reads over the banks) and each lane then owns 8
   // consecutive columns of a row: a row of the tile leaves as one 128-byte segment.
@@ -1475,6 +1504,147 @@ static int launch_gemm_either(const bf16_t* A, const bf16_t* B, bf16_t* C, int M
   IRON_LAUNCH_CHECK();
 }
 
+// A residual product of few rows over a long K, followed by the RMSNorm of its rows (a prompt chunk's
+// down projection: 512 live rows x 2048 columns over K = 8192, then the next layer's input norm).
+// 128 x 128 tiles would occupy a quarter of the CUs and the 64 x 64 ones that fill the chip fetch
+// every operand row twice as often, so a tile's K is dealt over `splits` blocks -- chosen on the
+// device by the row bound: 4 while the live tiles fill a quarter of the chip, 2 up to half, else
+// whole K -- each leaving its float32 sums in a workspace slice.  A second launch, a block a row,
+// adds a row's slices in slice order (the same sums whatever ran first), rounds once, adds the
+// residual, stores the row and norms it as rmsnorm_kernel does: that launch stands where the
+// norm's own stood, so the slices' sum costs no launch of its own.
+constexpr int kSplitKMax = 4;
+__device__ __host__ inline int splitk_for(int live_tiles) {
+  return live_tiles * 4 <= 256 ? 4 : (live_tiles * 2 <= 256 ? 2 : 1);
+}
+// Rows a slice of the workspace holds when K is dealt `splits` ways: the most that split count runs for.
+__device__ __host__ inline size_t splitk_slice_rows(int splits, int tiles_n) {
+  return (size_t)((256 / splits) / tiles_n) * 128;
+}
+
+__global__ __launch_bounds__(256) void gemm_splitk_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+                                                          bf16_t* __restrict__ C, int M, int N, int K,
+                                                          const int* __restrict__ valid, Tiling whole, QkvTail tail,
+                                                          float* __restrict__ partial) {
+  const int Mv = bound_or(valid, M);
+  const int tiles_n = whole.tiles_n, live_tiles = ((Mv + 127) / 128) * tiles_n;
+  const int splits = splitk_for(live_tiles), id = blockIdx.x;
+  if (splits == 1) {   // whole K a block, the residual in its epilogue: iron_gemm_residual_bf16's 128 x 128 launch
+    if (id < whole.tiles_m * whole.tiles_n)
+      gemm_nt16_body<false>(A, B, C, M, N, K, valid, whole.tiles_m, whole.tiles_n, whole.patched, tail);
+    return;
+  }
+  // The live (tile, slice) pairs are the first ids, so that they go out one a CU whatever the
+  // launch's size; an XCD (id mod 8) serves one slice of K and a band of tile columns, whose
+  // A and B pieces it then re-reads from its own L2.
+  const int live = live_tiles * splits;
+  if (id >= live) return;
+  int tile, split;
+  if (live % 8 == 0) {
+    const int xcd = id & 7, per = 8 / splits;
+    split = xcd % splits;
+    tile = (id >> 3) * per + xcd / splits;
+  } else {
+    split = id % splits;
+    tile = id / splits;
+  }
+  tail.residual = nullptr;   // the second launch adds it
+  tail.k_len = K / splits;
+  tail.k_begin = split * tail.k_len;
+  tail.partial = partial + (size_t)split * splitk_slice_rows(splits, tiles_n) * N;
+  tail.tile_plus1 = tile + 1;
+  gemm_nt16_body<false>(A, B, C, M, N, K, valid, (Mv + 127) / 128, tiles_n, 0, tail);
+}
+
+// The second launch: row `blockIdx.x` of C finished (from the slices, or as the first launch left
+// it where K was not dealt) and normed into Y.  A thread holds CHUNKS 16-byte pieces of the row;
+// every load of a piece goes out before any is used, through bounded buffers (a thread past the
+// row's end reads zeros and takes no branch).  The norm's arithmetic is rmsnorm_kernel's, sum by
+// sum, so Y is what iron_rmsnorm_bf16 makes of C bit for bit.
+template <int CHUNKS>
+__global__ __launch_bounds__(256) void gemm_finish_rows_kernel(const float* __restrict__ partial,
+                                                               const bf16_t* residual, float scale, bf16_t* C,
+                                                               const bf16_t* __restrict__ gain,
+                                                               bf16_t* __restrict__ Y, int M, int N, float eps,
+                                                               const int* __restrict__ valid, int tiles_n) {
+  const int row = blockIdx.x, nchunk = N >> 3;
+  const __amdgpu_buffer_rsrc_t gain_bytes = bounded_bytes(gain, N * 2);
+  uint4 gains[CHUNKS];
+#pragma unroll
+  for (int i = 0; i < CHUNKS; ++i) gains[i] = load_bounded(gain_bytes, 16 * (threadIdx.x + 256 * i));
+  const int Mv = bound_or(valid, M);
+  if (row >= Mv) return;
+  const int splits = splitk_for(((Mv + 127) / 128) * tiles_n);
+  uint4* c_row = reinterpret_cast<uint4*>(C + (size_t)row * N);
+  uint4 held[CHUNKS];
+  if (splits == 1) {
+    const __amdgpu_buffer_rsrc_t row_bytes = bounded_bytes(c_row, N * 2);
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) held[i] = load_bounded(row_bytes, 16 * (threadIdx.x + 256 * i));
+  } else {
+    const size_t slice = splitk_slice_rows(splits, tiles_n) * N;
+    const __amdgpu_buffer_rsrc_t res_bytes = bounded_bytes(residual + (size_t)row * N, N * 2);
+    uint4 added[CHUNKS], part[CHUNKS][kSplitKMax][2];
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      added[i] = load_bounded(res_bytes, 16 * (threadIdx.x + 256 * i));
+#pragma unroll
+      for (int sl = 0; sl < kSplitKMax; ++sl) {
+        // slices past the split count: an empty buffer, zeros
+        const __amdgpu_buffer_rsrc_t sums = bounded_bytes(partial + (sl < splits ? sl : 0) * slice + (size_t)row * N,
+                                                          sl < splits ? N * 4 : 0);
+        part[i][sl][0] = load_bounded(sums, 32 * (threadIdx.x + 256 * i));
+        part[i][sl][1] = load_bounded(sums, 32 * (threadIdx.x + 256 * i) + 16);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      float x[8], rf[8];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        f32x4 sum = __builtin_bit_cast(f32x4, part[i][0][h]);
+#pragma unroll
+        for (int sl = 1; sl < kSplitKMax; ++sl)
+          if (sl < splits) sum += __builtin_bit_cast(f32x4, part[i][sl][h]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[4 * h + e] = sum[e];
+      }
+      unpack8(added[i], rf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = fmaf(scale, round_bf16(x[e]), rf[e]);
+      held[i] = pack8(x);
+      const int c = threadIdx.x + 256 * i;
+      if (c < nchunk) c_row[c] = held[i];
+    }
+  }
+
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < CHUNKS; ++i) {
+    float f[8];
+    unpack8(held[i], f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
+  }
+  ss = wave_sum(ss);
+  __shared__ float part_sums[4];
+  if ((threadIdx.x & 63) == 0) part_sums[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float total = part_sums[0] + part_sums[1] + part_sums[2] + part_sums[3];
+  const float inv = 1.0f / sqrtf(total / (float)N + eps);
+  uint4* y_row = reinterpret_cast<uint4*>(Y + (size_t)row * N);
+#pragma unroll
+  for (int i = 0; i < CHUNKS; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    float f[8], g[8];
+    unpack8(held[i], f);
+    unpack8(gains[i], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = round_bf16(f[j] * inv) * g[j];
+    if (c < nchunk) y_row[c] = pack8(f);
+  }
+}
+
 // A gated feed-forward's two first projections on one 128 x 128 tile position AT ONCE: a stage is the
 // A tile and both weights' tiles (48 KB, three stages), an A fragment read out of LDS serves both
 // products, and the gated epilogue has both accumulators in registers in the same layout, so the
@@ -1804,6 +1974,59 @@ extern "C" int iron_gemm_residual_bf16(const uint16_t* A, const uint16_t* B, con
   tail.residual = R;
   tail.residual_scale = residual_scale;
   return gemm_with_tail("gemm_residual", A, B, R, C, M, N, K, tail, valid, stream);
+}
+
+// Whether (and with how much workspace) a residual product followed by its rows' norm is worth
+// dealing its K over several blocks: whole 128-column tiles too few to fill the chip at some row
+// count, a K long enough to cut, rows a block of the second launch can hold.
+extern "C" int64_t iron_gemm_residual_norm_workspace_bytes(int M, int N, int K) {
+  if (M < 128 || N < 128 || N % 128 != 0 || N > 8192 || K < 4096 || K % (BK * kSplitKMax) != 0) return 0;
+  const int tiles_n = N / 128;
+  // splits x the rows a split count runs for is the same for every split count: 256 tiles' worth of rows.
+  return (int64_t)(256 / tiles_n) * 128 * N * (int64_t)sizeof(float);
+}
+
+extern "C" int iron_gemm_residual_norm_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* R,
+                                            const uint16_t* gain, uint16_t* C, uint16_t* Y, int M, int N, int K,
+                                            float residual_scale, float eps, const int* valid, void* workspace,
+                                            void* stream) {
+  IRON_REQUIRE(A && B && R && gain && C && Y && workspace, "gemm_residual_norm: null operand");
+  IRON_REQUIRE(iron_gemm_residual_norm_workspace_bytes(M, N, K) > 0,
+               "gemm_residual_norm: M (%d) at least 128, N (%d) a multiple of 128 up to 8192, K (%d) a multiple of %d "
+               "from 4096 on (other shapes: iron_gemm_residual_bf16, then iron_rmsnorm_bf16)", M, N, K, BK * kSplitKMax);
+  IRON_REQUIRE(K <= (1 << 22), "gemm_residual_norm: K (%d) may be at most 2^22 (a tile's rows are addressed with 32-bit offsets)", K);
+  IRON_REQUIRE((((uintptr_t)A | (uintptr_t)B | (uintptr_t)R | (uintptr_t)gain | (uintptr_t)C | (uintptr_t)Y |
+                 (uintptr_t)workspace) & 15) == 0,
+               "gemm_residual_norm: operands must be 16-byte aligned");
+  IRON_REQUIRE(Y != C && Y != R, "gemm_residual_norm: the normed rows need a buffer of their own");
+  hipStream_t s = (hipStream_t)stream;
+  int tiles_m = (M + 127) / 128;
+  const int tiles_n = N / 128;
+  // Whole-K tiles in the XCD-aware order where whole patches allow it (the added tile rows lie past M).
+  if (tiles_m >= 8 && !patched_order(tiles_m, tiles_n) && patched_order((tiles_m + 7) & ~7, tiles_n))
+    tiles_m = (tiles_m + 7) & ~7;
+  const Tiling whole{tiles_m, tiles_n, patched_order(tiles_m, tiles_n)};
+  QkvTail tail{};
+  tail.residual = R;
+  tail.residual_scale = residual_scale;
+  constexpr size_t lds = (size_t)NT_STAGES * 256 * BK * 2;
+  static LdsOptIn opt_in;
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_splitk_kernel), lds); e != hipSuccess) {
+    set_error("gemm_residual_norm: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  const int blocks = whole.tiles_m * whole.tiles_n > 256 ? whole.tiles_m * whole.tiles_n : 256;
+  hipLaunchKernelGGL(gemm_splitk_kernel, dim3(blocks), dim3(256), lds, s, A, B, C, M, N, K, valid, whole, tail,
+                     (float*)workspace);
+  const int chunks = (N / 8 + 255) / 256;
+#define IRON_FINISH(CH)                                                                                          \
+  hipLaunchKernelGGL((gemm_finish_rows_kernel<CH>), dim3(M), dim3(256), 0, s, (const float*)workspace, R,        \
+                     residual_scale, C, gain, Y, M, N, eps, valid, tiles_n)
+  if (chunks <= 1) IRON_FINISH(1);
+  else if (chunks == 2) IRON_FINISH(2);
+  else IRON_FINISH(4);
+#undef IRON_FINISH
+  IRON_LAUNCH_CHECK();
 }
 
 extern "C" int iron_gemm_gated_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* G, uint16_t* C, int M,

@@ -79,6 +79,30 @@ def gemm_residual(A, B, R, C, *, M, N, K, residual_scale=1.0, valid=None):
                                         ptr(_word(valid, "valid")), current_stream()), "iron_gemm_residual_bf16")
 
 
+def gemm_residual_norm_workspace_bytes(M, N, K) -> int:
+    """Bytes of workspace ``gemm_residual_norm`` needs; 0 for a shape it refuses."""
+    return int(lib().iron_gemm_residual_norm_workspace_bytes(M, N, K))
+
+
+def gemm_residual_norm(A, B, R, gain, C, Y, workspace, *, M, N, K, eps, residual_scale=1.0, valid=None):
+    """``C = residual_scale * (A @ B.T) + R`` and ``Y = rmsnorm(C) * gain`` over few rows and a long K:
+    K dealt over several blocks a tile while the bound leaves the chip idle, float32 sums in
+    ``workspace`` (any contents), the rows finished and normed by a second launch."""
+    _numel(_dev(A, "A"), M * K, "A")
+    _numel(_dev(B, "B"), N * K, "B")
+    _numel(_dev(R, "R"), M * N, "R")
+    _numel(_dev(gain, "gain"), N, "gain")
+    _numel(_dev(C, "C"), M * N, "C")
+    _numel(_dev(Y, "Y"), M * N, "Y")
+    need = gemm_residual_norm_workspace_bytes(M, N, K)
+    if need and _dev(workspace, "workspace", None).numel() * workspace.element_size() < need:
+        raise ValueError(f"gemm_residual_norm: workspace holds {workspace.numel() * workspace.element_size()} bytes, "
+                         f"{need} needed")
+    check(lib().iron_gemm_residual_norm_bf16(ptr(A), ptr(B), ptr(R), ptr(gain), ptr(C), ptr(Y), M, N, K,
+                                             float(residual_scale), float(eps), ptr(_word(valid, "valid")),
+                                             ptr(workspace), current_stream()), "iron_gemm_residual_norm_bf16")
+
+
 def gemm_gated(A, B, G, C, *, M, N, K, activation="silu", valid=None):
     """``C = act(G) * (A @ B.T)`` over many rows, B stored ``(N, K)``; ``activation`` "silu" or
     "gelu_tanh"."""

@@ -328,6 +328,69 @@ def test_gemm_residual_epilogue(cuda, M, Kdim, N, rows, scale):
     close(from_torch(Rd)[:lim], want[:lim], rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("M,Kdim,N,rows,scale", [
+    (2048, 8192, 2048, 512, 1.0),     # a prompt chunk's down projection: K dealt four ways, a slice an XCD pair
+    (2048, 4096, 2048, 1024, 1.0),    # two ways
+    (2048, 4096, 2048, 1281, 0.22),   # whole K: the first launch is the plain residual product's
+    (512, 4096, 2048, None, 1.0),
+    (256, 4096, 128, 130, 1.0),       # one tile column, a tile row the bound cuts
+    (384, 4096, 384, 300, -0.5),      # pairs that do not fill whole XCD rounds
+    (256, 4096, 4096, 77, 1.0),       # two pieces of a row a thread
+    (128, 4608, 8192, None, 1.0)])    # four
+def test_gemm_residual_then_rmsnorm_with_k_dealt_over_blocks(cuda, M, Kdim, N, rows, scale):
+    """A residual product of few rows over a long K and the norm of its rows as two launches: the
+    product's K dealt over several blocks a tile (float32 sums through a workspace holding garbage),
+    the rows finished and normed by the second.  C against the oracle's product and sum; Y is the
+    norm kernel's of that C bit for bit, and within tolerance of the oracle's norm of it; rows past
+    the bound are not touched; in place on the residual stream."""
+    rng = np.random.default_rng(M + N + Kdim)
+    lim = M if rows is None else rows
+    A, B, R, gain = bf(rng, M, Kdim), bf(rng, N, Kdim, scale=0.02), bf(rng, M, N), bf(rng, N)
+    product = ops.gemm(A[:lim], B, b_col_maj=True)
+    want = ops.axpy(scale, product, R[:lim])
+    # The product is rounded before the sum: where the float32 sums differ in their last bits it may
+    # round to the neighbouring bf16 (2^-7 of it at most), whatever the sum then cancels to.
+    ulp = np.abs(scale * product) * 2.0 ** -7
+
+    def near(got, want):
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        bad = ~(err <= 1e-2 + 1e-2 * np.abs(want) + ulp)
+        assert not bad.any(), f"{bad.sum()}/{bad.size} outside the tolerance; max err {err.max():.5f}"
+
+    if rows is not None:
+        A[rows:] = np.nan
+    valid = None if rows is None else word(rows, cuda)
+    need = K.gemm_residual_norm_workspace_bytes(M, N, Kdim)
+    assert need > 0
+    ws = torch.full((need // 4,), float("nan"), dtype=torch.float32, device=cuda)
+    Ad, Bd, Rd, gd = dev(A, cuda), dev(B, cuda), dev(R, cuda), dev(gain, cuda)
+    C, Y = out_like((M, N), cuda, fill=7.0), out_like((M, N), cuda, fill=7.0)
+    K.gemm_residual_norm(Ad, Bd, Rd, gd, C, Y, ws, M=M, N=N, K=Kdim, eps=1e-6, residual_scale=scale, valid=valid)
+    got = from_torch(C)
+    near(got[:lim], want)
+    assert np.all(got[lim:] == 7.0) and bool((Y[lim:] == 7.0).all())
+    normed = out_like((M, N), cuda, fill=7.0)
+    K.rmsnorm(C, gd, normed, rows=M, cols=N, eps=1e-6, valid=valid)
+    assert torch.equal(Y[:lim], normed[:lim])
+    close(from_torch(Y)[:lim], ops.rms_norm(got[:lim], gain, epsilon=1e-6), rtol=1e-2, atol=1e-2)
+    # again over the workspace the first call left, in place on the residual stream: the same bits
+    Y2 = out_like((M, N), cuda, fill=7.0)
+    K.gemm_residual_norm(Ad, Bd, Rd, gd, Rd, Y2, ws, M=M, N=N, K=Kdim, eps=1e-6, residual_scale=scale, valid=valid)
+    assert torch.equal(Rd[:lim], C[:lim]) and torch.equal(Y2[:lim], Y[:lim])
+    assert np.array_equal(from_torch(Rd)[lim:], R[lim:])
+
+
+def test_gemm_residual_then_rmsnorm_refuses_other_shapes(cuda):
+    """Shapes whose K is too short to deal, or whose rows the second launch cannot hold, report no
+    workspace and are refused with a reason before any launch."""
+    for M, N, Kdim in ((64, 2048, 8192), (512, 2048, 2048), (512, 2000, 8192), (512, 16384, 8192), (512, 2048, 8192 + 64)):
+        assert K.gemm_residual_norm_workspace_bytes(M, N, Kdim) == 0
+    t, w = out_like((512 * 2048,), cuda, fill=0.0), out_like((2048 * 2048,), cuda, fill=0.0)
+    with pytest.raises(Exception, match="iron_gemm_residual_norm_bf16 refused"):
+        K.gemm_residual_norm(t, w, t, t[:2048], t, out_like((512 * 2048,), cuda), torch.empty(16, device=cuda),
+                             M=512, N=2048, K=2048, eps=1e-6)
+
+
 @pytest.mark.parametrize("M,Kdim,N,rows,activation", [
     (2048, 2048, 8192, 512, "silu"), (2048, 256, 8192, None, "silu"), (2048, 256, 2048, 1500, "silu"),
     (256, 128, 512, 100, "silu"), (128, 64, 64, None, "silu"), (4096, 192, 1024, 3000, "silu"), (200, 128, 136, None, "silu"),

@@ -327,6 +327,11 @@ def test_a_512_token_prompt_in_a_2048_row_chunk_at_llama_1b_width(cuda):
     gpu.load_versions()
     cpu.load_versions()
     try:
+        # a layer's down projection, its residual and the next layer's input norm are one run (K dealt
+        # over several blocks a tile under this bound, the rows finished and normed by a second launch)
+        kinds = [f.kind for f in gpu.prompt_chunk._fused.values()]
+        assert kinds.count("gemm_add_norm") == config.num_hidden_layers - 1
+        assert kinds.count("gemm_add") == config.num_hidden_layers + 1
         tokens = np.random.default_rng(2).integers(0, config.vocab_size, 512)
         want, got = cpu.logits(tokens), gpu.logits(tokens)
         assert_close(got, want)
