@@ -1215,7 +1215,7 @@ constexpr int BIG_KB = IRON_BIG_KB;   // k per stage: 64 (2 stages); 32 (4 stage
 #define BIG_OUT_ROW_BYTES(TN) ((TN) * 64 + 16)
 constexpr int BIG_STAGE_BYTES = (BIG_BM + BIG_BN) * BK * 2;
 
-template <int WAVES, int KB, bool B_KN = false>
+template <int WAVES, int KB, bool B_KN = false, bool STREAM_OUT = false>
 __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
                                                 bf16_t* __restrict__ C, int M, int N, int K,
                                                 const int* __restrict__ valid, int tiles_m, int tiles_n,
@@ -1429,21 +1429,32 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   constexpr int ORPI = 64 / LPRW;     // rows per instruction
   const int lr = lane / LPRW, lc = lane % LPRW;
   bf16_t* cbase = C + (size_t)(m0 + wm * 128) * N + n0 + wn * TN * 32 + lc * 8;
+  // STREAM_OUT (the launch sets it over a long K): the tile leaves by non-temporal stores, so C's
+  // lines do not stay in the XCD's L2 among the A and B panels its blocks re-read (8192^3: 790 ->
+  // 750 us; 1 to 5 % from K = 4096 on, and 1.5 % slower at K = 2048, where a tile's stores are a
+  // larger part of its time).  A template argument: as a branch on K the compiler merged the two
+  // stores into one plain one.
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 #pragma unroll 4
   for (int r0 = 0; r0 < 128; r0 += ORPI) {
     const int r = r0 + lr;
     const uint4 v = *reinterpret_cast<const uint4*>(ot + r * OROWB + lc * 16);
-    if (m0 + wm * 128 + r < Mv) *reinterpret_cast<uint4*>(cbase + (size_t)r * N) = v;
+    if (m0 + wm * 128 + r < Mv) {
+      if constexpr (STREAM_OUT)
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x4_t, v), reinterpret_cast<u32x4_t*>(cbase + (size_t)r * N));
+      else
+        *reinterpret_cast<uint4*>(cbase + (size_t)r * N) = v;
+    }
   }
 }
 
-template <int WAVES, int KB, bool B_KN = false>
+template <int WAVES, int KB, bool B_KN = false, bool STREAM_OUT = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_nt256_kernel(const bf16_t* __restrict__ A,
                                                          const bf16_t* __restrict__ B,
                                                          bf16_t* __restrict__ C, int M, int N, int K,
                                                          const int* __restrict__ valid, int tiles_m,
                                                          int tiles_n, int patched) {
-  gemm_nt256_body<WAVES, KB, B_KN>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched);
+  gemm_nt256_body<WAVES, KB, B_KN, STREAM_OUT>(A, B, C, M, N, K, valid, tiles_m, tiles_n, patched);
 }
 
 // A row bound read on the device decides which tile size fills the chip best (512 valid rows of
@@ -1875,21 +1886,30 @@ static int launch_gemm_gated_pair(const bf16_t* A, const bf16_t* Bg, const bf16_
   IRON_LAUNCH_CHECK();
 }
 
-template <bool B_KN = false>
-static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
-                             const int* valid, hipStream_t s) {
+template <bool B_KN, bool STREAM_OUT>
+static int launch_gemm_nt256_as(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
+                                const int* valid, hipStream_t s) {
   const int tiles_m = M / BIG_BM, tiles_n = N / BIG_BN;
   constexpr size_t out_bytes = (size_t)BIG_WAVES * 128 * BIG_OUT_ROW_BYTES(8 / BIG_WAVES * 2);
   const size_t lds = out_bytes > (size_t)2 * BIG_STAGE_BYTES ? out_bytes : (size_t)2 * BIG_STAGE_BYTES;
   static LdsOptIn opt_in;
-  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>), lds); e != hipSuccess) {
+  if (hipError_t e = opt_in.ensure(reinterpret_cast<const void*>(&gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN, STREAM_OUT>), lds);
+      e != hipSuccess) {
     set_error("gemm: %s", hipGetErrorString(e));
     return (int)e;
   }
   const int patched = (tiles_m % 8 == 0 && tiles_n % 4 == 0 && ((tiles_m / 8) * (tiles_n / 4)) % 8 == 0) ? 1 : 0;
-  hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s, A, B, C, M, N, K, valid,
-                     tiles_m, tiles_n, patched);
+  hipLaunchKernelGGL((gemm_nt256_kernel<BIG_WAVES, BIG_KB, B_KN, STREAM_OUT>), dim3(tiles_m * tiles_n), dim3(BIG_WAVES * 64), lds, s,
+                     A, B, C, M, N, K, valid, tiles_m, tiles_n, patched);
   IRON_LAUNCH_CHECK();
+}
+
+// Over a long K the tiles leave by non-temporal stores (see the body's epilogue).
+template <bool B_KN = false>
+static int launch_gemm_nt256(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, int K,
+                             const int* valid, hipStream_t s) {
+  if (K >= 4096) return launch_gemm_nt256_as<B_KN, true>(A, B, C, M, N, K, valid, s);
+  return launch_gemm_nt256_as<B_KN, false>(A, B, C, M, N, K, valid, s);
 }
 
 }  // namespace iron
