@@ -220,6 +220,24 @@ __device__ __forceinline__ short4v lds_read_tr16_at(unsigned lds_addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFFSET));
   return v;
 }
+// A 16-byte LDS read the compiler does not count (for loops that also issue the reads above: the
+// waits it would insert count only the reads it knows, so they come out too strict and wait for
+// reads issued long after the one that is needed).  The result must pass through lds_wait_for<N>().
+template <int OFFSET>
+__device__ __forceinline__ bf16x8 lds_read_b128_at(unsigned lds_addr) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "the offset field holds 16 bits");
+  i32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFFSET));
+  return __builtin_bit_cast(bf16x8, v);
+}
+// Waits until at most N LDS reads issued after `frag`'s are outstanding (they return in order).
+template <int N>
+__device__ __forceinline__ void lds_wait_for(bf16x8& frag) {
+  static_assert(N >= 0 && N <= 15, "the counter's field holds four bits");
+  i32x4 v = __builtin_bit_cast(i32x4, frag);
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
+  frag = __builtin_bit_cast(bf16x8, v);
+}
 struct TrFrag {   // the two halves of a fragment, as the reads deliver them
   short4v lo, hi;
 };

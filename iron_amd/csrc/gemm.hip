@@ -15,6 +15,8 @@
 #include "../../include/iron_hip.h"
 #include "common.h"
 
+#include <type_traits>
+
 
 namespace iron {
 
@@ -654,12 +656,32 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
   // transposing read hands a 16-lane group the 4 k-rows x 16 columns its lanes point at, turned
   // round (a lane gets 4 k of one column): rows 8 kq .. + 3, then 8 kq + 4 .. + 7.
   const int tr_k = 8 * kq + ((lane & 15) >> 2), tr_n = wn * 64 + 4 * (lane & 3);
-  const unsigned kn_base = (unsigned)(size_t)IRON_LDS_PTR(smem_nt) + NT_A_BYTES;
-  auto b_frag_kn = [&](int stage_bytes, int ks, int j, TrFrag& t) {
-    const int k = ks * 32 + tr_k, n = tr_n + j * 16;   // kn_swizzle(k + 4) = kn_swizzle(k): k % 8 < 4
-    const unsigned at = kn_base + stage_bytes + (((n >> 3) ^ kn_swizzle(k)) << 4) + ((n & 4) << 1);
-    t.lo = lds_read_tr16(at + k * 256);
-    t.hi = lds_read_tr16(at + (k + 4) * 256);
+  const unsigned lds_base_nt = (unsigned)(size_t)IRON_LDS_PTR(smem_nt);
+  const unsigned kn_base = lds_base_nt + NT_A_BYTES;
+  // The lane's place in a stage's B tile for tile j (k-step 0, low half) is fixed for the whole loop;
+  // the k-step (32 rows on) and the high half (4 rows on) leave the swizzle as it is -- kn_swizzle(k +
+  // 4) = kn_swizzle(k) for k % 8 < 4, and k + 32 keeps the bits it reads -- and the (K,N) loop is
+  // unrolled over the four stage buffers, so k-step, half and stage all ride in the reads' offset
+  // fields (16 bits: a second set of lane addresses two stages on) and a fragment read costs no
+  // vector arithmetic at all: with one wave a SIMD every vector instruction between two MFMAs is
+  // time off the matrix pipe (sixteen adds a k-step, then four, then none: 2048^3 25.0 -> 23.5 -> 22.7 us).
+  unsigned kn_lane[2][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = tr_n + j * 16;
+    kn_lane[0][j] = kn_base + (((n >> 3) ^ kn_swizzle(tr_k)) << 4) + ((n & 4) << 1) + tr_k * 256;
+    kn_lane[1][j] = kn_lane[0][j] + 2 * NT_STAGE_BYTES;
+  }
+  auto b_frag_kn = [&](auto stage_c, int ks, int j, TrFrag& t) {
+    constexpr int STAGE = decltype(stage_c)::value, OFF = (STAGE & 1) * NT_STAGE_BYTES;
+    const unsigned at = kn_lane[STAGE >> 1][j];
+    if (ks == 0) {
+      t.lo = lds_read_tr16_at<OFF>(at);
+      t.hi = lds_read_tr16_at<OFF + 4 * 256>(at);
+    } else {
+      t.lo = lds_read_tr16_at<OFF + 32 * 256>(at);
+      t.hi = lds_read_tr16_at<OFF + 36 * 256>(at);
+    }
   };
   TrFrag tfb[2][4];
   // The compiler does not count the transposing reads: a k-step's B fragments pass through this
@@ -672,26 +694,54 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
 #pragma unroll
     for (int j = 0; j < 4; ++j) b[j] = tr_join(tfb[ks][j]);
   };
+  // (K,N): the A fragments are read by uncounted reads as well, so that every wait of the loop is
+  // this code's own.  With counted A reads the compiler's waits for them took no account of the
+  // transposing reads issued in between and came out as "all but two outstanding" where eleven
+  // were in flight: each k-step waited an LDS trip for fragments of the NEXT one (a quarter of
+  // the loop's time).  The lane's place in a stage for k-step ks; tile row i is the read's offset.
+  unsigned a_lane[2][2];   // [stage / 2][k-step]
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    a_lane[0][ks] = lds_base_nt + a_row + (((ks * 4 + kq) ^ swz) << 4);
+    a_lane[1][ks] = a_lane[0][ks] + 2 * NT_STAGE_BYTES;
+  }
+  auto a_frags_kn = [&](auto stage_c, int ks, int i, bf16x8& out) {
+    constexpr int STAGE = decltype(stage_c)::value, OFF = (STAGE & 1) * NT_STAGE_BYTES;
+    const unsigned at = a_lane[STAGE >> 1][ks];
+    if (i == 0) out = lds_read_b128_at<OFF + 0 * 16 * 128>(at);
+    else if (i == 1) out = lds_read_b128_at<OFF + 1 * 16 * 128>(at);
+    else if (i == 2) out = lds_read_b128_at<OFF + 2 * 16 * 128>(at);
+    else out = lds_read_b128_at<OFF + 3 * 16 * 128>(at);
+  };
 
   wait_vmcnt<(NT_STAGES - 2) * LOADS>();   // stage 0 has landed once only the two younger ones are out
   block_barrier();
   bf16x8 af[2][4], bfr[2][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    if constexpr (B_KN) b_frag_kn(0, 0, i, tfb[0][i]);
+    if constexpr (B_KN) b_frag_kn(std::integral_constant<int, 0>{}, 0, i, tfb[0][i]);
     else bfr[0][i] = b_frag(smem_nt, 0, i);
   }
   __builtin_amdgcn_sched_barrier(0);   // B's reads first, then A's: join_b counts on that order
 #pragma unroll
-  for (int i = 0; i < 4; ++i) af[0][i] = a_frag(smem_nt, 0, i);
-  for (int kt = 0; kt < nk; ++kt) {
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (B_KN) a_frags_kn(std::integral_constant<int, 0>{}, 0, i, af[0][i]);
+    else af[0][i] = a_frag(smem_nt, 0, i);
+  }
+  // One stage of the loop.  stage_c: kt % NT_STAGES where the caller knows it (the (K,N) loop,
+  // unrolled over the stage buffers), -1 where it does not.
+  auto stage_step = [&](int kt, auto stage_c) {
+    constexpr int STAGE = decltype(stage_c)::value;
+    static_assert(STAGE < 0 || B_KN, "only the (K,N) loop names its stage");
     // Prefetch goes into the buffer of stage kt-1.  Past the end the last stage is fetched again
     // (into buffers nobody reads any more) rather than branch: every iteration issues the same
     // loads, which keeps the wait counts exact and the scheduling region whole.
     const int kn = min(kt + NT_STAGES - 1, nk - 1);
-    char* nst = smem_nt + ((kt + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
-    const char* st = smem_nt + (kt % NT_STAGES) * NT_STAGE_BYTES;
-    const char* st1 = smem_nt + ((kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
+    const int s_now = STAGE >= 0 ? STAGE : kt % NT_STAGES;
+    char* nst = smem_nt + ((s_now + NT_STAGES - 1) % NT_STAGES) * NT_STAGE_BYTES;
+    const char* st = smem_nt + s_now * NT_STAGE_BYTES;
+    const char* st1 = smem_nt + ((s_now + 1) % NT_STAGES) * NT_STAGE_BYTES;
+    constexpr int STAGE_NEXT = STAGE >= 0 ? (STAGE + 1) % NT_STAGES : 0;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       if (ks == 1) {
@@ -703,26 +753,57 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
         block_barrier();
       }
       const char* from = ks == 0 ? st : st1;
-      const int from_bytes = ((ks == 0 ? kt : kt + 1) % NT_STAGES) * NT_STAGE_BYTES;
       const int nks = ks ^ 1;
       if constexpr (B_KN) join_b(ks, bfr[ks]);
       // Source order is issue order (nothing crosses a sched_barrier): after an MFMA one fragment
       // read of the next k-step (B's first: its first MFMAs need all of them) or one load goes out.
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (B_KN) {
+          // Reads in flight when tile row i starts, in issue order: this k-step's A fragments from
+          // i on, then what this k-step has issued for the next one (8 transposing reads during
+          // row 0, 4 A reads during row 1): fragment i has arrived once all but those after it have.
+          if (i == 0) lds_wait_for<3>(af[ks][0]);         // after join_b: a1 a2 a3 may be out
+          else if (i == 1) lds_wait_for<10>(af[ks][1]);   // a2 a3 + 8
+          else if (i == 2) lds_wait_for<13>(af[ks][2]);   // a3 + 8 + 4
+          else lds_wait_for<12>(af[ks][3]);               // 8 + 4
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           mfma_16x16x32_in_place(acc[i][j], bfr[ks][j], af[ks][i]);
           __builtin_amdgcn_sched_barrier(0);
           const int slot = i * 4 + j;
           if (slot < 4) {
-            if constexpr (B_KN) b_frag_kn(from_bytes, nks, slot, tfb[nks][slot]);
-            else bfr[nks][slot] = b_frag(from, nks, slot);
-          } else if (slot < 8) af[nks][slot - 4] = a_frag(from, nks, slot - 4);
-          else if (slot & 1) issue_one(nst, kn, ks * 4 + (slot - 9) / 2);
+            if constexpr (B_KN) {
+              if (ks == 0) b_frag_kn(std::integral_constant<int, (STAGE >= 0 ? STAGE : 0)>{}, nks, slot, tfb[nks][slot]);
+              else b_frag_kn(std::integral_constant<int, STAGE_NEXT>{}, nks, slot, tfb[nks][slot]);
+            } else {
+              bfr[nks][slot] = b_frag(from, nks, slot);
+            }
+          } else if (slot < 8) {
+            if constexpr (B_KN) {
+              if (ks == 0) a_frags_kn(std::integral_constant<int, (STAGE >= 0 ? STAGE : 0)>{}, nks, slot - 4, af[nks][slot - 4]);
+              else a_frags_kn(std::integral_constant<int, STAGE_NEXT>{}, nks, slot - 4, af[nks][slot - 4]);
+            } else {
+              af[nks][slot - 4] = a_frag(from, nks, slot - 4);
+            }
+          } else if (slot & 1) issue_one(nst, kn, ks * 4 + (slot - 9) / 2);
           __builtin_amdgcn_sched_barrier(0);
         }
+      }
     }
+  };
+  if constexpr (B_KN) {
+    for (int kt0 = 0; kt0 < nk; kt0 += NT_STAGES) {
+      stage_step(kt0, std::integral_constant<int, 0>{});
+      if (kt0 + 1 < nk) stage_step(kt0 + 1, std::integral_constant<int, 1>{});
+      if (kt0 + 2 < nk) stage_step(kt0 + 2, std::integral_constant<int, 2>{});
+      if (kt0 + 3 < nk) stage_step(kt0 + 3, std::integral_constant<int, 3>{});
+    }
+    static_assert(NT_STAGES == 4, "the loop above names the four stage buffers");
+  } else {
+    for (int kt = 0; kt < nk; ++kt) stage_step(kt, std::integral_constant<int, -1>{});
   }
 
   wait_vmcnt<0>();   // the idle fetches of the last iterations land ...
