@@ -1394,25 +1394,65 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   // transposing read hands a 16-lane group the 4 x 16 block its lanes point at (4 k-rows, each
   // lane 4 columns) turned round: the lane gets 4 k of one column.  Rows 8 kq .. + 3 and 8 kq + 4 .. + 7.
   const int tr_k = 8 * kq + ((lane & 15) >> 2), tr_n = wn * NT * 16 + 4 * (lane & 3);
-  const unsigned kn_base = (unsigned)(size_t)IRON_LDS_PTR(smem_big) + A_BYTES;
+  const unsigned lds_base_big = (unsigned)(size_t)IRON_LDS_PTR(smem_big);
+  const unsigned kn_base = lds_base_big + A_BYTES;
+  // The lane's place in a stage's B tile for tile j (k-step 0, low half) is fixed before the loop; the
+  // k-step (32 rows on) and the high half (4 rows on) leave the swizzle as it is and ride in the
+  // reads' offset fields, so a k-step's reads cost one vector add a tile (the stage) and no more.
+  // (Unrolled over its two stage buffers so that the stage too is an offset field, as the 128 x 128
+  // loop is, this kernel spilled a hundred registers: two waves a SIMD leave it 256.)
+  unsigned kn_lane[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = tr_n + j * 16;
+    kn_lane[j] = kn_base + (((n >> 3) ^ kn_swizzle(tr_k)) << 4) + ((n & 4) << 1) + tr_k * 512;
+  }
   auto b_frag_kn = [&](int stage_bytes, int ks, int j, TrFrag& t) {
-    const int k = ks * 32 + tr_k, n = tr_n + j * 16;   // kn_swizzle(k + 4) = kn_swizzle(k): k % 8 < 4
-    const unsigned at = kn_base + stage_bytes + (((n >> 3) ^ kn_swizzle(k)) << 4) + ((n & 4) << 1);
-    t.lo = lds_read_tr16(at + k * 512);
-    t.hi = lds_read_tr16(at + (k + 4) * 512);
+    const unsigned at = kn_lane[j] + stage_bytes;
+    if (ks == 0) {
+      t.lo = lds_read_tr16_at<0>(at);
+      t.hi = lds_read_tr16_at<4 * 512>(at);
+    } else {
+      t.lo = lds_read_tr16_at<32 * 512>(at);
+      t.hi = lds_read_tr16_at<36 * 512>(at);
+    }
+  };
+  // (K,N): the A fragments are read by uncounted reads as well, so that every wait of the loop is
+  // this code's own (the compiler's waits for counted A reads take no account of the transposing
+  // reads issued in between and come out far too strict).  A k-step's fragments, A's and B's, are
+  // all issued before join_b's wait at its start, which they pass through.
+  const unsigned a_lane[2] = {lds_base_big + a_row + (((0 * 4 + kq) ^ swz) << 4), lds_base_big + a_row + (((1 * 4 + kq) ^ swz) << 4)};
+  auto a_frag_kn = [&](int stage_bytes, int ks, int i, bf16x8& out) {
+    const unsigned at = a_lane[ks] + stage_bytes;
+    if (i == 0) out = lds_read_b128_at<0 * 16 * ROWB>(at);
+    else if (i == 1) out = lds_read_b128_at<1 * 16 * ROWB>(at);
+    else if (i == 2) out = lds_read_b128_at<2 * 16 * ROWB>(at);
+    else if (i == 3) out = lds_read_b128_at<3 * 16 * ROWB>(at);
+    else if (i == 4) out = lds_read_b128_at<4 * 16 * ROWB>(at);
+    else if (i == 5) out = lds_read_b128_at<5 * 16 * ROWB>(at);
+    else if (i == 6) out = lds_read_b128_at<6 * 16 * ROWB>(at);
+    else out = lds_read_b128_at<7 * 16 * ROWB>(at);
   };
   TrFrag tfb[2][NT];
-  // The compiler does not count the transposing reads: a k-step's B fragments pass through this
-  // wait (every LDS read issued so far) before they are joined into operands.
-  auto join_b = [&](int ks, bf16x8 (&b)[NT]) {
+  // The compiler does not count these reads: a k-step's fragments pass through this wait (every LDS
+  // read issued so far) before they are used.
+  auto join_b = [&](int ks, bf16x8 (&b)[NT], bf16x8 (&a)[8]) {
+    i32x4 a0 = __builtin_bit_cast(i32x4, a[0]), a1 = __builtin_bit_cast(i32x4, a[1]), a2 = __builtin_bit_cast(i32x4, a[2]),
+          a3 = __builtin_bit_cast(i32x4, a[3]), a4 = __builtin_bit_cast(i32x4, a[4]), a5 = __builtin_bit_cast(i32x4, a[5]),
+          a6 = __builtin_bit_cast(i32x4, a[6]), a7 = __builtin_bit_cast(i32x4, a[7]);
     if constexpr (NT == 4)
       asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tfb[ks][0].lo), "+v"(tfb[ks][0].hi), "+v"(tfb[ks][1].lo), "+v"(tfb[ks][1].hi),
-                                             "+v"(tfb[ks][2].lo), "+v"(tfb[ks][2].hi), "+v"(tfb[ks][3].lo), "+v"(tfb[ks][3].hi));
+                                             "+v"(tfb[ks][2].lo), "+v"(tfb[ks][2].hi), "+v"(tfb[ks][3].lo), "+v"(tfb[ks][3].hi),
+                                             "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7));
     else
       asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tfb[ks][0].lo), "+v"(tfb[ks][0].hi), "+v"(tfb[ks][1].lo), "+v"(tfb[ks][1].hi),
                                              "+v"(tfb[ks][2].lo), "+v"(tfb[ks][2].hi), "+v"(tfb[ks][3].lo), "+v"(tfb[ks][3].hi),
                                              "+v"(tfb[ks][4].lo), "+v"(tfb[ks][4].hi), "+v"(tfb[ks][5].lo), "+v"(tfb[ks][5].hi),
-                                             "+v"(tfb[ks][6].lo), "+v"(tfb[ks][6].hi), "+v"(tfb[ks][7].lo), "+v"(tfb[ks][7].hi));
+                                             "+v"(tfb[ks][6].lo), "+v"(tfb[ks][6].hi), "+v"(tfb[ks][7].lo), "+v"(tfb[ks][7].hi),
+                                             "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7));
+    a[0] = __builtin_bit_cast(bf16x8, a0); a[1] = __builtin_bit_cast(bf16x8, a1); a[2] = __builtin_bit_cast(bf16x8, a2);
+    a[3] = __builtin_bit_cast(bf16x8, a3); a[4] = __builtin_bit_cast(bf16x8, a4); a[5] = __builtin_bit_cast(bf16x8, a5);
+    a[6] = __builtin_bit_cast(bf16x8, a6); a[7] = __builtin_bit_cast(bf16x8, a7);
 #pragma unroll
     for (int j = 0; j < NT; ++j) b[j] = tr_join(tfb[ks][j]);
   };
@@ -1421,7 +1461,10 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
   block_barrier();
   bf16x8 af[2][8], bfr[2][NT];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) af[0][i] = a_frag(smem_big, 0, i);
+  for (int i = 0; i < 8; ++i) {
+    if constexpr (B_KN) a_frag_kn(0, 0, i, af[0][i]);
+    else af[0][i] = a_frag(smem_big, 0, i);
+  }
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     if constexpr (B_KN) b_frag_kn(0, 0, j, tfb[0][j]);
@@ -1449,7 +1492,7 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
     const int st_bytes = (kt % STAGES) * STAGE_BYTES, nst_bytes = ((kt + 1) % STAGES) * STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      if constexpr (B_KN) join_b(ks, bfr[ks]);
+      if constexpr (B_KN) join_b(ks, bfr[ks], af[ks]);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int quarter = ks * 2 + (i >> 2), q = i & 3;   // q: the quarter's tile row
@@ -1469,13 +1512,18 @@ __device__ __forceinline__ void gemm_nt256_body(const bf16_t* __restrict__ A, co
               else bfr[1][slot] = b_frag(st, 1, slot);
             } else if ((slot - NT) % Q0_EVERY == 0 && (slot - NT) / Q0_EVERY < INST) issue_half(nst, k1, 1, (slot - NT) / Q0_EVERY);
           } else if (quarter == 1) {
-            if (slot < 8) af[1][slot] = a_frag(st, 1, slot);
+            if (slot < 8) {
+              if constexpr (B_KN) a_frag_kn(st_bytes, 1, slot, af[1][slot]);
+              else af[1][slot] = a_frag(st, 1, slot);
+            }
           } else if (quarter == 3) {
             if (slot < NT) {
               if constexpr (B_KN) b_frag_kn(nst_bytes, 0, slot, tfb[0][slot]);
               else bfr[0][slot] = b_frag(nst, 0, slot);
-            } else if (slot < Q3_FIRST) af[0][slot - NT] = a_frag(nst, 0, slot - NT);
-            else if ((slot - Q3_FIRST) % Q3_EVERY == 0 && (slot - Q3_FIRST) / Q3_EVERY < INST)
+            } else if (slot < Q3_FIRST) {
+              if constexpr (B_KN) a_frag_kn(nst_bytes, 0, slot - NT, af[0][slot - NT]);
+              else af[0][slot - NT] = a_frag(nst, 0, slot - NT);
+            } else if ((slot - Q3_FIRST) % Q3_EVERY == 0 && (slot - Q3_FIRST) / Q3_EVERY < INST)
               issue_half(st, k2, 0, (slot - Q3_FIRST) / Q3_EVERY);
           }
           __builtin_amdgcn_sched_barrier(0);
