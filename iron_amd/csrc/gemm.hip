@@ -1073,11 +1073,14 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
   af[0] = frag(smem_q3, a_off, 0);
 #pragma unroll
   for (int j = 0; j < NACC; ++j) bfr[0][j] = frag(smem_q3, b_off + j * 32 * 128, 0);
-  for (int kt = 0; kt < nk; ++kt) {
+  // One stage of the loop, which is unrolled over the three stage buffers (stage_c = kt % Q3_STAGES):
+  // a fragment's stage then rides in its read's offset field instead of a vector add a read.
+  auto stage_step = [&](int kt, auto stage_c) {
+    constexpr int S = decltype(stage_c)::value;
     const int kn = min(kt + Q3_STAGES - 1, nk - 1);
-    char* nst = smem_q3 + ((kt + Q3_STAGES - 1) % Q3_STAGES) * Q3_STAGE_BYTES;
-    const char* st = smem_q3 + (kt % Q3_STAGES) * Q3_STAGE_BYTES;
-    const char* st1 = smem_q3 + ((kt + 1) % Q3_STAGES) * Q3_STAGE_BYTES;
+    char* nst = smem_q3 + ((S + Q3_STAGES - 1) % Q3_STAGES) * Q3_STAGE_BYTES;
+    const char* st = smem_q3 + S * Q3_STAGE_BYTES;
+    const char* st1 = smem_q3 + ((S + 1) % Q3_STAGES) * Q3_STAGE_BYTES;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
@@ -1103,6 +1106,12 @@ __device__ __forceinline__ void qkv_heads_body(const bf16_t* __restrict__ A, con
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  };
+  static_assert(Q3_STAGES == 3, "the loop below names the three stage buffers");
+  for (int kt0 = 0; kt0 < nk; kt0 += Q3_STAGES) {
+    stage_step(kt0, std::integral_constant<int, 0>{});
+    if (kt0 + 1 < nk) stage_step(kt0 + 1, std::integral_constant<int, 1>{});
+    if (kt0 + 2 < nk) stage_step(kt0 + 2, std::integral_constant<int, 2>{});
   }
   }
   wait_vmcnt<0>();   // the idle fetches of the last iterations land before the block's LDS is released
