@@ -499,10 +499,16 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
         model.release()
         return None, None
 
-    t0 = time.perf_counter()
-    carry = prefill()
-    torch.cuda.synchronize()
-    ttft = time.perf_counter() - t0
+    # The time to the first token: the median of five prefills of the same prompt (host clock around a
+    # call and its synchronization; one sample moves by a tenth with the host's scheduling).
+    ttfts = []
+    for _ in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        carry = prefill()
+        torch.cuda.synchronize()
+        ttfts.append(time.perf_counter() - t0)
+    ttft = float(np.median(ttfts))
 
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -522,7 +528,7 @@ def bench_decoder(torch, dev, steps, warmup, with_cpu, probe_steps=0):
     per_token = weight_bytes + kv_bytes
     tok_s = steps / (ms / 1e3)
     out = {"tok_s": round(tok_s, 1), "ms_per_token": round(ms / steps, 4), "ttft_ms": round(ttft * 1e3, 2),
-           "prefill_tokens": 512, "decode_steps": steps, "wall_s": round(wall, 4),
+           "ttft_runs_ms": [round(t * 1e3, 2) for t in ttfts], "prefill_tokens": 512, "decode_steps": steps, "wall_s": round(wall, 4),
            "bytes_per_token": int(per_token), "GBps": round(per_token * tok_s / 1e9, 1),
            "frac_hbm": round(per_token * tok_s / 1e9 / HBM_PEAK_GBS, 4),
            "steps_recorded": len(decode.recording.steps),
