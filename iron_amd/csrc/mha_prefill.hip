@@ -135,7 +135,8 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int e = 0; e < 16; ++e) oacc[t][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;   // the running max is of the raw (unscaled) scores
+  float m_run = -INFINITY, l_run = 0.f;   // the reference maximum (of the raw, unscaled scores) and the sum against it
+  float mc = 0.f;                         // the reference in the exp2 domain, 0 while it is -inf
 
   // Keys this block's live queries can see.
   const int q_last = min(q0 + BQW, q_tokens) - 1;
@@ -279,10 +280,19 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
           for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
         rmax = max_with_other_half(rmax);
-        const float m_new = fmaxf(m_run, rmax);
-        const float mc = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
-        const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc));  // exp2(-inf) = 0 at the start
-        m_run = m_new;
+        // The reference the exponents are taken against follows the maxima lazily: it moves, and
+        // the sums so far are rescaled, only when some query's maximum has left it more than
+        // kLazyBits doublings behind (a probability is then at most 2^kLazyBits).  Moving on every
+        // new maximum rescaled two tiles in three at S = 8192: any of a wave's 32 queries decides.
+        const bool moves = __builtin_amdgcn_ballot_w64((rmax - m_run) * scale_log2 > kLazyBits) != 0;   // -inf - -inf: no
+        float alpha = 1.f;
+        if (moves) {
+          const float m_new = fmaxf(m_run, rmax);
+          const float mc_new = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
+          alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc_new));  // exp2(-inf) = 0 at the start
+          m_run = m_new;
+          mc = mc_new;
+        }
         float rsum = 0.f;
         bf16x8 pf[2][2];
 #pragma unroll
@@ -298,8 +308,7 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
             pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
           }
         l_run = l_run * alpha + rsum;
-        // After the first tiles a new maximum is rare: rescale O only when some query's moved.
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+        if (moves) {   // the output sums follow the reference (here, where the scores' registers are free again)
 #pragma unroll
           for (int t = 0; t < DT; ++t)
 #pragma unroll
