@@ -30,6 +30,7 @@ __device__ __forceinline__ float max_with_other_half(float x) {
 constexpr int BQ = 128;   // query rows per block (four waves of 32; 64 where a block is two)
 constexpr int BKV = 64;   // key rows per tile
 constexpr float kLazyBits = 8.f;        // how far a maximum may run ahead of the reference the exponents are taken against
+constexpr float kSumLow = 0x1p-60f, kSumHigh = 0x1p24f;   // a tile's sum of exponentials outside this range: take its maximum and redo it
 constexpr int kCUs = 256;                // compute units the block orders below assume
 constexpr int kFewBlocks = 512;          // launches of fewer blocks than this halve their blocks' queries (S = 1024 at 32 heads: 18.5 -> 13.9 us)
 constexpr int kWideBigBlocks = 512;     // wide heads: launches of at least this many 128-query blocks keep that size
@@ -274,39 +275,54 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
             for (int e = 0; e < 16; ++e)
               sacc[t][e] = (unsigned)(rel + 32 * t + 8 * (e >> 2) + (e & 3)) > see_span ? -INFINITY : sacc[t][e];
         }
-        float rmax = sacc[0][0];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
-        rmax = max_with_other_half(rmax);
         // The reference the exponents are taken against follows the maxima lazily: it moves, and
         // the sums so far are rescaled, only when some query's maximum has left it more than
-        // kLazyBits doublings behind (a probability is then at most 2^kLazyBits).  Moving on every
-        // new maximum rescaled two tiles in three at S = 8192: any of a wave's 32 queries decides.
-        const bool moves = __builtin_amdgcn_ballot_w64((rmax - m_run) * scale_log2 > kLazyBits) != 0;   // -inf - -inf: no
-        float alpha = 1.f;
-        if (moves) {
-          const float m_new = fmaxf(m_run, rmax);
-          const float mc_new = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
-          alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc_new));  // exp2(-inf) = 0 at the start
-          m_run = m_new;
-          mc = mc_new;
-        }
-        float rsum = 0.f;
+        // kLazyBits doublings behind (moving on every new maximum rescaled two tiles in three at
+        // S = 8192: any of a wave's 32 queries decides).  And a tile is first tried WITHOUT its
+        // maximum: the exponentials against the reference as it stands, and only if some query's
+        // sum of them is out of a wide range (a score far above the reference, or all of them
+        // so far below it that the sum vanishes) is the maximum taken and the tile redone -- the
+        // arithmetic is floating point throughout, so any reference that neither overflows nor
+        // underflows gives the same quotient.  Edge tiles and queries that have no reference yet
+        // take the maximum at once.
+        bool careful = edge || __builtin_amdgcn_ballot_w64(m_run == -INFINITY) != 0;
+        bool moves = false;
+        float alpha = 1.f, rsum;
         bf16x8 pf[2][2];
+        for (;;) {
+          if (careful) {
+            float rmax = sacc[0][0];
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            float p[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              p[j] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * h + j], scale_log2, -mc));
-              rsum += p[j];
+              for (int e = 0; e < 16; ++e) rmax = fmaxf(rmax, sacc[t][e]);
+            rmax = max_with_other_half(rmax);
+            moves = __builtin_amdgcn_ballot_w64((rmax - m_run) * scale_log2 > kLazyBits) != 0;   // -inf - -inf: no
+            if (moves) {
+              const float m_new = fmaxf(m_run, rmax);
+              const float mc_new = (m_new == -INFINITY) ? 0.f : m_new * scale_log2;
+              alpha = __builtin_amdgcn_exp2f(fmaf(m_run, scale_log2, -mc_new));  // exp2(-inf) = 0 at the start
+              m_run = m_new;
+              mc = mc_new;
             }
-            pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
           }
+          rsum = 0.f;
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              float p[8];
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                p[j] = __builtin_amdgcn_exp2f(fmaf(sacc[t][8 * h + j], scale_log2, -mc));
+                rsum += p[j];
+              }
+              pf[t][h] = __builtin_bit_cast(bf16x8, pack8(p));
+            }
+          if (careful) break;
+          if (__builtin_amdgcn_ballot_w64(!(rsum >= kSumLow && rsum <= kSumHigh)) == 0) break;
+          careful = true;
+        }
         l_run = l_run * alpha + rsum;
         if (moves) {   // the output sums follow the reference (here, where the scores' registers are free again)
 #pragma unroll

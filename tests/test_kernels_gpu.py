@@ -750,6 +750,38 @@ def test_mha_prefill_llama_shape(cuda, S):
     close(got, want)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("shape", ["huge_range", "rising", "falling", "constant", "far_below_zero", "far_above_zero"])
+def test_mha_prefill_scores_that_move_the_softmax_reference(cuda, d, shape):
+    """The exponentials are taken against a reference that follows the maxima lazily, and a tile is
+    first tried without taking its maximum at all: scores spread over hundreds of doublings, scores
+    that rise or fall along the keys by far more than float32's exponent range holds, equal scores,
+    and scores all far below or far above zero (where a reference of zero would under- or overflow)
+    against the oracle's softmax, causal and not, over many tiles."""
+    rng = np.random.default_rng(len(shape) + d)
+    H, G, S = 4, 2, 1100
+    Q, Kc, Vc = bf(rng, S, H, d), bf(rng, S, G, d), bf(rng, S, G, d)
+    ramp = np.linspace(0.0, 1.0, S, dtype=np.float32)[:, None, None]
+    scale = None
+    if shape == "huge_range":
+        Q, Kc = round_bf16(Q * 6), round_bf16(Kc * 6)            # scaled scores of a few hundred either way
+    elif shape in ("rising", "falling"):
+        # one direction of the head carries a score that climbs (or drops) by ~1500 along the keys
+        Q[..., 0] = 8.0
+        Kc[..., 0] = round_bf16((ramp if shape == "rising" else 1 - ramp) * 190.0)[..., 0]
+        scale = 1.0
+    elif shape == "constant":
+        Q[:], Kc[:] = 0.0, 0.0
+    else:
+        Q[..., 0] = 16.0
+        Kc[..., 0] = -40.0 if shape == "far_below_zero" else 40.0   # every score near -640 / +640 before the scale
+        scale = 1.0
+    for causal in (True, False):
+        got, want = run_prefill(cuda, Q, Kc, Vc, H=H, G=G, d=d, seq=S, seq_len=S, kv_len=S, causal=causal, scale=scale)
+        assert not np.isnan(got).any()
+        close(got, want)
+
+
 @pytest.mark.parametrize("interleaved", [False, True])
 @pytest.mark.parametrize("causal,window", [(True, None), (True, 100), (False, 70), (False, None)])
 def test_mha_prefill_masks_and_layouts(cuda, causal, window, interleaved):
