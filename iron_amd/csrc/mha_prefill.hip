@@ -9,7 +9,9 @@
 // the online softmax are in-lane reductions plus one exchange with lane^32, and
 // the probabilities are already laid out as the B operand of O^T = V^T P^T.  V^T
 // fragments come from the transposing LDS read.  All softmax state is f32 in the
-// exp2 domain.
+// exp2 domain; the reference the exponents are taken against follows the maxima
+// lazily, and a tile whose sums of exponentials stay in range never takes its
+// maximum (tile_step below).
 #include "../../include/iron_hip.h"
 #include "common.h"
 
