@@ -1390,6 +1390,21 @@ def test_sample_special_values_and_row_bounds(cuda):
         K.sample(dev(logits, cuda), dr, tok, k_max=65)
 
 
+def test_sample_leaves_its_workspace_ready_for_the_next_draw(cuda):
+    # The block count in the workspace's first words must be zero when a draw starts; every draw
+    # puts it back, so one zeroed workspace serves any number of draws, of changing lengths.
+    rng = np.random.default_rng(23)
+    logits = round_bf16(rng.normal(0, 3, 128256))
+    rows = _draw_rows(rng, 12)
+    lg, dr = dev(logits, cuda), torch.from_numpy(np.ascontiguousarray(rows)).to(cuda)
+    ws = K.sample_workspace(logits.size, cuda)
+    tok = torch.full((1,), -1, dtype=torch.int32, device=cuda)
+    for i, n in enumerate([128256, 100, 51866, 128256, 4096, 1003] * 2):
+        K.sample(lg, dr, tok, n=n, row=word(4 * i, cuda), workspace=ws)
+        assert int(tok.item()) == _host_draw(logits[:n], rows[i]), (i, n)
+        assert not ws[:2].any(), (i, n)
+
+
 def test_eval_words_advances_a_decode_step(cuda):
     words = torch.tensor([11, 40, 0, 0, 0, 0, 0, 0], dtype=torch.int32, device=cuda)
     # position += 1; kv_valid = position + 1; rope_row = min(position, 5); half = position >> 1;
