@@ -19,7 +19,11 @@ namespace iron {
 constexpr int kMaxSplits = 128;      // what the workspace holds per head
 constexpr int kScanMaxSplits = 128;  // the lane-scan kernels' own limit
 constexpr int kSingleMaxKeys = 2048;  // lane-scan kernels: caches up to this many rows take the one-launch kernel
-constexpr int kShortKeys = 2048;      // one-shape launch: up to this many live keys one block a query head writes O itself
+// One-shape launch: up to this many live keys one block a query head writes O itself.  Where the two
+// forms cost the same inside that launch shape (32 / 8 heads of 64, an 8192-row cache, us at 1024 /
+// 1280 / 1536 / 2048 live keys: one block a head 8.0 / 8.8 / 9.7 / 12.1, split + merge 9.0 / 9.0 /
+// 9.0 / 9.5).
+constexpr int kShortKeys = 1408;
 constexpr int kComputeUnits = 256;    // MI355X: what the split count is sized for
 
 // 2^x for x <= 0 by the hardware's own instruction: a softmax weight small enough to be a denormal
@@ -640,24 +644,28 @@ __global__ __launch_bounds__(64 * WAVES) void mha_decode_either_kernel(
   }
 }
 
-// The splits' merge, a block of four waves a head: thread (part, d) sums column d over the splits
-// part, part + 4, ... that hold keys, 32 of them at a time, and the four parts are folded through LDS.
-// A thread's first 32 are requested together with the bound, before it is known how many of them hold
-// anything (the workspace is the caller's own memory, whatever it holds): one trip to memory, not two,
-// for up to 128 splits.  Leaves at once where the scan's blocks wrote the output themselves.
-template <int D>
+// The splits' merge, a block of 4 D threads a head: thread (part, pair) sums columns 2 pair and
+// 2 pair + 1 over the splits part, part + 8, ... that hold keys, PER of them at a time, and the eight
+// parts are folded through LDS.  A thread's first PER are requested together with the bound, before
+// it is known how many of them hold anything (the workspace is the caller's own memory, whatever it
+// holds): one trip to memory, not two, for up to 8 PER splits (PER = 8 where the launch has at most
+// 64 splits, so that no thread asks twice for a split).  Every load is 8 bytes -- a split's maximum
+// and sum, or two columns: the launch's time is its load instructions (one column and one word a
+// load took 1.3 us longer at 64 splits).  Leaves at once where the scan's blocks wrote the output
+// themselves.
+template <int D, int PER>
 __global__ __launch_bounds__(4 * D) void mha_decode_either_merge_kernel(
     const float* __restrict__ part, bf16_t* __restrict__ O, int nsplit, int share_log2, int kv_len, int window,
     const int* __restrict__ kv_valid, int short_keys) {
-  const int head = blockIdx.x, t = threadIdx.x % D, quarter = threadIdx.x / D;
+  constexpr int PAIRS = D / 2;
+  const int head = blockIdx.x, t = threadIdx.x % PAIRS, eighth = threadIdx.x / PAIRS;
   const float* p = part + (size_t)head * nsplit * (D + 2);
-  float m[32], l[32], a[32];
+  float2 ml[PER], a[PER];
 #pragma unroll
-  for (int i = 0; i < 32; ++i) {
-    const int s = min(quarter + 4 * i, nsplit - 1);
-    m[i] = p[s * (D + 2)];
-    l[i] = p[s * (D + 2) + 1];
-    a[i] = p[s * (D + 2) + 2 + t];
+  for (int i = 0; i < PER; ++i) {
+    const int s = min(eighth + 8 * i, nsplit - 1);
+    ml[i] = *reinterpret_cast<const float2*>(p + s * (D + 2));
+    a[i] = *reinterpret_cast<const float2*>(p + s * (D + 2) + 2 + 2 * t);
   }
   const int kv_tokens = bound_or(kv_valid, kv_len);
   const int first = (window >= 0) ? max(0, kv_tokens - 1 - window) : 0;
@@ -665,48 +673,54 @@ __global__ __launch_bounds__(4 * D) void mha_decode_either_merge_kernel(
   if (live <= short_keys) return;
   const int chunk = decode_chunk(live, nsplit, share_log2);
   const int used = (live + chunk - 1) / chunk;
-  float mx = -INFINITY, lt = 0.f, at = 0.f;
-  for (int s0 = quarter; s0 < used; s0 += 128) {
-    if (s0 >= 128) {
+  float mx = -INFINITY, lt = 0.f, at0 = 0.f, at1 = 0.f;
+  for (int s0 = eighth; s0 < used; s0 += 8 * PER) {
+    if (s0 >= 8 * PER) {
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
-        const int s = min(s0 + 4 * i, used - 1);
-        m[i] = p[s * (D + 2)];
-        l[i] = p[s * (D + 2) + 1];
-        a[i] = p[s * (D + 2) + 2 + t];
+      for (int i = 0; i < PER; ++i) {
+        const int s = min(s0 + 8 * i, used - 1);
+        ml[i] = *reinterpret_cast<const float2*>(p + s * (D + 2));
+        a[i] = *reinterpret_cast<const float2*>(p + s * (D + 2) + 2 + 2 * t);
       }
     }
     float cm = mx;
 #pragma unroll
-    for (int i = 0; i < 32; ++i)
-      if (s0 + 4 * i < used) cm = fmaxf(cm, m[i]);
+    for (int i = 0; i < PER; ++i)
+      if (s0 + 8 * i < used) cm = fmaxf(cm, ml[i].x);
     const float keep = (mx == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mx - cm);
     lt *= keep;
-    at *= keep;
+    at0 *= keep;
+    at1 *= keep;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      const bool in = s0 + 4 * i < used && m[i] != -INFINITY;
-      const float e = in ? __builtin_amdgcn_exp2f(m[i] - cm) : 0.f;
-      lt = fmaf(in ? l[i] : 0.f, e, lt);
-      at = fmaf(in ? a[i] : 0.f, e, at);
+    for (int i = 0; i < PER; ++i) {
+      const bool in = s0 + 8 * i < used && ml[i].x != -INFINITY;
+      const float e = in ? __builtin_amdgcn_exp2f(ml[i].x - cm) : 0.f;
+      lt = fmaf(in ? ml[i].y : 0.f, e, lt);
+      at0 = fmaf(in ? a[i].x : 0.f, e, at0);
+      at1 = fmaf(in ? a[i].y : 0.f, e, at1);
     }
     mx = cm;
   }
-  __shared__ float fm[4][D], fl[4][D], fa[4][D];
-  fm[quarter][t] = mx;
-  fl[quarter][t] = lt;
-  fa[quarter][t] = at;
+  __shared__ float fm[8][PAIRS], fl[8][PAIRS];
+  __shared__ float2 fa[8][PAIRS];
+  fm[eighth][t] = mx;
+  fl[eighth][t] = lt;
+  fa[eighth][t] = make_float2(at0, at1);
   __syncthreads();
-  if (quarter != 0) return;
-  float top = fmaxf(fmaxf(fm[0][t], fm[1][t]), fmaxf(fm[2][t], fm[3][t]));
-  float ls = 0.f, as = 0.f;
+  if (eighth != 0) return;
+  float top = fm[0][t];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 1; k < 8; ++k) top = fmaxf(top, fm[k][t]);
+  float ls = 0.f, as0 = 0.f, as1 = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
     const float e = (fm[k][t] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fm[k][t] - top);
     ls = fmaf(fl[k][t], e, ls);
-    as = fmaf(fa[k][t], e, as);
+    as0 = fmaf(fa[k][t].x, e, as0);
+    as1 = fmaf(fa[k][t].y, e, as1);
   }
-  O[(size_t)head * D + t] = f32_to_bf16(ls > 0.f ? as / ls : 0.f);
+  const unsigned lo = f32_to_bf16(ls > 0.f ? as0 / ls : 0.f), hi = f32_to_bf16(ls > 0.f ? as1 / ls : 0.f);
+  reinterpret_cast<unsigned*>(O + (size_t)head * D)[t] = lo | (hi << 16);
 }
 
 template <int D, int G>
@@ -752,8 +766,12 @@ static int launch_decode_either(const bf16_t* Q, const bf16_t* K, const bf16_t* 
   hipLaunchKernelGGL((mha_decode_either_kernel<D, WAVES>), dim3(sets, nsplit), dim3(64 * WAVES), lds, s, Q, K, V, O,
                      part, kv_heads, group, hpb_log2, kv_len, scale_log2, window, row_stride, head_stride, kv_valid,
                      kv_first, kv_rows, short_keys);
-  hipLaunchKernelGGL((mha_decode_either_merge_kernel<D>), dim3(kv_heads * group), dim3(4 * D), 0, s, part, O, nsplit,
-                     (WAVES == 16 ? 4 : 3) - hpb_log2, kv_len, window, kv_valid, short_keys);
+  if (nsplit <= 64)
+    hipLaunchKernelGGL((mha_decode_either_merge_kernel<D, 8>), dim3(kv_heads * group), dim3(4 * D), 0, s, part, O,
+                       nsplit, (WAVES == 16 ? 4 : 3) - hpb_log2, kv_len, window, kv_valid, short_keys);
+  else
+    hipLaunchKernelGGL((mha_decode_either_merge_kernel<D, 16>), dim3(kv_heads * group), dim3(4 * D), 0, s, part, O,
+                       nsplit, (WAVES == 16 ? 4 : 3) - hpb_log2, kv_len, window, kv_valid, short_keys);
   return 0;
 }
 
@@ -778,7 +796,7 @@ static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, u
                "mha_decode: heads (%d) must be a positive multiple of kv_heads (%d)", heads, kv_heads);
   IRON_REQUIRE(kv_len > 0, "mha_decode: kv_len (%d) must be positive", kv_len);
   IRON_REQUIRE(scale >= 0.f && scale < INFINITY, "mha_decode: scale must be finite and not negative");
-  IRON_REQUIRE((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)workspace) & 15) == 0,
+  IRON_REQUIRE((((uintptr_t)Q | (uintptr_t)K | (uintptr_t)V | (uintptr_t)O | (uintptr_t)workspace) & 15) == 0,
                "mha_decode: operands must be 16-byte aligned");
   const int G = heads / kv_heads;
   const long row_stride = kv_interleaved ? (long)kv_heads * d : d;
@@ -801,7 +819,7 @@ static int mha_decode(const uint16_t* Q, const uint16_t* K, const uint16_t* V, u
   IRON_REQUIRE(form != 2 || either_fits,
                "mha_decode: the one-shape launch takes d = 64 or 128, up to 16 query heads a KV head and keys within 2^31 bytes");
   const int upto = short_keys > 0 ? short_keys : kShortKeys;
-  if (form == 2 || (form == 0 && either_fits && kv_len > upto)) {
+  if (form == 2 || (form == 0 && either_fits && kv_len > (short_keys > 0 ? short_keys : kSingleMaxKeys))) {
     const int rc = d == 64 ? launch_decode_either<64, 16>(Q, K, V, O, part, kv_heads, G, kv_len, scale_log2, window, row_stride,
                                                           head_stride, kv_valid, kv_first, kv_rows, upto, s)
                            : launch_decode_either<128, 8>(Q, K, V, O, part, kv_heads, G, kv_len, scale_log2, window, row_stride,
