@@ -588,59 +588,55 @@ __global__ __launch_bounds__(64 * WAVES) void mha_decode_either_kernel(
   l_run += __shfl_xor(l_run, 32, 64);
 
   // Waves hand (max, sum, O^T column) per head over through LDS (the stage buffers, once every wave
-  // is out of its loop); thread (head, d) folds the waves of its KV head, every read issued before
-  // the first is used.
+  // is out of its loop); thread (head, pair of d) folds the waves of its KV head, every read issued
+  // before the first is used.  Eight bytes a write and a read: at a step or two a wave the launch is
+  // as long as its instructions, these among them.
   __syncthreads();
   float* hand = reinterpret_cast<float*>(smem_dec);   // [WAVES][group][D + 2]
   static_assert(16 * (D + 2) * 4 <= 2 * TILE, "a wave's hand-over fits its own stage buffers");
   if (n < group) {
     float* mine = hand + ((size_t)wave * group + n) * (D + 2);
-    if (q == 0) {
-      mine[0] = m_ref;
-      mine[1] = l_run;
+    if (q == 0) *reinterpret_cast<float2*>(mine) = make_float2(m_ref, l_run);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      *reinterpret_cast<float2*>(mine + 2 + 16 * dt + 4 * q) = make_float2(oacc[dt][0], oacc[dt][1]);
+      *reinterpret_cast<float2*>(mine + 4 + 16 * dt + 4 * q) = make_float2(oacc[dt][2], oacc[dt][3]);
     }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mine[2 + 16 * dt + 4 * q + i] = oacc[dt][i];
   }
   __syncthreads();
   // Column hg = (head of the block's, query head of its group) lies in waves hw, hw + hpb, ...: entry
   // hg + j hpb group of the hand-over for j < share.
   const int share = 1 << share_log2;
   const int wave_step = (group << hpb_log2) * (D + 2);
-  for (int idx = tid; idx < (group << hpb_log2) * D; idx += 64 * WAVES) {
-    const int hg = idx / D, dd = idx % D;
+  for (int idx = tid; idx < (group << hpb_log2) * (D / 2); idx += 64 * WAVES) {
+    const int hg = idx / (D / 2), pair = idx % (D / 2);
     const float* col = hand + (size_t)hg * (D + 2);
-    float mv[WAVES], lv[WAVES], av[WAVES];
+    float2 mlv[WAVES], av[WAVES];
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      mv[w] = -INFINITY;
-      lv[w] = av[w] = 0.f;
+      mlv[w] = make_float2(-INFINITY, 0.f);
+      av[w] = make_float2(0.f, 0.f);
       if (w < share) {   // uniform over the block
-        mv[w] = col[w * wave_step];
-        lv[w] = col[w * wave_step + 1];
-        av[w] = col[w * wave_step + 2 + dd];
+        mlv[w] = *reinterpret_cast<const float2*>(col + w * wave_step);
+        av[w] = *reinterpret_cast<const float2*>(col + w * wave_step + 2 + 2 * pair);
       }
     }
     float mx = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, mv[w]);
-    float lt = 0.f, at = 0.f;
+    for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, mlv[w].x);
+    float lt = 0.f, at0 = 0.f, at1 = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float e = (mv[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mv[w] - mx) * scale_log2);
-      lt = fmaf(lv[w], e, lt);
-      at = fmaf(av[w], e, at);
+      const float e = (mlv[w].x == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((mlv[w].x - mx) * scale_log2);
+      lt = fmaf(mlv[w].y, e, lt);
+      at0 = fmaf(av[w].x, e, at0);
+      at1 = fmaf(av[w].y, e, at1);
     }
     // part layout: [head][split][D + 2] = {max in the exp2 domain, sum, O[D]}.
     const int head = (blockIdx.x << hpb_log2) * group + hg;
     float* out = part + ((size_t)head * nsplit + split) * (D + 2);
-    out[2 + dd] = at;
-    if (dd == 0) {
-      out[0] = (mx == -INFINITY) ? -INFINITY : mx * scale_log2;
-      out[1] = lt;
-    }
+    *reinterpret_cast<float2*>(out + 2 + 2 * pair) = make_float2(at0, at1);
+    if (pair == 0) *reinterpret_cast<float2*>(out) = make_float2((mx == -INFINITY) ? -INFINITY : mx * scale_log2, lt);
   }
 }
 
