@@ -30,6 +30,16 @@ constexpr int kComputeUnits = 256;    // MI355X: what the split count is sized f
 // counts as 0, which saves the library routine's rescaling around every call.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// f(x of this lane, x of lane ^ SPAN) for SPAN = 16 or 32: the swap leaves one of the two in each
+// operand (which is which depends on the lane's side; f is symmetric).
+template <int SPAN, typename F>
+__device__ __forceinline__ float across_rows(float x, F f) {
+  float a = x, b = x;
+  if (SPAN == 16) asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  else asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return f(a, b);
+}
+
 typedef __bf16 bf16x2_v __attribute__((ext_vector_type(2)));
 // The dot product of two 16-byte runs of bf16.
 __device__ __forceinline__ float dot8(const uint4& a, const uint4& b) {
@@ -130,24 +140,33 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
     }
   }
 
-  // Merge the RW lane groups of the wave (lanes that share `sub`).
+  // Merge the RW lane groups of the wave (lanes that share `sub`): the maximum over them first, one
+  // rescaling of a group's sums to it, then plain sums -- lane ^ 8 by a DPP rotation inside the row,
+  // lane ^ 16 and lane ^ 32 by the row and half swaps, no trip through LDS (as three rounds of
+  // shuffled (max, sum, columns) with two exponentials each, this tail was a tenth of the launch at
+  // a few hundred keys).
 #pragma unroll
   for (int g = 0; g < G; ++g) {
+    float mw = m[g];
+    if (LPR <= 8) mw = fmaxf(mw, IRON_DPP(0.f, mw, 0x128, 0xF));   // row_ror:8
+    if (LPR <= 16) mw = across_rows<16>(mw, [](float a, float b) { return fmaxf(a, b); });
+    if (LPR <= 32) mw = across_rows<32>(mw, [](float a, float b) { return fmaxf(a, b); });
+    const float ref = (mw == -INFINITY) ? 0.f : mw;
+    const float a = fast_exp2(m[g] - ref);   // 0 for a group that saw no key
+    float v[9];
+    v[8] = l[g] * a;
 #pragma unroll
-    for (int o = LPR; o < 64; o <<= 1) {
-      const float mo = __shfl_xor(m[g], o, 64);
-      const float lo2 = __shfl_xor(l[g], o, 64);
-      const float mx = fmaxf(m[g], mo);
-      const float ref = (mx == -INFINITY) ? 0.f : mx;
-      const float a = exp2f(m[g] - ref), b = exp2f(mo - ref);
-      l[g] = l[g] * a + lo2 * b;
+    for (int i = 0; i < 8; ++i) v[i] = acc[g][i] * a;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float ao = __shfl_xor(acc[g][i], o, 64);
-        acc[g][i] = acc[g][i] * a + ao * b;
-      }
-      m[g] = mx;
+    for (int i = 0; i < 9; ++i) {
+      if (LPR <= 8) v[i] += IRON_DPP(0.f, v[i], 0x128, 0xF);
+      if (LPR <= 16) v[i] = across_rows<16>(v[i], [](float a, float b) { return a + b; });
+      if (LPR <= 32) v[i] = across_rows<32>(v[i], [](float a, float b) { return a + b; });
     }
+    l[g] = v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = v[i];
+    m[g] = mw;
   }
 }
 
