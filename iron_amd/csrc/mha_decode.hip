@@ -226,7 +226,7 @@ __global__ __launch_bounds__(256) void mha_decode_kernel(
     float lt = 0.f, at = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float e = exp2f(sm[w][g] - ref);
+      const float e = fast_exp2(sm[w][g] - ref);
       lt += sl[w][g] * e;
       at += sacc[w][g][dd] * e;
     }
@@ -259,7 +259,7 @@ __global__ void mha_decode_merge_kernel(const float* __restrict__ part, bf16_t* 
   mx = -INFINITY;
   for (int w = 0; w < (int)(blockDim.x >> 6); ++w) mx = fmaxf(mx, red[0][w]);
   const float ref = (mx == -INFINITY) ? 0.f : mx;
-  const float e = exp2f(m - ref);  // 0 for the lanes past nsplit (m = -inf)
+  const float e = fast_exp2(m - ref);  // 0 for the lanes past nsplit (m = -inf)
   if (t < nsplit) wgt[t] = e;
   float ls = wave_sum(l * e);
   if (lane == 0) red[1][wave] = ls;
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(1024) void mha_decode_single_kernel(
     float lt = 0.f, at = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float e = exp2f(sm[w] - ref);
+      const float e = fast_exp2(sm[w] - ref);
       lt += sl[w] * e;
       at += sacc[w][dd] * e;
     }
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(64 * WAVES) void mha_decode_either_kernel(
       float lt = 0.f, at = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) {
-        const float e = exp2f(sm[w] - ref);
+        const float e = fast_exp2(sm[w] - ref);
         lt += sl[w] * e;
         at += sacc[w * D + tid] * e;
       }
