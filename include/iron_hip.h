@@ -271,8 +271,9 @@ int iron_mha_prefill_at_bf16(const uint16_t* Q, const uint16_t* K, const uint16_
 /* Attention, one query (decode; the reference's "packed" MHA, seq_len == 1).
  * Q,O: (heads, d).  K,V as above.  kv_tokens = *kv_valid (or kv_len); the query sits at
  * kv_tokens - 1.  workspace: iron_mha_decode_workspace_bytes(heads, d) bytes of device memory.
+ * Q, K, V, O and workspace 16-byte aligned.
  * d in {64, 128} with up to 16 query heads a KV head, d = 256 with 1, 2, 3, 4, 5, 6 or 8, or d = 512
- * with any.  The launches depend on (heads, kv_heads, d) and on whether kv_len can pass 1024 rows;
+ * with any.  The launches depend on (heads, kv_heads, d) and on whether kv_len can pass 2048 rows;
  * what they read, and how the keys are dealt over the chip, follow *kv_valid (a cache's length only
  * sizes the buffers: the reference's "attention over a cache costs the context, not the cache",
  * iron/operators/mha.py:275-278).
