@@ -163,7 +163,7 @@ def bench_decode_kernels(torch, K, dev, n, rng):
     qkv_bytes = 2 * ((H + 2 * G) * D * E + 2 * E + (H + 2 * G) * D)
     caches = pool(2 * L * G * D * 2, lambda: (drawn(L, G, D, scale=1.0), drawn(L, G, D, scale=1.0)))
     ws = pool(qkv_bytes, lambda: (drawn(H * D, E), drawn(G * D, E), drawn(G * D, E)))
-    add("norm + q/k/v + RoPE + cache write", "decode_qkv_kernel<64,1,false>", 16, qkv_bytes,
+    add("norm + q/k/v + RoPE + cache write", "decode_qkv_kernel<64,1,false,2>", 16, qkv_bytes,
         [(lambda w=w, c=caches[i % len(caches)]: K.decode_qkv(x, gain, w[0], w[1], w[2], angles, q, c[0], c[1], eps=1e-5,
                                                                hidden=E, heads=H, kv_heads=G, d=D, cache_rows=L,
                                                                position=position)) for i, w in enumerate(ws)])
@@ -654,7 +654,7 @@ DOMINANT_TRAFFIC_BYTES: dict[str, int] = {
     "gemv_fused_kernel<2,1,true,2>": 67_353_000,     # norm + gate/up + SiLU*mul: 67.222 MB fetched + 0.131 written
     "gemv_fused_kernel<2,4,false,1>": 33_783_000,    # down projection + residual: 33.750 + 0.033
     "gemv_fused_kernel<4,1,true,0>": 526_446_000,    # final norm + LM head: 525.42 + 1.03
-    "decode_qkv_kernel<64,1,false>": 12_749_000,     # norm + q/k/v + RoPE + cache rows: 12.70 + 0.05
+    "decode_qkv_kernel<64,1,false,2>": 12_753_000,   # norm + q/k/v + RoPE + cache rows: 12.708 + 0.045
     "gemv_fused_kernel<1,1,false,1>": 8_513_000,     # o projection + residual: 8.48 + 0.03
 }
 

@@ -156,10 +156,12 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
   }
 }
 
-// Attention's first half for one token.  A block takes a PAIR of projection rows: for q and k
-// the rows (h, j) and (h, j + D/2) that RoPE rotates together, for v two adjacent rows.
+// Attention's first half for one token.  A block takes PAIRS pairs of projection rows: for q and k
+// a pair is the rows (h, j) and (h, j + D/2) that RoPE rotates together, for v two adjacent rows
+// (with PAIRS = 2 the block's activation and gain loads, and its norm, serve four rows -- what the
+// gate/up launch's blocks have; the pairs of a block are of one kind, which even pair counts ensure).
 // TABLE: x is to be read from row *x_row of x_table (and left in x by the first block).
-template <int D, int CH, bool TABLE>
+template <int D, int CH, bool TABLE, int PAIRS>
 __global__ __launch_bounds__(256) void decode_qkv_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ nw, float eps,
     const bf16_t* __restrict__ Wq, const bf16_t* __restrict__ Wk, const bf16_t* __restrict__ Wv,
@@ -169,33 +171,41 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
     const bf16_t* __restrict__ x_table, const int* __restrict__ x_row, int x_rows) {
   constexpr int HALF = D / 2;
   __shared__ float scratch4[4];
-  __shared__ float part[4][2];
+  __shared__ float part[4][PAIRS][2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int pair = blockIdx.x;
+  const int pair0 = blockIdx.x * PAIRS;
   const int q_pairs = heads * HALF, k_pairs = kv_heads * HALF;
 
+  // The block's kind (0 q, 1 k, 2 v) and its first pair's rows; pair p's follow at + p (+ 2 p for v).
   const bf16_t* Wm;
-  int r0, r1, j = 0, kind;  // kind 0 q, 1 k, 2 v
-  if (pair < q_pairs) { kind = 0; Wm = Wq; const int h = pair / HALF; j = pair % HALF; r0 = h * D + j; r1 = r0 + HALF; }
-  else if (pair < q_pairs + k_pairs) { kind = 1; Wm = Wk; const int p = pair - q_pairs; const int h = p / HALF; j = p % HALF; r0 = h * D + j; r1 = r0 + HALF; }
-  else { kind = 2; Wm = Wv; const int p = pair - q_pairs - k_pairs; r0 = 2 * p; r1 = r0 + 1; }
+  int r0, step, j = 0, kind;
+  if (pair0 < q_pairs) { kind = 0; Wm = Wq; const int h = pair0 / HALF; j = pair0 % HALF; r0 = h * D + j; step = HALF; }
+  else if (pair0 < q_pairs + k_pairs) { kind = 1; Wm = Wk; const int p = pair0 - q_pairs; const int h = p / HALF; j = p % HALF; r0 = h * D + j; step = HALF; }
+  else { kind = 2; Wm = Wv; const int p = pair0 - q_pairs - k_pairs; r0 = 2 * p; step = 1; }
+  const int next = kind == 2 ? 2 : 1;   // from a pair's first row to the next pair's
 
   Activation<CH, true> act;
-  uint4 w0[CH], w1[CH];
+  uint4 w0[PAIRS][CH], w1[PAIRS][CH];
   if (!TABLE) {
     act.issue(x, nw, K);
-    load_row<CH>(Wm + (size_t)r0 * K, K, w0);
-    load_row<CH>(Wm + (size_t)r1 * K, K, w1);
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+      load_row<CH>(Wm + (size_t)(r0 + p * next) * K, K, w0[p]);
+      load_row<CH>(Wm + (size_t)(r0 + p * next + step) * K, K, w1[p]);
+    }
   } else {
     // The token's row of an embedding table, named by a device word (held inside the table): the row
     // is read where it lies and the first block leaves the copy the layer's residual sum will read,
     // so the step's gather needs no launch of its own.  Everything that does not wait for the word
     // goes out ahead of it.
     act.issue_gains(nw, K);
-    load_row<CH>(Wm + (size_t)r0 * K, K, w0);
-    load_row<CH>(Wm + (size_t)r1 * K, K, w1);
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+      load_row<CH>(Wm + (size_t)(r0 + p * next) * K, K, w0[p]);
+      load_row<CH>(Wm + (size_t)(r0 + p * next + step) * K, K, w1[p]);
+    }
     act.issue_row(x_table + (size_t)max(0, min(*x_row, x_rows - 1)) * K, K);
-    if (pair == 0) {
+    if (blockIdx.x == 0) {
 #pragma unroll
       for (int i = 0; i < CH; ++i) {
         const int c = threadIdx.x + 256 * i;
@@ -204,7 +214,7 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
     }
   }
   // `angles` is the step's row itself, or a whole table whose row a device word names (held inside).
-  // What the block's last thread needs after the last barrier -- the pair's angle and the position
+  // What the block's last threads need after the last barrier -- their pair's angle and the position
   // word -- is asked for here, behind the rows' loads (the word that names the angles' row is a trip
   // to memory of its own, which nothing above waits for) and under their trip to memory.
   // (The two words pinned here, among the loads in flight: left free, the compiler moves the position's
@@ -212,29 +222,34 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   int pos_ahead = *position, angle_at = angle_row != nullptr ? *angle_row : 0;
   asm volatile("" : "+s"(pos_ahead), "+s"(angle_at));
   angles += (size_t)max(0, min(angle_at, angle_rows - 1)) * D;
-  const float c_ahead = bf16_to_f32(angles[2 * j]), s_ahead = bf16_to_f32(angles[2 * j + 1]);
+  const int mine = min((int)threadIdx.x, PAIRS - 1);   // the pair this thread finishes, if it finishes one
+  const float c_ahead = bf16_to_f32(angles[2 * (j + mine)]), s_ahead = bf16_to_f32(angles[2 * (j + mine) + 1]);
   float xf[CH][8];
   act.finish(eps, K, scratch4, xf);
-  const float a0 = wave_sum(dot_row<CH>(w0, xf)), a1 = wave_sum(dot_row<CH>(w1, xf));
-  if (lane == 0) { part[wave][0] = a0; part[wave][1] = a1; }
+#pragma unroll
+  for (int p = 0; p < PAIRS; ++p) {
+    const float a0 = wave_sum(dot_row<CH>(w0[p], xf)), a1 = wave_sum(dot_row<CH>(w1[p], xf));
+    if (lane == 0) { part[wave][p][0] = a0; part[wave][p][1] = a1; }
+  }
   __syncthreads();
-  if (threadIdx.x != 0) return;
-  float y0 = round_bf16(part[0][0] + part[1][0] + part[2][0] + part[3][0]);  // the projections' own rounding
-  float y1 = round_bf16(part[0][1] + part[1][1] + part[2][1] + part[3][1]);
+  if (threadIdx.x >= PAIRS) return;
+  const int p = threadIdx.x, ra = r0 + p * next, rb = ra + step;
+  float y0 = round_bf16(part[0][p][0] + part[1][p][0] + part[2][p][0] + part[3][p][0]);  // the projections' own rounding
+  float y1 = round_bf16(part[0][p][1] + part[1][p][1] + part[2][p][1] + part[3][p][1]);
   if (kind != 2) {
     const float c = c_ahead, s = s_ahead;
     const float t0 = y0 * c - y1 * s, t1 = y1 * c + y0 * s;
     y0 = t0; y1 = t1;
   }
   if (kind == 0) {
-    q_out[r0] = f32_to_bf16(y0);
-    q_out[r1] = f32_to_bf16(y1);
+    q_out[ra] = f32_to_bf16(y0);
+    q_out[rb] = f32_to_bf16(y1);
   } else {
     const int pos = pos_ahead;
     if (pos >= 0 && pos < cache_rows) {
       bf16_t* dst = (kind == 1 ? keys : values) + (size_t)pos * kv_heads * D;
-      dst[r0] = f32_to_bf16(y0);
-      dst[r1] = f32_to_bf16(y1);
+      dst[ra] = f32_to_bf16(y0);
+      dst[rb] = f32_to_bf16(y1);
     }
   }
 }
@@ -437,19 +452,23 @@ static int decode_qkv(const uint16_t* x, const uint16_t* norm_w, float eps, cons
   IRON_REQUIRE(x_row == nullptr || (x_table != nullptr && x_rows > 0), "decode_qkv: a row of a table of %d rows", x_rows);
   const int pairs = heads * (d / 2) + 2 * kv_heads * (d / 2);
   const int ch = hidden <= 2048 ? 1 : (hidden <= 4096 ? 2 : 4);
+  // Two pairs a block where a row is at most 4 KB (its chunks one a thread) and no block would span
+  // two kinds of rows or a pair's two halves (q's and k's pair counts a multiple of D/2: even).
+  const int per = ch == 1 ? 2 : 1;
   hipStream_t s = (hipStream_t)stream;
-#define IRON_QKV(DD, C)                                                                             \
-  if (d == DD && ch == C) {                                                                         \
+#define IRON_QKV(DD, C, P)                                                                          \
+  if (d == DD && ch == C && per == P) {                                                             \
     if (x_row == nullptr)                                                                           \
-      hipLaunchKernelGGL((decode_qkv_kernel<DD, C, false>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
+      hipLaunchKernelGGL((decode_qkv_kernel<DD, C, false, P>), dim3(pairs / P), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv, \
                          angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row,        \
                          angle_rows, x_table, x_row, x_rows);                                                          \
     else                                                                                            \
-      hipLaunchKernelGGL((decode_qkv_kernel<DD, C, true>), dim3(pairs), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv,  \
+      hipLaunchKernelGGL((decode_qkv_kernel<DD, C, true, P>), dim3(pairs / P), dim3(256), 0, s, x, norm_w, eps, Wq, Wk, Wv,  \
                          angles, q_out, keys, values, hidden, heads, kv_heads, cache_rows, position, angle_row,        \
                          angle_rows, x_table, x_row, x_rows);                                                          \
   }
-  IRON_QKV(64, 1) IRON_QKV(64, 2) IRON_QKV(64, 4) IRON_QKV(128, 1) IRON_QKV(128, 2) IRON_QKV(128, 4)
+  IRON_QKV(64, 1, 1) IRON_QKV(64, 2, 1) IRON_QKV(64, 4, 1) IRON_QKV(128, 1, 1) IRON_QKV(128, 2, 1) IRON_QKV(128, 4, 1)
+  IRON_QKV(64, 1, 2) IRON_QKV(128, 1, 2)
 #undef IRON_QKV
   IRON_LAUNCH_CHECK();
 }
