@@ -50,26 +50,30 @@ struct Activation {
 #pragma unroll
     for (int i = 0; i < CH; ++i) xv[i] = load_bounded(run, 16 * ((int)threadIdx.x + 256 * i));
   }
-  // With NORM the block sums the squares together (one barrier).
-  __device__ __forceinline__ void finish(float eps, int K, float* scratch4, float (&xf)[CH][8]) {
+  // With NORM the block sums the squares together (one barrier).  The activation comes out as it
+  // went in, packed bf16 (what the norm rounds to): the dot products below take it in pairs.
+  __device__ __forceinline__ void finish(float eps, int K, float* scratch4, uint4 (&xp)[CH]) {
+    if (!NORM) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) xp[i] = xv[i];
+      return;
+    }
+    float xf[CH][8];
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       unpack8(xv[i], xf[i]);
-      if (NORM) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ss = fmaf(xf[i][j], xf[i][j], ss);
-      }
+      for (int j = 0; j < 8; ++j) ss = fmaf(xf[i][j], xf[i][j], ss);
     }
-    if (NORM) {
-      const float inv = 1.0f / sqrtf(block_sum(ss, scratch4) / (float)K + eps);
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch4) / (float)K + eps);
 #pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        float g[8];
-        unpack8(gv[i], g);
+    for (int i = 0; i < CH; ++i) {
+      float g[8];
+      unpack8(gv[i], g);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) xf[i][j] = round_bf16(round_bf16(xf[i][j] * inv) * g[j]);
-      }
+      for (int j = 0; j < 8; ++j) xf[i][j] = round_bf16(xf[i][j] * inv) * g[j];
+      xp[i] = pack8(xf[i]);   // the product's own rounding
     }
   }
 };
@@ -82,15 +86,20 @@ __device__ __forceinline__ void load_row(const bf16_t* __restrict__ row, int K, 
   for (int i = 0; i < CH; ++i) w[i] = load_bounded_stream(run, 16 * ((int)threadIdx.x + 256 * i));
 }
 
+// A row's chunks times the activation's: two-element dot products of the bf16 pairs as they were
+// loaded (v_dot2c_f32_bf16: exact products, float32 sums) -- a quarter of the instructions of
+// widening both sides and a multiply-add an element, and what a resident block does after its
+// loads have landed is time its CU's share of the memory system idles.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 template <int CH>
-__device__ __forceinline__ float dot_row(const uint4 (&w)[CH], const float (&xf)[CH][8]) {
+__device__ __forceinline__ float dot_row(const uint4 (&w)[CH], const uint4 (&xp)[CH]) {
   float acc = 0.f;
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    float wf[8];
-    unpack8(w[i], wf);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc = fmaf(wf[j], xf[i][j], acc);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[i].x), __builtin_bit_cast(bf16x2_t, xp[i].x), acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[i].y), __builtin_bit_cast(bf16x2_t, xp[i].y), acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[i].z), __builtin_bit_cast(bf16x2_t, xp[i].z), acc, false);
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[i].w), __builtin_bit_cast(bf16x2_t, xp[i].w), acc, false);
   }
   return acc;
 }
@@ -128,7 +137,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(const bf16_t* __restric
     load_row<CH>(W + (size_t)row * K, K, w[0][r]);
     if (MATS == 2) load_row<CH>(W2 + (size_t)row * K, K, w[MATS - 1][r]);
   }
-  float xf[CH][8];
+  uint4 xf[CH];
   act.finish(eps, K, scratch4, xf);
 #pragma unroll
   for (int m = 0; m < MATS; ++m)
@@ -224,7 +233,7 @@ __global__ __launch_bounds__(256) void decode_qkv_kernel(
   angles += (size_t)max(0, min(angle_at, angle_rows - 1)) * D;
   const int mine = min((int)threadIdx.x, PAIRS - 1);   // the pair this thread finishes, if it finishes one
   const float c_ahead = bf16_to_f32(angles[2 * (j + mine)]), s_ahead = bf16_to_f32(angles[2 * (j + mine) + 1]);
-  float xf[CH][8];
+  uint4 xf[CH];
   act.finish(eps, K, scratch4, xf);
 #pragma unroll
   for (int p = 0; p < PAIRS; ++p) {
