@@ -252,7 +252,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A,
             *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
           } else {
             const float v[4] = {v0, v1, v2, v3};
-            for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(v[e]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)   // (constant indices: a runtime trip count puts the array in scratch memory)
+              if (n + e < N) p[e] = f32_to_bf16(v[e]);
           }
         } else {
           const int n = nb + frag_row, m = mb + 8 * q + hi;
@@ -506,7 +508,9 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
         rf[0] = __uint_as_float(rv.x << 16); rf[1] = __uint_as_float(rv.x & 0xffff0000u);
         rf[2] = __uint_as_float(rv.y << 16); rf[3] = __uint_as_float(rv.y & 0xffff0000u);
       } else {
-        for (int e = 0; e < 4 && n + e < N; ++e) rf[e] = bf16_to_f32(r[e]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) rf[e] = bf16_to_f32(r[e]);
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -518,7 +522,9 @@ __device__ __forceinline__ void gemm_nt64_body(const bf16_t* __restrict__ A, con
       *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(acc[0][4 * q], acc[0][4 * q + 1]),
                                                 pack_bf16(acc[0][4 * q + 2], acc[0][4 * q + 3]));
     } else {
-      for (int e = 0; e < 4 && n + e < N; ++e) p[e] = f32_to_bf16(acc[0][4 * q + e]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < N) p[e] = f32_to_bf16(acc[0][4 * q + e]);
     }
   }
 }
@@ -876,7 +882,9 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
         if (whole) {
           unpack8(res_ahead ? res[r] : *reinterpret_cast<const uint4*>(qkv.residual + (size_t)m * N + out_n), rf);
         } else {
-          for (int e = 0; e < 8 && out_n + e < N; ++e) rf[e] = bf16_to_f32(qkv.residual[(size_t)m * N + out_n + e]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e)   // (constant indices: a runtime trip count puts the array in scratch memory)
+            if (out_n + e < N) rf[e] = bf16_to_f32(qkv.residual[(size_t)m * N + out_n + e]);
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -887,8 +895,10 @@ __device__ __forceinline__ void gemm_nt16_body(const bf16_t* __restrict__ A, con
     if (whole) {
       *reinterpret_cast<uint4*>(p) = v;
     } else {
-      const bf16_t* h = reinterpret_cast<const bf16_t*>(&v);
-      for (int e = 0; e < 8 && out_n + e < N; ++e) p[e] = h[e];
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (out_n + e < N) p[e] = (bf16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
     }
   }
 }
@@ -1949,8 +1959,10 @@ __device__ __forceinline__ void gemm_nt16_pair_body(const bf16_t* __restrict__ A
       if (whole) {
         *reinterpret_cast<uint4*>(p) = v;
       } else {
-        const bf16_t* h = reinterpret_cast<const bf16_t*>(&v);
-        for (int e = 0; e < 8 && out_n + e < N; ++e) p[e] = h[e];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (out_n + e < N) p[e] = (bf16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
