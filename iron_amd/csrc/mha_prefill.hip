@@ -363,15 +363,14 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
       // fragment's place in its stage is an immediate of the read and the buffer arithmetic goes
       // (S = 2048: 3.5 % faster).  Where a CU holds several blocks at different places of the loop
       // the three-fold code measured 2.4 % slower (S = 8192), so there the loop stays rolled.
-      int step = 0;
-      for (; step + STAGES <= steps; step += STAGES) {
+      // An odd count of steps is rounded up: the added step is past every half's last tile and, like
+      // the odd half's own last step may be, only keeps the loads and the wait counts going (a tail
+      // of single steps would be two more copies of the body, whose registers spilled).
+      static_assert(STAGES == 2, "the loop below names the buffers");
+      for (int step = 0; step < steps; step += STAGES) {
         tile_step(step, 0);
         tile_step(step + 1, 1);
-        if constexpr (STAGES > 2) tile_step(step + 2, 2);
       }
-      static_assert(STAGES == 2 || STAGES == 3, "the tail below names the buffers");
-      if (step < steps) tile_step(step, 0);
-      if (step + 1 < steps) tile_step(step + 1, 1);
     } else {
       for (int step = 0; step < steps; ++step) tile_step(step, step % STAGES);
     }
