@@ -410,7 +410,11 @@ __global__ __launch_bounds__(64 * W * SPLIT) __attribute__((amdgpu_waves_per_eu(
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = (q_live && l_tot > 0.f) ? 1.0f / l_tot : 0.f;
   if (my_q < seq) {
-    bf16_t* op = Oh + (size_t)my_q * q_row_stride;
+    // (The row's address is made here: computed where its inputs first are, it is 64 bits a lane held
+    // -- at eight waves a block, spilled -- through the whole loop.)
+    int row = my_q;
+    asm volatile("" : "+v"(row));
+    bf16_t* op = Oh + (size_t)row * q_row_stride;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -708,7 +712,9 @@ __global__ __launch_bounds__(64 * W, 2) void mha_prefill_wide_kernel(
     l_tot += __shfl_xor(l_tot, 32, 64);
     const float inv = (q_live[u] && l_tot > 0.f) ? 1.0f / l_tot : 0.f;
     if (my_q[u] < seq) {
-      bf16_t* op = Oh + (size_t)my_q[u] * q_row_stride + 4 * q;
+      int row = my_q[u];   // (the address made here, as in the kernel above)
+      asm volatile("" : "+v"(row));
+      bf16_t* op = Oh + (size_t)row * q_row_stride + 4 * q;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
         *reinterpret_cast<uint2*>(op + 16 * dt) = make_uint2(pack_bf16(oacc[u][dt][0] * inv, oacc[u][dt][1] * inv),
