@@ -80,16 +80,22 @@ __device__ __forceinline__ void decode_scan(const bf16_t* __restrict__ Q, const 
   Vh += sub * 8;
 
   for (int base = lo; base < hi; base += stride) {
+    // Every key row of the pass is asked for before any value row: a CU's address path takes a
+    // block's loads one after another (16 cycles each), and the scores and their exponentials then
+    // run while the value rows are still on their way.
     uint4 kv[U], vv[U];
     bool live[U];
+    size_t off[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int r = base + u * RW + rg;
       live[u] = r < hi;
-      const size_t off = (size_t)(live[u] ? r : (hi - 1)) * row_stride;
-      kv[u] = STREAM ? load_stream(reinterpret_cast<const uint4*>(Kh + off)) : *reinterpret_cast<const uint4*>(Kh + off);
-      vv[u] = STREAM ? load_stream(reinterpret_cast<const uint4*>(Vh + off)) : *reinterpret_cast<const uint4*>(Vh + off);
+      off[u] = (size_t)(live[u] ? r : (hi - 1)) * row_stride;
+      kv[u] = STREAM ? load_stream(reinterpret_cast<const uint4*>(Kh + off[u])) : *reinterpret_cast<const uint4*>(Kh + off[u]);
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      vv[u] = STREAM ? load_stream(reinterpret_cast<const uint4*>(Vh + off[u])) : *reinterpret_cast<const uint4*>(Vh + off[u]);
     float s[U][G];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
