@@ -11,6 +11,8 @@
 
 namespace iron {
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
 template <int RPW, int KSPLIT>
 __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ W,
                                                    const bf16_t* __restrict__ x,
@@ -52,14 +54,15 @@ __global__ __launch_bounds__(256) void gemv_kernel(const bf16_t* __restrict__ W,
       uint4 wv[RPW];
 #pragma unroll
       for (int r = 0; r < RPW; ++r) wv[r] = load_stream(wrow[r] + c);
-      float xf[8];
-      unpack8(xv[c], xf);
+      // Two-element dot products of the bf16 pairs as loaded (v_dot2c_f32_bf16: exact products,
+      // float32 sums), as the fused one-row kernels take theirs.
+      const uint4 xp = xv[c];
 #pragma unroll
       for (int r = 0; r < RPW; ++r) {
-        float wf[8];
-        unpack8(wv[r], wf);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[r] = fmaf(wf[i], xf[i], acc[r]);
+        acc[r] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wv[r].x), __builtin_bit_cast(bf16x2_t, xp.x), acc[r], false);
+        acc[r] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wv[r].y), __builtin_bit_cast(bf16x2_t, xp.y), acc[r], false);
+        acc[r] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wv[r].z), __builtin_bit_cast(bf16x2_t, xp.z), acc[r], false);
+        acc[r] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wv[r].w), __builtin_bit_cast(bf16x2_t, xp.w), acc[r], false);
       }
     }
   }
